@@ -1,0 +1,102 @@
+/*
+ * rk_npu_hip.h -- MI355X-only additions to the rk_npu_* C API.
+ *
+ * None of these entry points has a counterpart in the reference.  They exist
+ * because the reference API hands over host buffers and blocks, which on a
+ * discrete GPU puts a PCIe copy on both sides of every call.  Callers that
+ * keep activations in HBM between layers (and the benchmark, which must time
+ * the device path with inputs already resident) use the *_device variants:
+ * same validation, same kernels, device pointers in and out, work enqueued on
+ * the context's stream without waiting for it.
+ *
+ * Rules for the *_device calls:
+ *   - pointers are device pointers valid on the context's device;
+ *   - the call returns after enqueueing; rk_npu_hip_sync() (or any blocking
+ *     reference call on the same context) waits for completion;
+ *   - input rejection that needs a look at the data (NaN / Inf activations,
+ *     non-finite SwiGLU middle) is reported by rk_npu_hip_sync() as
+ *     RK_NPU_ERR_PARAM for the work enqueued since the previous sync;
+ *   - the workspace stays BUSY only while the call enqueues, so the caller
+ *     must not reuse a workspace from another thread before syncing.
+ */
+#ifndef RK_NPU_HIP_H
+#define RK_NPU_HIP_H
+
+#include "rk_npu_moe_w8.h"
+#include "rk_npu_quant_matmul.h"
+#include "rk_npu_w4a8.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The context's hipStream_t (as void*), its device ordinal, and hardware facts
+ * used to print rooflines. */
+void* rk_npu_hip_stream(rk_npu_ctx* ctx);
+int rk_npu_hip_device(const rk_npu_ctx* ctx);
+int rk_npu_hip_device_info(const rk_npu_ctx* ctx, char* arch, int arch_len, int* cu_count,
+                           int* clock_khz);
+/* Wait for the context's stream; returns RK_NPU_ERR_PARAM if a kernel since the
+ * last sync flagged rejected input, RK_NPU_ERR_SUBMIT on a runtime failure. */
+int rk_npu_hip_sync(rk_npu_ctx* ctx);
+
+/* Plain device memory helpers so that non-HIP callers can stage buffers. */
+void* rk_npu_hip_malloc(rk_npu_ctx* ctx, size_t bytes);
+void rk_npu_hip_free(rk_npu_ctx* ctx, void* ptr);
+int rk_npu_hip_upload(rk_npu_ctx* ctx, void* dst_device, const void* src_host, size_t bytes);
+int rk_npu_hip_download(rk_npu_ctx* ctx, void* dst_host, const void* src_device, size_t bytes);
+
+/* Stream timing (HIP events on the context's stream). */
+typedef struct rk_npu_hip_event rk_npu_hip_event;
+rk_npu_hip_event* rk_npu_hip_event_create(void);
+void rk_npu_hip_event_free(rk_npu_hip_event* event);
+int rk_npu_hip_event_record(rk_npu_ctx* ctx, rk_npu_hip_event* event);
+/* Waits for `stop`; microseconds between the two records. */
+int rk_npu_hip_event_elapsed_us(rk_npu_hip_event* start, rk_npu_hip_event* stop, double* us);
+
+/* Device-resident variants of the blocking run calls. */
+int rk_npu_i8i8i32_run_device(rk_npu_matmul_workspace* workspace,
+                              const rk_npu_i8i8i32_weights* weights, const int8_t* A_device,
+                              int32_t* C_device);
+int rk_npu_f16i8f16_run_dynamic_device(rk_npu_matmul_workspace* workspace,
+                                       const rk_npu_f16i8f16_weights* weights,
+                                       const uint16_t* A_device, uint16_t* C_device);
+int rk_npu_f32i8f32_run_dynamic_device(rk_npu_matmul_workspace* workspace,
+                                       const rk_npu_f32i8f32_weights* weights,
+                                       const float* A_device, float* C_device);
+int rk_npu_w4a8_run_f16_device(rk_npu_w4a8_workspace* workspace,
+                               const rk_npu_w4a8_weights* weights, const uint16_t* A_device,
+                               uint16_t* C_device);
+int rk_npu_w4a8_run_f32_device(rk_npu_w4a8_workspace* workspace,
+                               const rk_npu_w4a8_weights* weights, const float* A_device,
+                               float* C_device);
+int rk_npu_w4a8_run_ffn_f32_device(rk_npu_w4a8_workspace* gate_up,
+                                   const rk_npu_w4a8_weights* gate_up_weights,
+                                   rk_npu_w4a8_workspace* down,
+                                   const rk_npu_w4a8_weights* down_weights, const float* A_device,
+                                   float* middle_device, float* C_device);
+int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* workspace,
+                                 const rk_npu_moe_w8_weights* weights, int rows,
+                                 const float* input_device, const int32_t* expert_ids_device,
+                                 const float* route_weights_device, float* output_device);
+
+/* Parity probes: the exact intermediates of the most recent run on a
+ * workspace, copied to host.  q is the int8 activation matrix [M, K] in
+ * row-major order, a_scale the per-row scales [M].  Blocking. */
+int rk_npu_matmul_workspace_read_quantized(rk_npu_matmul_workspace* workspace, int8_t* q,
+                                           float* a_scale);
+int rk_npu_w4a8_workspace_read_quantized(rk_npu_w4a8_workspace* workspace, int8_t* q,
+                                         float* a_scale);
+/* int32 accumulators sum_k q[m,k] * B[k,n] of a W4A8 weight for host
+ * activations A (fp32), through the same quantize + GEMM kernels.  Blocking. */
+int rk_npu_w4a8_run_i32(rk_npu_w4a8_workspace* workspace, const rk_npu_w4a8_weights* weights,
+                        const float* A, int32_t* acc);
+
+/* Test hook: make the n-th next device allocation fail (1 = the next one,
+ * 0 = off), to exercise RK_NPU_ERR_NOMEM / NULL-return paths from the host. */
+void rk_npu_hip_fail_alloc_after(int n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RK_NPU_HIP_H */

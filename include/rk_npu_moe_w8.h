@@ -1,0 +1,122 @@
+/*
+ * rk_npu_moe_w8.h -- routed W8A8 SwiGLU experts (optional shared expert) on
+ * MI355X.  The router is external: callers pass top-k expert ids and
+ * coefficients.  Names, struct layouts and defaults follow the reference's
+ * include/rk_npu_moe_w8.h (types :12-65, entry points :69-81 and :148-173).
+ *
+ * Numerical contract (fp32 arithmetic):
+ *   token quantization: s = maxabs ? maxabs/127 : 1 ; q = RNE(clamp(x*(1/s), -127, 127))
+ *   gate/up:  g = ((float)acc_g * s) * gs[n],  u = ((float)acc_u * s) * gs[I+n]
+ *   hidden  = (g / (1 + exp(-g))) * u   with the degree-7 fp32 exp of the
+ *             reference (src/rk_npu_swiglu_fp32_neon.h:13-51)
+ *   s2      = maxabs(hidden) ? maxabs/127 : 1 ; q2 = RNE(clamp(hidden*(1/s2)))
+ *   out[t,n] = sum over slots in order of fma(((float)acc2 * s2) * ds[n], w_slot, out)
+ *             with the shared expert last and coefficient 1.
+ * Routes with coefficient 0 are dropped before any device work; a call whose
+ * every route is dropped zero-fills the output.
+ *
+ * Differences from the RK3588 limits: intermediate may be up to 8192 (the
+ * reference stops at 512 because of a fixed CPU scratch row); npu_cores,
+ * cpu_threads, native_input and timeout_ms are range-checked and unused.
+ * The W4 / mixed / slot-bank / blob import-export entry points of the
+ * reference header (:88-143) are not part of this library.
+ */
+#ifndef RK_NPU_MOE_W8_H
+#define RK_NPU_MOE_W8_H
+
+#define RK_NPU_MOE_QUANT_BLOB_VERSION 3u
+#include "rk_npu_common.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* reference :12-25.  Only RK_NPU_MOE_MIDDLE_CPU (the exact fp32 middle) is
+ * accepted here; the approximate LUT middle is rejected at workspace_create. */
+typedef enum rk_npu_moe_middle {
+    RK_NPU_MOE_MIDDLE_CPU = 0,
+    RK_NPU_MOE_MIDDLE_NPU_LUT = 1
+} rk_npu_moe_middle;
+
+/* reference :27-32 */
+typedef struct rk_npu_moe_w8_weight_config {
+    int hidden;         /* >= 64, multiple of 32        */
+    int intermediate;   /* 32..8192, multiple of 32     */
+    int routed_experts; /* 1..4096                      */
+    int shared_expert;  /* 0 or 1; its index is routed_experts */
+} rk_npu_moe_w8_weight_config;
+
+/* reference :34-44 */
+typedef struct rk_npu_moe_w8_config {
+    uint32_t struct_size;
+    rk_npu_moe_w8_weight_config weights;
+    int max_rows;     /* 1..256 */
+    int top_k;        /* 1..min(routed_experts, 8) */
+    int npu_cores;    /* 1..3 */
+    int cpu_threads;  /* 1..4 */
+    int native_input; /* 0 or 1 */
+    rk_npu_moe_middle middle;
+    uint32_t timeout_ms; /* 1..60000 */
+} rk_npu_moe_w8_config;
+
+/* One expert's host tensors; copied by weights_create (reference :46-53). */
+typedef struct rk_npu_moe_w8_expert {
+    const int8_t* gate_up;       /* [hidden, 2*intermediate], gate columns then up columns */
+    const float* gate_up_scales; /* [2*intermediate], finite > 0 */
+    const int8_t* down;          /* [intermediate, hidden] */
+    const float* down_scales;    /* [hidden], finite > 0 */
+} rk_npu_moe_w8_expert;
+
+/* reference :55-62.  input_us = token quantize + scatter, schedule_us =
+ * device-side sort by expert, gate_us / down_us = grouped GEMMs,
+ * middle_cpu_us = the re-quantize kernel, combine_us = weighted sum,
+ * sync_us = host<->device copies. */
+typedef struct rk_npu_moe_w8_timings {
+    double input_us, schedule_us, build_us, sync_us, gather_us;
+    double gate_us, middle_npu_us, middle_cpu_us, down_us, combine_us;
+    double lut_load_us;
+    double total_us;
+    uint32_t gather_tasks, middle_tasks, gemm_tasks;
+} rk_npu_moe_w8_timings;
+
+typedef struct rk_npu_moe_w8_weights rk_npu_moe_w8_weights;
+typedef struct rk_npu_moe_w8_workspace rk_npu_moe_w8_workspace;
+
+/* {sizeof, {hidden, intermediate, routed_experts, shared_expert}, max_rows,
+ *  top_k, npu_cores 3, cpu_threads 4, native_input 0, MIDDLE_CPU, 1000 ms}
+ * (reference :69-71) */
+void rk_npu_moe_w8_config_init(rk_npu_moe_w8_config* config, int hidden, int intermediate,
+                               int routed_experts, int shared_expert, int top_k, int max_rows);
+
+/* experts[routed_experts + shared_expert]; NULL on invalid configuration,
+ * scale or allocation failure (reference :76-78). */
+rk_npu_moe_w8_weights* rk_npu_moe_w8_weights_create(rk_npu_iommu_domain* domain,
+                                                    const rk_npu_moe_w8_weight_config* config,
+                                                    const rk_npu_moe_w8_expert* experts);
+void rk_npu_moe_w8_weights_free(rk_npu_moe_w8_weights* weights);
+rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* domain,
+                                                        const rk_npu_moe_w8_config* config);
+void rk_npu_moe_w8_workspace_free(rk_npu_moe_w8_workspace* workspace);
+
+/* Device bytes held (reference :148-149). */
+uint64_t rk_npu_moe_w8_weights_device_bytes(const rk_npu_moe_w8_weights* weights);
+uint64_t rk_npu_moe_w8_workspace_device_bytes(const rk_npu_moe_w8_workspace* workspace);
+
+/* expert_ids / route_weights are [rows, top_k]; ids in [0, routed_experts),
+ * coefficients finite and >= 0; output is fp32 [rows, hidden]; input, ids and
+ * coefficients must not overlap output; 1 <= rows <= max_rows.
+ * (reference :166-173) */
+int rk_npu_moe_w8_run_quantized(rk_npu_moe_w8_workspace* workspace,
+                                const rk_npu_moe_w8_weights* weights, int rows,
+                                const int8_t* input, const float* row_scales,
+                                const int32_t* expert_ids, const float* route_weights,
+                                float* output, rk_npu_moe_w8_timings* timings);
+int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
+                          const rk_npu_moe_w8_weights* weights, int rows, const float* input,
+                          const int32_t* expert_ids, const float* route_weights,
+                          float* output, rk_npu_moe_w8_timings* timings);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RK_NPU_MOE_W8_H */

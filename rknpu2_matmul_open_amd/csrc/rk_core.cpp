@@ -1,0 +1,286 @@
+// Context, domain tags, error strings, device buffers and the generic part of
+// the MI355X extension API.  Replaces the device core of the reference
+// (src/rk_npu_core.cpp:98-183: open / close / strerror / domain handles); the
+// GEM / dmabuf half of that file has no equivalent because HBM allocations are
+// private to this library.
+#include <cerrno>
+#include <cstdlib>
+#include <new>
+
+#include "rk_host.h"
+#include "rk_npu_hip.h"
+
+namespace {
+std::atomic<uint64_t> g_next_ctx_id{1};
+}
+
+namespace rkhost {
+
+int DeviceBuffer::alloc(const Owner& owner, size_t bytes, bool zero) {
+    release();
+    if (!owner.ctx) return RK_NPU_ERR_PARAM;
+    void* p = nullptr;
+    // round to whole 32-bit words so the fill kernel can clear it
+    const size_t rounded = (bytes + 15) / 16 * 16;
+    int rc = rkh_malloc(owner.ctx->device, &p, rounded);
+    if (rc) return map_error(rc);
+    if (zero) {
+        rc = rkh_fill32(owner.ctx->stream, p, 0u, rounded / 4);
+        if (rc) {
+            rkh_free(owner.ctx->device, p);
+            return map_error(rc);
+        }
+    }
+    ptr_ = p;
+    bytes_ = rounded;
+    owner_ = owner;
+    auto& mem = owner.ctx->memory[owner.domain_id];
+    const uint64_t live = mem.live_bytes.fetch_add(rounded) + rounded;
+    uint64_t peak = mem.peak_bytes.load();
+    while (live > peak && !mem.peak_bytes.compare_exchange_weak(peak, live)) {
+    }
+    mem.creates.fetch_add(1);
+    return RK_NPU_OK;
+}
+
+void DeviceBuffer::release() {
+    if (!ptr_) return;
+    // Work that may still read the buffer is on the context's stream.
+    rkh_sync(owner_.ctx->stream);
+    rkh_free(owner_.ctx->device, ptr_);
+    auto& mem = owner_.ctx->memory[owner_.domain_id];
+    mem.live_bytes.fetch_sub(bytes_);
+    mem.destroys.fetch_add(1);
+    ptr_ = nullptr;
+    bytes_ = 0;
+}
+
+StageTimer::StageTimer(void* stream, bool enabled) : stream_(stream), enabled_(enabled) {}
+StageTimer::~StageTimer() {
+    for (int i = 0; i < count_; ++i) rkh_event_destroy(events_[i]);
+}
+void StageTimer::mark() {
+    if (!enabled_ || count_ >= 12) return;
+    void* e = nullptr;
+    if (rkh_event_create(&e)) return;
+    rkh_event_record(e, stream_);
+    events_[count_++] = e;
+}
+double StageTimer::span_us(int from, int to) {
+    if (!enabled_ || from < 0 || to >= count_ || from >= to) return 0.0;
+    double us = 0.0;
+    if (rkh_event_elapsed_us(events_[from], events_[to], &us)) return 0.0;
+    return us;
+}
+
+BadFlag::~BadFlag() { rkh_host_free(host_); }
+int BadFlag::init(const Owner& owner) {
+    int rc = dev_.alloc(owner, sizeof(int), true);
+    if (rc) return rc;
+    void* h = nullptr;
+    rc = rkh_host_alloc(&h, sizeof(int));
+    if (rc) return map_error(rc);
+    host_ = static_cast<int*>(h);
+    *host_ = 0;
+    return RK_NPU_OK;
+}
+int BadFlag::enqueue_readback(void* stream) {
+    return map_error(rkh_d2h(stream, host_, dev_.as<>(), sizeof(int)));
+}
+bool BadFlag::consume(void* stream) {
+    if (!*host_) return false;
+    *host_ = 0;
+    rkh_fill32(stream, dev_.as<>(), 0u, 1);
+    return true;
+}
+bool consume_device_flag(rk_npu_ctx* ctx, int* flag) {
+    int v = 0;
+    if (rkh_d2h(ctx->stream, &v, flag, sizeof(int)) || rkh_sync(ctx->stream)) return false;
+    if (!v) return false;
+    rkh_fill32(ctx->stream, flag, 0u, 1);
+    return true;
+}
+void note_pending_flag(rk_npu_ctx* ctx, int* flag) {
+    std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+    for (int* f : ctx->pending_flags)
+        if (f == flag) return;
+    ctx->pending_flags.push_back(flag);
+}
+
+int upload(const Owner& owner, DeviceBuffer& dst, const void* src, size_t bytes) {
+    int rc = dst.alloc(owner, bytes, false);
+    if (rc) return rc;
+    rc = rkh_h2d(owner.ctx->stream, dst.as<>(), src, bytes);
+    return map_error(rc);
+}
+
+} // namespace rkhost
+
+extern "C" {
+
+rk_npu_ctx* rk_npu_open(const char* dev) {
+    int device = 0;
+    if (dev) {
+        if (std::strncmp(dev, "hip:", 4) != 0 || !dev[4]) {
+            errno = ENODEV;
+            return nullptr;
+        }
+        char* end = nullptr;
+        const long v = std::strtol(dev + 4, &end, 10);
+        if (*end || v < 0 || v > 1023) {
+            errno = ENODEV;
+            return nullptr;
+        }
+        device = (int)v;
+    }
+    if (device >= rkh_device_count()) {
+        errno = ENODEV;
+        return nullptr;
+    }
+    rk_npu_ctx* ctx = new (std::nothrow) rk_npu_ctx();
+    if (!ctx) {
+        errno = ENOMEM;
+        return nullptr;
+    }
+    ctx->device = device;
+    if (rkh_open(device, &ctx->stream, ctx->arch, (int)sizeof(ctx->arch), &ctx->cu_count,
+                 &ctx->clock_khz)) {
+        delete ctx;
+        errno = ENODEV;
+        return nullptr;
+    }
+    ctx->id = g_next_ctx_id.fetch_add(1);
+    return ctx;
+}
+
+void rk_npu_close(rk_npu_ctx* ctx) {
+    if (!ctx) return;
+    rkh_close(ctx->device, ctx->stream);
+    delete ctx;
+}
+
+const char* rk_npu_strerror(int code) {
+    switch (code) {
+    case RK_NPU_OK: return "ok";
+    case RK_NPU_ERR_OPEN: return "could not open device";
+    case RK_NPU_ERR_IOCTL: return "device runtime call failed";
+    case RK_NPU_ERR_PARAM: return "bad argument";
+    case RK_NPU_ERR_NOMEM: return "allocation failed or buffer too small";
+    case RK_NPU_ERR_SUBMIT: return "device job failed/timed out";
+    case RK_NPU_ERR_BUSY: return "workspace is already running";
+    case RK_NPU_ERR_DOMAIN: return "domain mismatch or unavailable";
+    case RK_NPU_ERR_IO: return "file I/O failed";
+    case RK_NPU_ERR_CACHE_MISS: return "tuning cache miss";
+    default: return "unknown error";
+    }
+}
+
+rk_npu_iommu_domain* rk_npu_iommu_domain_create(rk_npu_ctx* ctx, uint32_t domain_id) {
+    if (!ctx || domain_id >= RK_NPU_IOMMU_DOMAIN_COUNT) return nullptr;
+    rk_npu_iommu_domain* d = new (std::nothrow) rk_npu_iommu_domain();
+    if (!d) return nullptr;
+    d->ctx = ctx;
+    d->id = domain_id;
+    return d;
+}
+
+void rk_npu_iommu_domain_free(rk_npu_iommu_domain* domain) { delete domain; }
+
+uint32_t rk_npu_iommu_domain_id(const rk_npu_iommu_domain* domain) {
+    return domain ? domain->id : UINT32_MAX;
+}
+
+int rk_npu_iommu_domain_memory_stats(const rk_npu_iommu_domain* domain,
+                                     rk_npu_domain_memory_stats* stats) {
+    if (!domain || !domain->ctx || !stats) return RK_NPU_ERR_PARAM;
+    const auto& m = domain->ctx->memory[domain->id];
+    stats->live_bytes = m.live_bytes.load();
+    stats->peak_bytes = m.peak_bytes.load();
+    stats->creates = m.creates.load();
+    stats->destroys = m.destroys.load();
+    return RK_NPU_OK;
+}
+
+/* ---- MI355X extension: generic part ---- */
+
+void* rk_npu_hip_stream(rk_npu_ctx* ctx) { return ctx ? ctx->stream : nullptr; }
+int rk_npu_hip_device(const rk_npu_ctx* ctx) { return ctx ? ctx->device : -1; }
+
+int rk_npu_hip_device_info(const rk_npu_ctx* ctx, char* arch, int arch_len, int* cu_count,
+                           int* clock_khz) {
+    if (!ctx) return RK_NPU_ERR_PARAM;
+    if (arch && arch_len > 0) {
+        std::strncpy(arch, ctx->arch, (size_t)arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    if (cu_count) *cu_count = ctx->cu_count;
+    if (clock_khz) *clock_khz = ctx->clock_khz;
+    return RK_NPU_OK;
+}
+
+int rk_npu_hip_sync(rk_npu_ctx* ctx) {
+    if (!ctx) return RK_NPU_ERR_PARAM;
+    if (rkh_sync(ctx->stream)) return RK_NPU_ERR_SUBMIT;
+    std::vector<int*> flags;
+    {
+        std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+        flags.swap(ctx->pending_flags);
+    }
+    bool rejected = false;
+    for (int* f : flags) rejected |= rkhost::consume_device_flag(ctx, f);
+    return rejected ? RK_NPU_ERR_PARAM : RK_NPU_OK;
+}
+
+void* rk_npu_hip_malloc(rk_npu_ctx* ctx, size_t bytes) {
+    if (!ctx) return nullptr;
+    void* p = nullptr;
+    if (rkh_malloc(ctx->device, &p, bytes)) return nullptr;
+    return p;
+}
+void rk_npu_hip_free(rk_npu_ctx* ctx, void* ptr) {
+    if (!ctx || !ptr) return;
+    rkh_sync(ctx->stream);
+    rkh_free(ctx->device, ptr);
+}
+int rk_npu_hip_upload(rk_npu_ctx* ctx, void* dst_device, const void* src_host, size_t bytes) {
+    if (!ctx || !dst_device || !src_host) return RK_NPU_ERR_PARAM;
+    int rc = rkh_h2d(ctx->stream, dst_device, src_host, bytes);
+    if (!rc) rc = rkh_sync(ctx->stream);
+    return rkhost::map_error(rc);
+}
+int rk_npu_hip_download(rk_npu_ctx* ctx, void* dst_host, const void* src_device, size_t bytes) {
+    if (!ctx || !dst_host || !src_device) return RK_NPU_ERR_PARAM;
+    int rc = rkh_d2h(ctx->stream, dst_host, src_device, bytes);
+    if (!rc) rc = rkh_sync(ctx->stream);
+    return rkhost::map_error(rc);
+}
+
+struct rk_npu_hip_event {
+    void* handle = nullptr;
+};
+rk_npu_hip_event* rk_npu_hip_event_create(void) {
+    auto* e = new (std::nothrow) rk_npu_hip_event();
+    if (!e) return nullptr;
+    if (rkh_event_create(&e->handle)) {
+        delete e;
+        return nullptr;
+    }
+    return e;
+}
+void rk_npu_hip_event_free(rk_npu_hip_event* event) {
+    if (!event) return;
+    rkh_event_destroy(event->handle);
+    delete event;
+}
+int rk_npu_hip_event_record(rk_npu_ctx* ctx, rk_npu_hip_event* event) {
+    if (!ctx || !event) return RK_NPU_ERR_PARAM;
+    return rkhost::map_error(rkh_event_record(event->handle, ctx->stream));
+}
+int rk_npu_hip_event_elapsed_us(rk_npu_hip_event* start, rk_npu_hip_event* stop, double* us) {
+    if (!start || !stop || !us) return RK_NPU_ERR_PARAM;
+    return rkhost::map_error(rkh_event_elapsed_us(start->handle, stop->handle, us));
+}
+
+void rk_npu_hip_fail_alloc_after(int n) { rkh_fail_malloc_after(n); }
+
+} // extern "C"

@@ -1,0 +1,1206 @@
+// HIP kernels of the quantized-linear path for gfx950 (MI355X), and the C-ABI
+// launchers declared in rk_hip_shim.h.  Data layouts are described there.
+//
+// Kernel inventory (what bounds each one):
+//   pack_w8 / pack_w4     weight re-tiling at upload            (one-time)
+//   quant_rows            per-token absmax + int8 quantize      (HBM, tiny)
+//   gemv                  M <= 8 decode path, dot4, no MFMA     (HBM)
+//   gemm                  int8 MFMA 32x32x32, LDS double buffer (MFMA / HBM)
+//   splitk_epilogue       dequant / SwiGLU of split-K sums      (HBM, tiny)
+//   moe_route / combine   sort by expert, weighted sum          (latency)
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <float.h>
+
+#include "rk_hip_shim.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace {
+
+#define RKH_CHECK(expr)                                                        \
+    do {                                                                       \
+        hipError_t e_ = (expr);                                                \
+        if (e_ != hipSuccess) return e_ == hipErrorOutOfMemory ? RKH_ERR_NOMEM \
+                                                               : RKH_ERR_RUNTIME; \
+    } while (0)
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// Logical first column of physical 32-column block p.
+__device__ __forceinline__ int block_first_col(int p, int interleave_F) {
+    if (!interleave_F) return p * 32;
+    return (p & 1) ? interleave_F + (p >> 1) * 32 : (p >> 1) * 32;
+}
+
+// ------------------------------------------------------------------ fill
+__global__ void fill32_kernel(uint32_t* dst, uint32_t value, size_t words) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < words; i += stride) dst[i] = value;
+}
+
+// ------------------------------------------------------------ weight pack
+// One thread produces one lane's 16 bytes of one tile.
+__global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__ src, int K, int N,
+                                                      int KB, int interleave_F,
+                                                      uint8_t* __restrict__ dst, size_t total_chunks) {
+    const size_t chunk = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (chunk >= total_chunks) return;
+    const int lane = (int)(chunk & 63);
+    const size_t tile = chunk >> 6;
+    const int kb = (int)(tile % KB);
+    const int p = (int)(tile / KB);
+    const int n = block_first_col(p, interleave_F) + (lane & 31);
+    const int k0 = kb * 32 + (lane >> 5) * 16;
+    uint32_t w[4] = {0, 0, 0, 0};
+    const bool col_ok = interleave_F ? (p < N / 32) : (n < N);
+    if (col_ok) {
+        for (int j = 0; j < 16; ++j) {
+            const int k = k0 + j;
+            const uint32_t v = k < K ? (uint8_t)src[(size_t)k * N + n] : 0u;
+            w[j >> 2] |= v << ((j & 3) * 8);
+        }
+    }
+    reinterpret_cast<uint4*>(dst)[chunk] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ __launch_bounds__(256) void pack_w4_kernel(const int8_t* __restrict__ src, int K, int N,
+                                                      int KB2, int interleave_F,
+                                                      uint8_t* __restrict__ dst, size_t total_chunks,
+                                                      int* bad_flag) {
+    const size_t chunk = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (chunk >= total_chunks) return;
+    const int lane = (int)(chunk & 63);
+    const size_t tile = chunk >> 6;
+    const int kb2 = (int)(tile % KB2);
+    const int p = (int)(tile / KB2);
+    const int n = block_first_col(p, interleave_F) + (lane & 31);
+    const bool col_ok = interleave_F ? (p < N / 32) : (n < N);
+    uint32_t w[4] = {0, 0, 0, 0};
+    bool bad = false;
+    if (col_ok) {
+        for (int t = 0; t < 2; ++t) {            // the two 32-k halves of the super-tile
+            const int k0 = kb2 * 64 + t * 32 + (lane >> 5) * 16;
+            for (int j = 0; j < 16; ++j) {
+                const int k = k0 + j;
+                int code = 0;
+                if (k < K) {
+                    code = src[(size_t)k * N + n];
+                    if (code < -8 || code > 7) bad = true;
+                }
+                // word = t*2 + j/8 ; within the word: byte (j%8)%4, high nibble when (j%8) >= 4
+                const int k8 = j & 7;
+                const int shift = (k8 & 3) * 8 + (k8 >> 2) * 4;
+                w[t * 2 + (j >> 3)] |= (uint32_t)(code & 15) << shift;
+            }
+        }
+    }
+    if (bad && bad_flag) atomicOr(bad_flag, 1);
+    reinterpret_cast<uint4*>(dst)[chunk] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ------------------------------------------------------------- quant_rows
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+    return __half2float(__ushort_as_half(h));
+}
+
+template <typename T> struct RowLoader;
+template <> struct RowLoader<uint16_t> {
+    static __device__ __forceinline__ void load16(const uint16_t* row, int k0, int K, bool vec,
+                                                  float* out) {
+        if (vec && k0 + 16 <= K) {
+            const uint4 a = *reinterpret_cast<const uint4*>(row + k0);
+            const uint4 b = *reinterpret_cast<const uint4*>(row + k0 + 8);
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                out[2 * j] = half_bits_to_float((uint16_t)(w[j] & 0xffffu));
+                out[2 * j + 1] = half_bits_to_float((uint16_t)(w[j] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) out[j] = k0 + j < K ? half_bits_to_float(row[k0 + j]) : 0.0f;
+        }
+    }
+};
+template <> struct RowLoader<float> {
+    static __device__ __forceinline__ void load16(const float* row, int k0, int K, bool vec,
+                                                  float* out) {
+        if (vec && k0 + 16 <= K) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 v = *reinterpret_cast<const float4*>(row + k0 + 4 * j);
+                out[4 * j] = v.x; out[4 * j + 1] = v.y; out[4 * j + 2] = v.z; out[4 * j + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) out[j] = k0 + j < K ? row[k0 + j] : 0.0f;
+        }
+    }
+};
+template <> struct RowLoader<int8_t> {
+    static __device__ __forceinline__ void load16(const int8_t* row, int k0, int K, bool vec,
+                                                  float* out) {
+        (void)vec;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) out[j] = k0 + j < K ? (float)row[k0 + j] : 0.0f;
+    }
+};
+
+__device__ __forceinline__ bool not_finite(float x) {
+    return (__float_as_uint(x) & 0x7f800000u) == 0x7f800000u;
+}
+
+// Byte offset of the 16-byte chunk (row, chunk c = k/16) in a tiled int8 matrix.
+__device__ __forceinline__ size_t tiled_chunk_offset(int row, int c, int KB) {
+    const int kb = c >> 1, half = c & 1;
+    return ((size_t)(row >> 5) * KB + kb) * 1024 + (size_t)((row & 31) + 32 * half) * 16;
+}
+
+template <bool EVEN>
+__device__ __forceinline__ uint4 quantize16(const float* v, float inv) {
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        float q = v[j] * inv;
+        if (EVEN) {
+            q = fminf(q, 127.0f);
+            q = fmaxf(q, -127.0f);
+            q = rintf(q);
+        } else {
+            q = roundf(q);
+            q = q < 127.0f ? q : 127.0f;   // NaN -> 127, as the reference's std::min/std::max chain
+            q = q > -127.0f ? q : -127.0f;
+        }
+        const int code = (int)q;
+        w[j >> 2] |= (uint32_t)(code & 255) << ((j & 3) * 8);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+constexpr int QR_CACHE = 4; // 16-element chunks kept in registers per thread
+
+template <typename T>
+__global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
+    __shared__ float wave_max[4];
+    __shared__ int wave_bad[4];
+    const int m = blockIdx.x, t = threadIdx.x;
+    if (a.active_blocks && m >= a.active_blocks[0] * 32) return;
+    const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
+    const int nchunks = (K + 15) >> 4;
+    const T* row = static_cast<const T*>(a.src) + (size_t)m * K;
+    const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    const bool cached = nchunks <= 256 * QR_CACHE;
+    const int mode = a.mode;
+    const bool need_max = mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
+    const bool check = mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
+
+    float v[QR_CACHE][16];
+    float mx = 0.0f;
+    bool bad = false;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < QR_CACHE; ++i) {
+            const int c = t + i * 256;
+            if (c < nchunks) {
+                RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
+                if (need_max) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        mx = fmaxf(mx, fabsf(v[i][j]));
+                        bad |= not_finite(v[i][j]);
+                    }
+                }
+            }
+        }
+    } else if (need_max) {
+        for (int c = t; c < nchunks; c += 256) {
+            float tmp[16];
+            RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                mx = fmaxf(mx, fabsf(tmp[j]));
+                bad |= not_finite(tmp[j]);
+            }
+        }
+    }
+
+    float scale = 1.0f;
+    if (need_max) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        const unsigned long long bad_mask = __ballot(bad && check);
+        if (lane_id() == 0) {
+            wave_max[wave_id()] = mx;
+            wave_bad[wave_id()] = bad_mask != 0ull;
+        }
+        __syncthreads();
+        mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+        const int any_bad = wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3];
+        if (any_bad && t == 0 && a.bad_flag) atomicOr(a.bad_flag, 1);
+        if (mode == RKH_Q_W4A8) scale = mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN);
+        else scale = mx > 0.0f ? mx / 127.0f : 1.0f;
+    } else if (mode == RKH_Q_W8_STATIC || (mode == RKH_Q_COPY_I8 && a.scale)) {
+        scale = a.scale[m];
+    } else if (mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) {
+        const uint32_t bits = a.row_max_bits[m];
+        const float mxv = __uint_as_float(bits);
+        if (mode == RKH_Q_REUSE_BITS) {
+            if (bits >= 0x7f800000u) {
+                if (t == 0 && a.bad_flag) atomicOr(a.bad_flag, 1);
+                scale = 1.0f;
+            } else {
+                scale = mxv == 0.0f ? 1.0f : fmaxf(mxv / 127.0f, FLT_MIN);
+            }
+        } else {
+            scale = mxv != 0.0f ? mxv / 127.0f : 1.0f;
+        }
+    }
+    const float inv = mode == RKH_Q_COPY_I8 ? 1.0f : 1.0f / scale;
+    const bool even = mode == RKH_Q_MOE || mode == RKH_Q_REUSE_BITS_MOE;
+
+    int ndest = 1;
+    if (a.dest_rows) ndest = a.dest_stride;
+    if (t == 0) {
+        if (!a.dest_rows) {
+            if (a.scale && mode != RKH_Q_W8_STATIC && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
+            if (a.zero_bits) a.zero_bits[m] = 0u;
+        } else {
+            if (a.scale && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
+            for (int j = 0; j < ndest; ++j) {
+                const int d = a.dest_rows[(size_t)m * ndest + j];
+                if (d >= 0) {
+                    a.scale_rows[d] = scale;
+                    if (a.zero_bits) a.zero_bits[d] = 0u;
+                }
+            }
+        }
+    }
+
+    auto emit = [&](int c, const float* vals) {
+        const uint4 packed = even ? quantize16<true>(vals, inv) : quantize16<false>(vals, inv);
+        if (!a.dest_rows) {
+            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
+        } else {
+            for (int j = 0; j < ndest; ++j) {
+                const int d = a.dest_rows[(size_t)m * ndest + j];
+                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+            }
+        }
+    };
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < QR_CACHE; ++i) {
+            const int c = t + i * 256;
+            if (c < nchunks) emit(c, v[i]);
+        }
+    } else {
+        for (int c = t; c < nchunks; c += 256) {
+            float tmp[16];
+            RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+            emit(c, tmp);
+        }
+    }
+}
+
+// ------------------------------------------------------------- epilogues
+// Degree-7 fp32 exponential SiLU, step for step the sequence of the reference
+// (src/rk_npu_swiglu_fp32_neon.h:13-51): every fused step is an explicit fmaf.
+__device__ __forceinline__ float silu_poly(float g) {
+    float x = -g;
+    x = fminf(x, 80.0f);
+    x = fmaxf(x, -80.0f);
+    const float n = floorf(fmaf(x, 1.4426950408889634f, 0.5f));
+    float r = fmaf(-n, 0.693145751953125f, x);
+    r = fmaf(-n, 1.428606765330187e-6f, r);
+    float p = 1.0f / 5040.0f;
+    p = fmaf(p, r, 1.0f / 720.0f);
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    const float power = __uint_as_float((uint32_t)((int)n + 127) << 23);
+    const float d = 1.0f + p * power;
+    return g < -80.0f ? -0.0f : g / d;
+}
+
+__device__ __forceinline__ float dequant(int acc, float as, float ws) {
+    return __fmul_rn(__fmul_rn((float)acc, as), ws);
+}
+
+__device__ __forceinline__ void store_out(void* C, int epi, size_t index, int acc, float as,
+                                          float ws) {
+    if (epi == RKH_EPI_I32) {
+        static_cast<int32_t*>(C)[index] = acc;
+    } else if (epi == RKH_EPI_F16) {
+        static_cast<__half*>(C)[index] = __float2half_rn(dequant(acc, as, ws));
+    } else {
+        static_cast<float*>(C)[index] = dequant(acc, as, ws);
+    }
+}
+
+// ------------------------------------------------------------------ GEMV
+// One workgroup per physical 32-column block; the waves of the group split K
+// (k-tiles interleaved across waves so that neighbouring loads are adjacent in
+// memory); activations sit in LDS; lanes l and l+32 hold the two 16-byte
+// halves of a k-tile for column l%32, so the cross-lane reduction is one xor
+// shuffle, followed by a small LDS reduction across waves.
+constexpr int GEMV_WAVES = 8;
+constexpr int GEMV_UNROLL = 4;
+constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
+
+template <int MR, bool W4>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) {
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
+    __shared__ int red[GEMV_WAVES][MR][32];
+    const int lane = lane_id(), wave = wave_id();
+    const int half = lane >> 5;
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int p = blockIdx.x;
+    // chunk of K staged in LDS at a time (multiple of 64)
+    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
+    int acc[MR], folded[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = folded[m] = 0;
+
+    const uint8_t* wbase = g.W + (W4 ? (size_t)p * (Kp / 64) * 1024 : (size_t)p * KB * 1024);
+
+    for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
+        const int kc = min(kc_max, Kp - kc0);
+        // stage activations: row-major [MR][kc] in LDS from the tiled buffer
+        const int chunks = kc >> 4;
+        if (kc0) __syncthreads();
+        for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+            const int m = idx / chunks, c = idx - m * chunks;
+            const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+        }
+        __syncthreads();
+
+        if (!W4) {
+            const int tiles = kc >> 5, tile0 = kc0 >> 5;
+            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+                v4i w[GEMV_UNROLL];
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                    const int tt = tb + u * GEMV_WAVES;
+                    w[u] = tt < tiles
+                               ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                     wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
+                               : v4i{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                    const int tt = tb + u * GEMV_WAVES;
+                    if (tt < tiles) {
+#pragma unroll
+                        for (int m = 0; m < MR; ++m) {
+                            const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                            acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
+                        }
+                    }
+                }
+            }
+        } else {
+            const int tiles = kc >> 6, tile0 = kc0 >> 6; // super-tiles of 64 k
+            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+                v4i w[GEMV_UNROLL];
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                    const int tt = tb + u * GEMV_WAVES;
+                    w[u] = tt < tiles
+                               ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                     wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
+                               : v4i{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                    const int tt = tb + u * GEMV_WAVES;
+                    if (tt < tiles) {
+                        const int wv[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {       // the two 32-k halves
+                            const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
+                            const int hi0 = wv[2 * s] & 0xF0F0F0F0;
+                            const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
+                            const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
+#pragma unroll
+                            for (int m = 0; m < MR; ++m) {
+                                const v4i av = *reinterpret_cast<const v4i*>(
+                                    a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                                acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
+                                acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
+                                acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
+                                acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
+                            }
+                        }
+                    }
+                }
+            }
+            // int4 operands are carried as 16 * code; fold each K chunk's exact
+            // multiple-of-16 partial back so very long K cannot overflow int32.
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                folded[m] += acc[m] >> 4;
+                acc[m] = 0;
+            }
+        }
+    }
+
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        int v = W4 ? folded[m] : acc[m];
+        v += __shfl_xor(v, 32);
+        if (lane < 32) red[wave][m][lane] = v;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MR * 32; idx += GEMV_WAVES * 64) {
+        const int m = idx >> 5, j = idx & 31;
+        if (m >= g.M) continue;
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
+        const int n = block_first_col(p, g.interleave_F) + j;
+        if (n < g.N)
+            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum, g.a_scale ? g.a_scale[m] : 1.0f,
+                      g.w_scale ? g.w_scale[n] : 1.0f);
+    }
+}
+
+// ------------------------------------------------------------------ GEMM
+// Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn),
+// each wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is 64 deep:
+// the step's A tiles (BM/32 x 2 KiB) and W tiles are copied global -> register
+// -> LDS as whole 1 KiB tiles, so LDS reads are linear 16 bytes per lane
+// (bank-conflict free) and land directly in MFMA operand order.  Two LDS
+// buffers; the loads of step i+1 are issued before the MFMAs of step i.
+struct TileCoord { int mblk, nblk, kpart; };
+
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
+    // contiguous range of logical tiles so neighbours share its L2.
+    const int q = total >> 3, r = total & 7;
+    const int xcd = bid & 7, idx = bid >> 3;
+    return xcd * q + min(xcd, r) + idx;
+}
+
+template <int EPI>
+__device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i& acc, int row0,
+                                              int col_phys_block, int lane, const float* a_scale,
+                                              const float* w_scale, int m_limit) {
+    const int n = block_first_col(col_phys_block, g.interleave_F) + (lane & 31);
+    if (n >= g.N) return;
+    const float ws = EPI == RKH_EPI_I32 ? 1.0f : w_scale[n];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < m_limit) {
+            const float as = EPI == RKH_EPI_I32 ? 1.0f : a_scale[m];
+            store_out(g.C, EPI, (size_t)m * g.ldc + n, acc[r], as, ws);
+        }
+    }
+}
+
+// gate tile / up tile pair -> middle and per-row max bits
+__device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v16i& gate,
+                                                const v16i& up, int row0, int gate_phys_block,
+                                                int lane, const float* a_scale,
+                                                const float* w_scale, int m_limit) {
+    const int F = g.interleave_F;
+    const int n = (gate_phys_block >> 1) * 32 + (lane & 31);
+    const bool col_ok = n < F;
+    const float wg = col_ok ? w_scale[n] : 0.0f;
+    const float wu = col_ok ? w_scale[F + n] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        uint32_t bits = 0;
+        if (m < m_limit && col_ok) {
+            const float as = a_scale[m];
+            const float gf = dequant(gate[r], as, wg);
+            const float uf = dequant(up[r], as, wu);
+            const float y = __fmul_rn(silu_poly(gf), uf);
+            static_cast<float*>(g.C)[(size_t)m * g.ldc + n] = y;
+            bits = __float_as_uint(y) & 0x7fffffffu;
+        }
+        if (g.row_max_bits) {
+            // max over the 32 lanes that share this row
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+            if ((lane & 31) == 0 && m < m_limit && bits) atomicMax(g.row_max_bits + m, bits);
+        }
+    }
+}
+
+template <int WM, int WN, int TM, int TN, bool W4, int EPI, bool GROUPED>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int mblocks,
+                                                            int nblocks, int ksplit,
+                                                            int ksteps_per_part) {
+    constexpr int NW = WM * WN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    constexpr int A_CH = BM / 32 * 2;                 // 1 KiB chunks per K step
+    constexpr int B_CH = W4 ? BN / 32 : BN / 32 * 2;
+    constexpr int CH = A_CH + B_CH;
+    constexpr int LPW = (CH + NW - 1) / NW;           // chunk loads per wave per step
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][CH * 1024];
+
+    const int lane = lane_id(), wave = wave_id();
+    const int wm = wave / WN, wn = wave % WN;
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int ksteps_total = Kp / 64;
+
+    // ---- tile assignment
+    const int total = mblocks * nblocks * ksplit;
+    const int logical = xcd_remap(blockIdx.x, total);
+    const int kpart = logical / (mblocks * nblocks);
+    const int tile = logical - kpart * (mblocks * nblocks);
+    int mblk, nblk;
+    if (GROUPED) {
+        mblk = tile % mblocks;
+        nblk = tile / mblocks;
+        if (mblk * (BM / 32) >= g.num_blocks[0]) return;
+    } else {
+        constexpr int GM = 4; // m-blocks per super-group (L2 reuse of the W columns)
+        const int per_group = GM * nblocks;
+        const int group = tile / per_group;
+        const int first_m = group * GM;
+        const int gm = min(mblocks - first_m, GM);
+        const int in_group = tile - group * per_group;
+        mblk = first_m + in_group % gm;
+        nblk = in_group / gm;
+    }
+    const int kstep0 = kpart * ksteps_per_part;
+    const int ksteps = min(ksteps_per_part, ksteps_total - kstep0);
+    if (ksteps <= 0) return;
+
+    const uint8_t* Wb = g.W;
+    const float* w_scale = g.w_scale;
+    if (GROUPED) {
+        const int e = g.blk_expert[mblk * (BM / 32)];
+        Wb += (size_t)e * g.w_expert_stride;
+        if (w_scale) w_scale += (size_t)e * g.ws_expert_stride;
+    }
+
+    // ---- global -> LDS chunk assignment for this wave
+    const uint8_t* src[LPW];
+    int src_step[LPW]; // bytes to advance per K step
+    int lds_off[LPW];
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const int c = wave + i * NW;
+        if (c < A_CH) {
+            const int rb = mblk * (BM / 32) + (c >> 1);
+            src[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * 2 + (c & 1)) * 1024 + lane * 16;
+            src_step[i] = 2048;
+        } else if (c < CH) {
+            const int cb = c - A_CH;
+            if (W4) {
+                const int pb = nblk * (BN / 32) + cb;
+                src[i] = Wb + ((size_t)pb * (Kp / 64) + kstep0) * 1024 + lane * 16;
+                src_step[i] = 1024;
+            } else {
+                const int pb = nblk * (BN / 32) + (cb >> 1);
+                src[i] = Wb + ((size_t)pb * KB + (size_t)kstep0 * 2 + (cb & 1)) * 1024 + lane * 16;
+                src_step[i] = 2048;
+            }
+        } else {
+            src[i] = nullptr;
+            src_step[i] = 0;
+        }
+        lds_off[i] = c * 1024 + lane * 16;
+    }
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    v4i stage[LPW];
+    auto load_stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) {
+            if (wave + i * NW < CH) {
+                stage[i] = *reinterpret_cast<const v4i*>(src[i]);
+                src[i] += src_step[i];
+            }
+        }
+    };
+    auto store_stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LPW; ++i)
+            if (wave + i * NW < CH) *reinterpret_cast<v4i*>(&lds[buf][lds_off[i]]) = stage[i];
+    };
+
+    load_stage();
+    store_stage(0);
+    __syncthreads();
+
+    for (int s = 0; s < ksteps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < ksteps) load_stage();
+        const uint8_t* la = &lds[buf][0];
+        const uint8_t* lb = &lds[buf][A_CH * 1024];
+        if (!W4) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                v4i af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    af[i] = *reinterpret_cast<const v4i*>(la + ((wm * TM + i) * 2 + kt) * 1024 + lane * 16);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    bf[j] = *reinterpret_cast<const v4i*>(lb + ((wn * TN + j) * 2 + kt) * 1024 + lane * 16);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        } else {
+            v4i praw[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                praw[j] = *reinterpret_cast<const v4i*>(lb + (wn * TN + j) * 1024 + lane * 16);
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                v4i af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    af[i] = *reinterpret_cast<const v4i*>(la + ((wm * TM + i) * 2 + kt) * 1024 + lane * 16);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const int w0 = kt ? praw[j].z : praw[j].x;
+                    const int w1 = kt ? praw[j].w : praw[j].y;
+                    bf[j].x = (w0 << 4) & 0xF0F0F0F0;
+                    bf[j].y = w0 & 0xF0F0F0F0;
+                    bf[j].z = (w1 << 4) & 0xF0F0F0F0;
+                    bf[j].w = w1 & 0xF0F0F0F0;
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        if (s + 1 < ksteps) store_stage(buf ^ 1);
+        __syncthreads();
+    }
+
+    if (W4) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] >>= 4;
+    }
+
+    // ---- epilogue
+    const int m_limit = GROUPED ? g.num_blocks[0] * 32 : g.M;
+    if (ksplit > 1) {
+        // exact integer partial sums: accumulate into the zeroed scratch matrix
+        // (physical column order); a second kernel applies the epilogue.
+        const int ld = nblocks * BN;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int row0 = mblk * BM + (wm * TM + i) * 32;
+                const int col = (nblk * (BN / 32) + wn * TN + j) * 32 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    if (m < m_limit && acc[i][j][r])
+                        atomicAdd(g.splitk_acc + (size_t)m * ld + col, acc[i][j][r]);
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int row0 = mblk * BM + (wm * TM + i) * 32;
+        if constexpr (EPI == RKH_EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < TN; j += 2)
+                epilogue_swiglu(g, acc[i][j], acc[i][j + 1], row0, nblk * (BN / 32) + wn * TN + j,
+                                lane, g.a_scale, w_scale, m_limit);
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                epilogue_tile<EPI>(g, acc[i][j], row0, nblk * (BN / 32) + wn * TN + j, lane,
+                                   g.a_scale, w_scale, m_limit);
+        }
+    }
+}
+
+// Epilogue over the split-K scratch matrix; re-zeroes what it consumed so the
+// scratch is clean for the next call.
+__global__ __launch_bounds__(256) void splitk_epilogue_kernel(rkh_gemm_args g, int ld) {
+    const int m = blockIdx.y;
+    const int F = g.interleave_F;
+    if (g.epilogue == RKH_EPI_SWIGLU) {
+        const int n = blockIdx.x * 256 + threadIdx.x; // middle column
+        uint32_t bits = 0;
+        if (n < F) {
+            const int pg = (n >> 5) * 2;
+            const size_t ig = (size_t)m * ld + pg * 32 + (n & 31), iu = ig + 32;
+            const int ag = g.splitk_acc[ig], au = g.splitk_acc[iu];
+            g.splitk_acc[ig] = 0;
+            g.splitk_acc[iu] = 0;
+            const float as = g.a_scale[m];
+            const float y = __fmul_rn(silu_poly(dequant(ag, as, g.w_scale[n])),
+                                      dequant(au, as, g.w_scale[F + n]));
+            static_cast<float*>(g.C)[(size_t)m * g.ldc + n] = y;
+            bits = __float_as_uint(y) & 0x7fffffffu;
+        }
+        if (g.row_max_bits) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+            if (lane_id() == 0 && bits) atomicMax(g.row_max_bits + m, bits);
+        }
+    } else {
+        const int pc = blockIdx.x * 256 + threadIdx.x; // physical column
+        const int n = block_first_col(pc >> 5, F) + (pc & 31);
+        if (pc < ld && n < g.N && (!F || (pc >> 5) < g.N / 32)) {
+            const size_t i = (size_t)m * ld + pc;
+            const int a = g.splitk_acc[i];
+            g.splitk_acc[i] = 0;
+            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, a, g.a_scale ? g.a_scale[m] : 1.0f,
+                      g.w_scale ? g.w_scale[n] : 1.0f);
+        }
+    }
+}
+
+// ------------------------------------------------------------- MoE route
+// Single workgroup.  Assignments (row-major over [rows, top_k]) with a non-zero
+// coefficient are bucketed by expert id, stably, each bucket padded to a
+// multiple of 32 rows; the shared expert (id == experts) gets every row.
+constexpr int ROUTE_MAX_EXPERTS = 2048;
+constexpr int ROUTE_WAVES = 4;
+
+__global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_route_args a) {
+    __shared__ int bins[ROUTE_WAVES][ROUTE_MAX_EXPERTS];
+    __shared__ int start[ROUTE_MAX_EXPERTS + 1];
+    __shared__ int partial[ROUTE_WAVES * 64];
+    const int t = threadIdx.x, lane = lane_id(), wave = wave_id();
+    const int E = a.experts, Etot = E + a.shared;
+    const int slots = a.top_k + a.shared;
+    const int n = a.rows * a.top_k;
+    for (int i = t; i < ROUTE_WAVES * Etot; i += ROUTE_WAVES * 64) bins[i / Etot][i % Etot] = 0;
+    __syncthreads();
+
+    const int chunks_total = (n + 63) / 64;
+    const int chunks_per_wave = (chunks_total + ROUTE_WAVES - 1) / ROUTE_WAVES;
+    const int first = wave * chunks_per_wave * 64;
+
+    auto same_key_mask = [&](int key) -> unsigned long long {
+        unsigned long long mask = __ballot(key >= 0);
+        for (int b = 0; b < 11; ++b) {
+            const unsigned long long set = __ballot((key >> b) & 1);
+            mask &= ((key >> b) & 1) ? set : ~set;
+        }
+        return key >= 0 ? mask : 0ull;
+    };
+
+    for (int c = 0; c < chunks_per_wave; ++c) {
+        const int i = first + c * 64 + lane;
+        int key = -1;
+        if (i < n && a.routes[i] != 0.0f) key = a.ids[i];
+        const unsigned long long mask = same_key_mask(key);
+        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull)
+            bins[wave][key] += __popcll(mask);
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+
+    // bucket sizes -> padded exclusive scan (256 threads x 8 experts)
+    constexpr int PER = ROUTE_MAX_EXPERTS / (ROUTE_WAVES * 64);
+    int sizes[PER];
+    int local = 0;
+    for (int j = 0; j < PER; ++j) {
+        const int e = t * PER + j;
+        int cnt = 0;
+        if (e < E) {
+            for (int w = 0; w < ROUTE_WAVES; ++w) cnt += bins[w][e];
+        } else if (e == E && a.shared) {
+            cnt = a.rows;
+        }
+        sizes[j] = (cnt + 31) & ~31;
+        local += sizes[j];
+    }
+    partial[t] = local;
+    __syncthreads();
+    for (int off = 1; off < ROUTE_WAVES * 64; off <<= 1) {
+        const int v = t >= off ? partial[t - off] : 0;
+        __syncthreads();
+        partial[t] += v;
+        __syncthreads();
+    }
+    int run = partial[t] - local;
+    for (int j = 0; j < PER; ++j) {
+        const int e = t * PER + j;
+        if (e <= Etot) start[e] = run;
+        if (e < Etot) {
+            for (int b = 0; b < sizes[j] / 32; ++b) {
+                const int blk = run / 32 + b;
+                if (blk < a.max_blocks) a.blk_expert[blk] = e;
+            }
+        }
+        run += sizes[j];
+    }
+    if (t == ROUTE_WAVES * 64 - 1) {
+        a.num_blocks[0] = min(partial[t] / 32, a.max_blocks);
+    }
+    __syncthreads();
+    // per-wave running offsets
+    for (int e = t; e < E; e += ROUTE_WAVES * 64) {
+        int base = start[e];
+        for (int w = 0; w < ROUTE_WAVES; ++w) {
+            const int cnt = bins[w][e];
+            bins[w][e] = base;
+            base += cnt;
+        }
+    }
+    __syncthreads();
+    int assigned = 0;
+    for (int c = 0; c < chunks_per_wave; ++c) {
+        const int i = first + c * 64 + lane;
+        int key = -1;
+        if (i < n && a.routes[i] != 0.0f) key = a.ids[i];
+        const unsigned long long mask = same_key_mask(key);
+        int dest = -1;
+        if (key >= 0) {
+            const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+            dest = bins[wave][key] + rank;
+            ++assigned;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull) bins[wave][key] += __popcll(mask);
+        __builtin_amdgcn_wave_barrier();
+        if (i < n) a.dest_rows[(size_t)(i / a.top_k) * slots + (i % a.top_k)] = dest;
+    }
+    if (a.shared)
+        for (int r = t; r < a.rows; r += ROUTE_WAVES * 64) a.dest_rows[(size_t)r * slots + a.top_k] = start[E] + r;
+    // total number of live assignments (for the all-routes-dropped check)
+    partial[t] = assigned;
+    __syncthreads();
+    if (t == 0) {
+        int total = a.shared ? a.rows : 0;
+        for (int i = 0; i < ROUTE_WAVES * 64; ++i) total += partial[i];
+        a.num_blocks[1] = total;
+    }
+}
+
+// out[t, n] = sum over slots, in slot order, of fma(Y[dest, n], w, out); the
+// shared expert is the last slot with coefficient 1.
+__global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a) {
+    const int tkn = blockIdx.y;
+    const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n >= a.H) return;
+    const int slots = a.top_k + a.shared;
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < slots; ++s) {
+        const int d = a.dest_rows[(size_t)tkn * slots + s];
+        if (d < 0) continue;
+        const float w = s < a.top_k ? a.routes[(size_t)tkn * a.top_k + s] : 1.0f;
+        const float4 y = *reinterpret_cast<const float4*>(a.Y + (size_t)d * a.H + n);
+        sum.x = fmaf(y.x, w, sum.x);
+        sum.y = fmaf(y.y, w, sum.y);
+        sum.z = fmaf(y.z, w, sum.z);
+        sum.w = fmaf(y.w, w, sum.w);
+    }
+    *reinterpret_cast<float4*>(a.out + (size_t)tkn * a.H + n) = sum;
+}
+
+// ------------------------------------------------------------- launchers
+template <int WM, int WN, int TM, int TN>
+int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    const bool grouped = g.blk_expert != nullptr;
+    const int mblocks = grouped ? (g.max_blocks + BM / 32 - 1) / (BM / 32) : (g.M + BM - 1) / BM;
+    const int cols = g.N;
+    const int nblocks = (cols + BN - 1) / BN;
+    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 64);
+    if (ksplit > ksteps_total) ksplit = ksteps_total;
+    if (ksplit < 1 || grouped) ksplit = 1;
+    const int per = (ksteps_total + ksplit - 1) / ksplit;
+    ksplit = (ksteps_total + per - 1) / per;
+    const dim3 grid(mblocks * nblocks * ksplit), block(WM * WN * 64);
+#define RK_LAUNCH(W4, EPI, GR)                                                              \
+    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, W4, EPI, GR>), grid, block, 0, st, g,   \
+                       mblocks, nblocks, ksplit, per)
+#define RK_BY_EPI(W4, GR)                                                  \
+    switch (g.epilogue) {                                                  \
+    case RKH_EPI_I32: RK_LAUNCH(W4, RKH_EPI_I32, GR); break;               \
+    case RKH_EPI_F16: RK_LAUNCH(W4, RKH_EPI_F16, GR); break;               \
+    case RKH_EPI_F32: RK_LAUNCH(W4, RKH_EPI_F32, GR); break;               \
+    case RKH_EPI_SWIGLU:                                                   \
+        if (TN % 2 == 0) RK_LAUNCH(W4, (TN % 2 == 0 ? RKH_EPI_SWIGLU : RKH_EPI_F32), GR); \
+        else return RKH_ERR_RUNTIME;                                       \
+        break;                                                             \
+    default: return RKH_ERR_RUNTIME;                                       \
+    }
+    if (grouped) {
+        if (g.w_int4) return RKH_ERR_RUNTIME;
+        RK_BY_EPI(false, true)
+    } else if (g.w_int4) {
+        RK_BY_EPI(true, false)
+    } else {
+        RK_BY_EPI(false, false)
+    }
+#undef RK_BY_EPI
+#undef RK_LAUNCH
+    RKH_CHECK(hipGetLastError());
+    if (ksplit > 1) {
+        const int ld = nblocks * BN;
+        const int width = g.epilogue == RKH_EPI_SWIGLU ? g.interleave_F : ld;
+        const dim3 egrid((width + 255) / 256, g.M);
+        hipLaunchKernelGGL(splitk_epilogue_kernel, egrid, dim3(256), 0, st, g, ld);
+        RKH_CHECK(hipGetLastError());
+    }
+    return RKH_OK;
+}
+
+template <int MR>
+int launch_gemv(hipStream_t st, const rkh_gemm_args& g) {
+    const int pblocks = (int)(rkh_align_up(g.N, 32) / 32);
+    const dim3 grid(pblocks), block(GEMV_WAVES * 64);
+    if (g.w_int4) hipLaunchKernelGGL((gemv_kernel<MR, true>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemv_kernel<MR, false>), grid, block, 0, st, g);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int g_fail_malloc_after = 0;
+
+} // namespace
+
+// =================================================================== C ABI
+extern "C" {
+
+int rkh_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int rkh_open(int device, void** stream_out, char* name_out, int name_len, int* cu_count,
+             int* clock_khz) {
+    RKH_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    RKH_CHECK(hipGetDeviceProperties(&prop, device));
+    if (name_out && name_len > 0) {
+        int i = 0;
+        for (; i < name_len - 1 && prop.gcnArchName[i]; ++i) name_out[i] = prop.gcnArchName[i];
+        name_out[i] = 0;
+    }
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    hipStream_t st;
+    RKH_CHECK(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    *stream_out = st;
+    return RKH_OK;
+}
+
+void rkh_close(int device, void* stream) {
+    if (hipSetDevice(device) != hipSuccess) return;
+    if (stream) {
+        (void)hipStreamSynchronize((hipStream_t)stream);
+        (void)hipStreamDestroy((hipStream_t)stream);
+    }
+}
+
+void rkh_fail_malloc_after(int n) { g_fail_malloc_after = n; }
+
+int rkh_malloc(int device, void** ptr, size_t bytes) {
+    *ptr = nullptr;
+    if (g_fail_malloc_after > 0 && --g_fail_malloc_after == 0) return RKH_ERR_NOMEM;
+    RKH_CHECK(hipSetDevice(device));
+    if (bytes == 0) bytes = 16;
+    RKH_CHECK(hipMalloc(ptr, bytes));
+    return RKH_OK;
+}
+
+void rkh_free(int device, void* ptr) {
+    if (!ptr) return;
+    if (hipSetDevice(device) != hipSuccess) return;
+    (void)hipFree(ptr);
+}
+
+int rkh_host_alloc(void** ptr, size_t bytes) {
+    *ptr = nullptr;
+    RKH_CHECK(hipHostMalloc(ptr, bytes ? bytes : 16, hipHostMallocDefault));
+    return RKH_OK;
+}
+void rkh_host_free(void* ptr) {
+    if (ptr) (void)hipHostFree(ptr);
+}
+
+int rkh_h2d(void* stream, void* dst, const void* src, size_t bytes) {
+    if (!bytes) return RKH_OK;
+    RKH_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    return RKH_OK;
+}
+int rkh_d2h(void* stream, void* dst, const void* src, size_t bytes) {
+    if (!bytes) return RKH_OK;
+    RKH_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    return RKH_OK;
+}
+int rkh_d2d(void* stream, void* dst, const void* src, size_t bytes) {
+    if (!bytes) return RKH_OK;
+    RKH_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return RKH_OK;
+}
+int rkh_fill32(void* stream, void* dst, uint32_t value, size_t words) {
+    if (!words) return RKH_OK;
+    const int blocks = (int)((words + 255) / 256 < 4096 ? (words + 255) / 256 : 4096);
+    hipLaunchKernelGGL(fill32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<uint32_t*>(dst), value, words);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+int rkh_sync(void* stream) {
+    RKH_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return RKH_OK;
+}
+
+int rkh_event_create(void** event) {
+    hipEvent_t e;
+    RKH_CHECK(hipEventCreate(&e));
+    *event = e;
+    return RKH_OK;
+}
+void rkh_event_destroy(void* event) {
+    if (event) (void)hipEventDestroy((hipEvent_t)event);
+}
+int rkh_event_record(void* event, void* stream) {
+    RKH_CHECK(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return RKH_OK;
+}
+int rkh_event_elapsed_us(void* start, void* stop, double* us) {
+    RKH_CHECK(hipEventSynchronize((hipEvent_t)stop));
+    float ms = 0.0f;
+    RKH_CHECK(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop));
+    *us = (double)ms * 1000.0;
+    return RKH_OK;
+}
+
+int rkh_pack_w8(void* stream, const int8_t* src, int K, int N, int interleave_F, uint8_t* dst) {
+    const int KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
+    const size_t pblocks = (size_t)(rkh_align_up(N, RKH_COL_ALIGN) / 32);
+    const size_t chunks = pblocks * KB * 64;
+    hipLaunchKernelGGL(pack_w8_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, src, K, N, KB, interleave_F, dst, chunks);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int rkh_pack_w4(void* stream, const int8_t* src, int K, int N, int interleave_F, uint8_t* dst,
+                int* bad_flag) {
+    const int KB2 = (int)(rkh_align_up(K, RKH_K_ALIGN) / 64);
+    const size_t pblocks = (size_t)(rkh_align_up(N, RKH_COL_ALIGN) / 32);
+    const size_t chunks = pblocks * KB2 * 64;
+    hipLaunchKernelGGL(pack_w4_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, src, K, N, KB2, interleave_F, dst, chunks, bad_flag);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
+    if (args->M <= 0) return RKH_OK;
+    const dim3 grid(args->M), block(256);
+    switch (args->in_dtype) {
+    case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args); break;
+    case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args); break;
+    case RKH_I8: hipLaunchKernelGGL(quant_rows_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args); break;
+    default: return RKH_ERR_RUNTIME;
+    }
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+// Dense launch plan: rows per workgroup follow M, shrinking while the output
+// grid cannot fill the 256 compute units; what is still missing is made up by
+// splitting K (exact: integer partial sums are added atomically).
+// int4 operands ride as 16 * code, so one K part may span at most 2^17 k
+// before the int32 sum could wrap.
+struct DensePlan { int bm, ksplit; };
+static int min_ksplit(int K, int w_int4) {
+    return w_int4 ? (int)((rkh_align_up(K, RKH_K_ALIGN) + 131071) / 131072) : 1;
+}
+static DensePlan dense_plan(int M, int N, int K, int w_int4) {
+    const int ksteps = (int)(rkh_align_up(K, RKH_K_ALIGN) / 64);
+    int bm = M > 64 ? 128 : M > 32 ? 64 : 32;
+    auto tiles_of = [&](int rows) { return (long)((M + rows - 1) / rows) * ((N + 255) / 256); };
+    while (bm > 32 && tiles_of(bm) < 160) bm >>= 1;
+    const long tiles = tiles_of(bm);
+    int s = 1;
+    if (tiles < 192) {
+        s = (int)((256 + tiles - 1) / tiles);
+        const int max_s = ksteps / 8 > 0 ? ksteps / 8 : 1; // at least 512 k per part
+        if (s > max_s) s = max_s;
+    }
+    const int need = min_ksplit(K, w_int4);
+    return {bm, s > need ? s : need};
+}
+
+size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
+    if (M <= 8) return 0;
+    if (dense_plan(M, N, K, w_int4).ksplit <= 1) return 0;
+    return (size_t)rkh_align_up(M, RKH_ROW_ALIGN) * (size_t)rkh_align_up(N, RKH_COL_ALIGN) * 4;
+}
+
+int rkh_gemm(void* stream, const rkh_gemm_args* args) {
+    const rkh_gemm_args& g = *args;
+    hipStream_t st = (hipStream_t)stream;
+    const bool grouped = g.blk_expert != nullptr;
+    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) {
+        if (g.M == 1) return launch_gemv<1>(st, g);
+        if (g.M == 2) return launch_gemv<2>(st, g);
+        if (g.M <= 4) return launch_gemv<4>(st, g);
+        return launch_gemv<8>(st, g);
+    }
+    if (grouped) return launch_gemm_cfg<1, 4, 1, 2>(st, g, 1);
+    const DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
+    int ksplit = plan.ksplit;
+    if (ksplit > 1 && !g.splitk_acc) {
+        if (min_ksplit(g.K, g.w_int4) > 1) return RKH_ERR_RUNTIME;
+        ksplit = 1;
+    }
+    const int bm = plan.bm;
+    if (bm == 128) return launch_gemm_cfg<2, 2, 2, 4>(st, g, ksplit);
+    if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2>(st, g, ksplit);
+    return launch_gemm_cfg<1, 4, 1, 2>(st, g, ksplit);
+}
+
+int rkh_moe_route(void* stream, const rkh_moe_route_args* args) {
+    if (args->experts + args->shared > ROUTE_MAX_EXPERTS) return RKH_ERR_RUNTIME;
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(ROUTE_WAVES * 64), 0, (hipStream_t)stream, *args);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args) {
+    const dim3 grid((args->H / 4 + 255) / 256, args->rows);
+    hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, (hipStream_t)stream, *args);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,431 @@
+// Routed W8A8 SwiGLU experts.
+//
+// Replaces src/rk_npu_moe_w8.cpp of the reference, where the CPU buckets
+// (token, slot) pairs by expert, the NPU gathers rows and runs one GEMM job
+// per <=128-row slice, and the CPU computes the SwiGLU middle row by row.
+// Here one call is six kernels on one stream:
+//   route (stable bucket by expert, 32-row padded) -> quantize tokens straight
+//   into their sorted rows -> grouped gate/up GEMM with fused SwiGLU + row max
+//   -> re-quantize (ties to even) -> grouped down GEMM -> weighted combine.
+// Validation and its order follow src/rk_npu_moe_w8.cpp:293-310,574-608,846-875.
+#include <algorithm>
+#include <new>
+
+#include "rk_host.h"
+#include "rk_npu_hip.h"
+#include "rk_npu_moe_w8.h"
+
+using namespace rkhost;
+
+namespace {
+
+constexpr int kMaxIntermediate = 8192; // the reference stops at 512 (fixed CPU row buffer)
+constexpr int kMaxExperts = 2047;      // routed + shared must fit the route kernel's tables
+
+bool valid(const rk_npu_moe_w8_weight_config& c) {
+    return c.hidden >= 64 && c.hidden % 32 == 0 && c.intermediate >= 32 &&
+           c.intermediate <= kMaxIntermediate && c.intermediate % 32 == 0 &&
+           c.routed_experts >= 1 && c.routed_experts <= kMaxExperts &&
+           (c.shared_expert == 0 || c.shared_expert == 1);
+}
+bool same(const rk_npu_moe_w8_weight_config& a, const rk_npu_moe_w8_weight_config& b) {
+    return a.hidden == b.hidden && a.intermediate == b.intermediate &&
+           a.routed_experts == b.routed_experts && a.shared_expert == b.shared_expert;
+}
+bool valid(const rk_npu_moe_w8_config& c) {
+    return c.struct_size == sizeof(c) && valid(c.weights) && c.max_rows >= 1 && c.max_rows <= 256 &&
+           c.top_k >= 1 && c.top_k <= std::min(c.weights.routed_experts, 8) && c.npu_cores >= 1 &&
+           c.npu_cores <= 3 && c.cpu_threads >= 1 && c.cpu_threads <= 4 &&
+           (c.native_input == 0 || c.native_input == 1) && c.timeout_ms >= 1 &&
+           c.timeout_ms <= 60000 && c.middle == RK_NPU_MOE_MIDDLE_CPU;
+}
+bool overlap(const void* a, size_t na, const void* b, size_t nb) {
+    const auto x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+    return x <= y ? y - x < na : x - y < nb;
+}
+
+} // namespace
+
+struct rk_npu_moe_w8_weights {
+    Owner owner;
+    rk_npu_moe_w8_weight_config config{};
+    int count = 0;              // routed + shared
+    size_t gate_stride = 0;     // bytes between experts in gate_up
+    size_t down_stride = 0;
+    DeviceBuffer gate_up;       // count x tiled int8 [align256(2I) x align64(H)], gate/up interleaved
+    DeviceBuffer down;          // count x tiled int8 [align256(H) x align64(I)]
+    DeviceBuffer gate_scales;   // count x [2I]
+    DeviceBuffer down_scales;   // count x [H]
+    uint64_t bytes() const {
+        return gate_up.bytes() + down.bytes() + gate_scales.bytes() + down_scales.bytes();
+    }
+};
+
+struct rk_npu_moe_w8_workspace {
+    Owner owner;
+    rk_npu_moe_w8_config config{};
+    int slots = 0, max_blocks = 0, sorted_rows = 0;
+    DeviceBuffer input;        // [max_rows, H] fp32 (or int8) as uploaded
+    DeviceBuffer token_scale;  // [max_rows]
+    DeviceBuffer ids, routes;  // [max_rows, top_k]
+    DeviceBuffer dest_rows;    // [max_rows, slots]
+    DeviceBuffer blk_expert;   // [max_blocks]
+    DeviceBuffer num_blocks;   // [2]
+    DeviceBuffer a_tiled;      // sorted token rows, tiled int8 [sorted_rows x align64(H)]
+    DeviceBuffer a_scale;      // [sorted_rows]
+    DeviceBuffer hidden;       // [sorted_rows, I] fp32
+    DeviceBuffer row_max;      // [sorted_rows]
+    DeviceBuffer h_tiled;      // re-quantized hidden, tiled int8 [sorted_rows x align64(I)]
+    DeviceBuffer h_scale;      // [sorted_rows]
+    DeviceBuffer y;            // [sorted_rows, H] fp32 expert outputs
+    DeviceBuffer out;          // [max_rows, H] fp32
+    BadFlag flag;
+    std::atomic_flag busy = ATOMIC_FLAG_INIT;
+    uint64_t bytes() const {
+        return input.bytes() + token_scale.bytes() + ids.bytes() + routes.bytes() +
+               dest_rows.bytes() + blk_expert.bytes() + num_blocks.bytes() + a_tiled.bytes() +
+               a_scale.bytes() + hidden.bytes() + row_max.bytes() + h_tiled.bytes() +
+               h_scale.bytes() + y.bytes() + out.bytes();
+    }
+    ~rk_npu_moe_w8_workspace() {
+        if (owner.ctx) {
+            std::lock_guard<std::mutex> lock(owner.ctx->pending_mutex);
+            auto& v = owner.ctx->pending_flags;
+            v.erase(std::remove(v.begin(), v.end(), flag.device()), v.end());
+        }
+    }
+};
+
+namespace {
+
+// Kernel sequence on device-resident inputs.  d_input is fp32 [rows, H] when
+// f32, else int8 [rows, H] with d_scales[rows].
+int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int rows,
+            const void* d_input, bool f32, const float* d_scales, const int32_t* d_ids,
+            const float* d_routes, float* d_out, StageTimer* timer) {
+    const auto& wc = ws->config.weights;
+    const int H = wc.hidden, I = wc.intermediate;
+    void* stream = ws->owner.ctx->stream;
+    auto mark = [&] { if (timer) timer->mark(); };
+
+    rkh_moe_route_args r{};
+    r.ids = d_ids;
+    r.routes = d_routes;
+    r.rows = rows;
+    r.top_k = ws->config.top_k;
+    r.experts = wc.routed_experts;
+    r.shared = wc.shared_expert;
+    r.dest_rows = ws->dest_rows.as<int>();
+    r.blk_expert = ws->blk_expert.as<int>();
+    r.num_blocks = ws->num_blocks.as<int>();
+    r.max_blocks = ws->max_blocks;
+    int rc = rkh_moe_route(stream, &r);
+    if (rc) return map_error(rc);
+    mark(); // 1: schedule
+
+    rkh_quant_args q{};
+    q.src = d_input;
+    q.in_dtype = f32 ? RKH_F32 : RKH_I8;
+    q.mode = f32 ? RKH_Q_MOE : RKH_Q_COPY_I8;
+    q.M = rows;
+    q.K = H;
+    q.scale = f32 ? ws->token_scale.as<float>() : const_cast<float*>(d_scales);
+    q.dst = ws->a_tiled.as<>();
+    q.bad_flag = ws->flag.device();
+    q.zero_bits = ws->row_max.as<uint32_t>();
+    q.dest_rows = ws->dest_rows.as<int>();
+    q.dest_stride = ws->slots;
+    q.scale_rows = ws->a_scale.as<float>();
+    rc = rkh_quant_rows(stream, &q);
+    if (rc) return map_error(rc);
+    mark(); // 2: input
+
+    rkh_gemm_args g{};
+    g.A = ws->a_tiled.as<>();
+    g.W = w->gate_up.as<>();
+    g.M = ws->sorted_rows;
+    g.N = 2 * I;
+    g.K = H;
+    g.interleave_F = I;
+    g.a_scale = ws->a_scale.as<float>();
+    g.w_scale = w->gate_scales.as<float>();
+    g.epilogue = RKH_EPI_SWIGLU;
+    g.C = ws->hidden.as<>();
+    g.ldc = I;
+    g.row_max_bits = ws->row_max.as<uint32_t>();
+    g.blk_expert = ws->blk_expert.as<int>();
+    g.num_blocks = ws->num_blocks.as<int>();
+    g.max_blocks = ws->max_blocks;
+    g.w_expert_stride = w->gate_stride;
+    g.ws_expert_stride = (size_t)2 * I;
+    rc = rkh_gemm(stream, &g);
+    if (rc) return map_error(rc);
+    mark(); // 3: gate
+
+    rkh_quant_args q2{};
+    q2.src = ws->hidden.as<>();
+    q2.in_dtype = RKH_F32;
+    q2.mode = RKH_Q_REUSE_BITS_MOE;
+    q2.M = ws->sorted_rows;
+    q2.K = I;
+    q2.scale = ws->h_scale.as<float>();
+    q2.dst = ws->h_tiled.as<>();
+    q2.row_max_bits = ws->row_max.as<uint32_t>();
+    q2.active_blocks = ws->num_blocks.as<int>();
+    rc = rkh_quant_rows(stream, &q2);
+    if (rc) return map_error(rc);
+    mark(); // 4: middle
+
+    rkh_gemm_args d{};
+    d.A = ws->h_tiled.as<>();
+    d.W = w->down.as<>();
+    d.M = ws->sorted_rows;
+    d.N = H;
+    d.K = I;
+    d.a_scale = ws->h_scale.as<float>();
+    d.w_scale = w->down_scales.as<float>();
+    d.epilogue = RKH_EPI_F32;
+    d.C = ws->y.as<>();
+    d.ldc = H;
+    d.blk_expert = ws->blk_expert.as<int>();
+    d.num_blocks = ws->num_blocks.as<int>();
+    d.max_blocks = ws->max_blocks;
+    d.w_expert_stride = w->down_stride;
+    d.ws_expert_stride = (size_t)H;
+    rc = rkh_gemm(stream, &d);
+    if (rc) return map_error(rc);
+    mark(); // 5: down
+
+    rkh_moe_combine_args c{};
+    c.Y = ws->y.as<float>();
+    c.dest_rows = ws->dest_rows.as<int>();
+    c.routes = d_routes;
+    c.rows = rows;
+    c.top_k = ws->config.top_k;
+    c.shared = wc.shared_expert;
+    c.H = H;
+    c.out = d_out;
+    rc = rkh_moe_combine(stream, &c);
+    mark(); // 6: combine
+    return map_error(rc);
+}
+
+int check_handles(const rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w) {
+    if (!same(ws->config.weights, w->config)) return RK_NPU_ERR_PARAM;
+    if (!w->owner.same(ws->owner)) return RK_NPU_ERR_DOMAIN;
+    return RK_NPU_OK;
+}
+
+// reference src/rk_npu_moe_w8.cpp:846-875 (argument checks, BUSY) and :574-608
+// (handle match, id / coefficient / scale validation before any device work).
+int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int rows,
+            const void* input, bool f32, const float* scales, const int32_t* ids,
+            const float* routes, float* output, rk_npu_moe_w8_timings* timings) {
+    if (timings) *timings = rk_npu_moe_w8_timings{};
+    if (!ws || !w || !input || !ids || !routes || !output || (!f32 && !scales) || rows < 1 ||
+        rows > ws->config.max_rows)
+        return RK_NPU_ERR_PARAM;
+    const int H = ws->config.weights.hidden, top = ws->config.top_k;
+    const size_t values = (size_t)rows * H, nslots = (size_t)rows * top;
+    if (overlap(input, values * (f32 ? 4 : 1), output, values * 4) ||
+        overlap(ids, nslots * 4, output, values * 4) || overlap(routes, nslots * 4, output, values * 4) ||
+        (!f32 && overlap(scales, (size_t)rows * 4, output, values * 4)))
+        return RK_NPU_ERR_PARAM;
+    BusyLock lock(ws->busy);
+    if (!lock) return RK_NPU_ERR_BUSY;
+    const auto t0 = Clock::now();
+    int rc = check_handles(ws, w);
+    if (rc) return rc;
+    const int E = ws->config.weights.routed_experts;
+    size_t live = ws->config.weights.shared_expert ? (size_t)rows : 0;
+    for (size_t i = 0; i < nslots; ++i) {
+        if (ids[i] < 0 || ids[i] >= E || !std::isfinite(routes[i]) || routes[i] < 0)
+            return RK_NPU_ERR_PARAM;
+        if (routes[i] != 0) ++live;
+    }
+    if (!f32 && !finite_positive(scales, (size_t)rows)) return RK_NPU_ERR_PARAM;
+    rk_npu_ctx* ctx = ws->owner.ctx;
+    if (!live) {
+        // every route dropped and no shared expert: the result is all zeros
+        // and no device work is issued -- but fp32 input must still be finite
+        if (f32) {
+            const float* x = static_cast<const float*>(input);
+            for (size_t i = 0; i < values; ++i)
+                if (!std::isfinite(x[i])) return RK_NPU_ERR_PARAM;
+        }
+        std::fill_n(output, values, 0.0f);
+        if (timings) timings->total_us = timings->combine_us = elapsed_us(t0);
+        return RK_NPU_OK;
+    }
+    StageTimer timer(ctx->stream, timings != nullptr);
+    {
+        std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+        rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, values * (f32 ? 4 : 1)));
+        if (!rc && !f32) rc = map_error(rkh_h2d(ctx->stream, ws->token_scale.as<>(), scales, (size_t)rows * 4));
+        if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->ids.as<>(), ids, nslots * 4));
+        if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->routes.as<>(), routes, nslots * 4));
+        timer.mark(); // 0
+        if (!rc)
+            rc = enqueue(ws, w, rows, ws->input.as<>(), f32, ws->token_scale.as<float>(),
+                         ws->ids.as<int32_t>(), ws->routes.as<float>(), ws->out.as<float>(), &timer);
+        if (!rc) rc = ws->flag.enqueue_readback(ctx->stream);
+    }
+    const int wait = map_error(rkh_sync(ctx->stream));
+    if (rc || wait) return rc ? rc : wait;
+    if (ws->flag.consume(ctx->stream)) return RK_NPU_ERR_PARAM; // NaN / Inf token
+    const auto t1 = Clock::now();
+    rc = map_error(rkh_d2h(ctx->stream, output, ws->out.as<>(), values * 4));
+    if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    if (timings) {
+        timings->schedule_us = timer.span_us(0, 1);
+        timings->input_us = timer.span_us(1, 2);
+        timings->gate_us = timer.span_us(2, 3);
+        timings->middle_cpu_us = timer.span_us(3, 4);
+        timings->down_us = timer.span_us(4, 5);
+        timings->combine_us = timer.span_us(5, 6);
+        timings->sync_us = elapsed_us(t1);
+        timings->gemm_tasks = 2;
+        timings->gather_tasks = 1;
+        timings->middle_tasks = 1;
+        timings->total_us = elapsed_us(t0);
+    }
+    return rc;
+}
+
+} // namespace
+
+extern "C" {
+
+void rk_npu_moe_w8_config_init(rk_npu_moe_w8_config* c, int hidden, int intermediate,
+                               int routed_experts, int shared_expert, int top_k, int max_rows) {
+    if (!c) return;
+    std::memset(c, 0, sizeof(*c));
+    c->struct_size = sizeof(*c);
+    c->weights.hidden = hidden;
+    c->weights.intermediate = intermediate;
+    c->weights.routed_experts = routed_experts;
+    c->weights.shared_expert = shared_expert;
+    c->max_rows = max_rows;
+    c->top_k = top_k;
+    c->npu_cores = 3;
+    c->cpu_threads = 4;
+    c->native_input = 0;
+    c->middle = RK_NPU_MOE_MIDDLE_CPU;
+    c->timeout_ms = 1000;
+}
+
+rk_npu_moe_w8_weights* rk_npu_moe_w8_weights_create(rk_npu_iommu_domain* domain,
+                                                    const rk_npu_moe_w8_weight_config* config,
+                                                    const rk_npu_moe_w8_expert* experts) {
+    if (!domain || !domain->ctx || !config || !experts || !valid(*config)) return nullptr;
+    const int H = config->hidden, I = config->intermediate;
+    const int count = config->routed_experts + config->shared_expert;
+    for (int e = 0; e < count; ++e) {
+        const auto& x = experts[e];
+        if (!x.gate_up || !x.down || !finite_positive(x.gate_up_scales, (size_t)2 * I) ||
+            !finite_positive(x.down_scales, (size_t)H))
+            return nullptr;
+    }
+    std::unique_ptr<rk_npu_moe_w8_weights> w(new (std::nothrow) rk_npu_moe_w8_weights());
+    if (!w) return nullptr;
+    w->owner.bind(domain);
+    w->config = *config;
+    w->count = count;
+    w->gate_stride = rkh_tiled_i8_bytes(2 * I, H, RKH_COL_ALIGN);
+    w->down_stride = rkh_tiled_i8_bytes(H, I, RKH_COL_ALIGN);
+    rk_npu_ctx* ctx = domain->ctx;
+    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
+    DeviceBuffer raw;
+    if (w->gate_up.alloc(w->owner, w->gate_stride * count, false) ||
+        w->down.alloc(w->owner, w->down_stride * count, false) ||
+        w->gate_scales.alloc(w->owner, (size_t)count * 2 * I * sizeof(float), false) ||
+        w->down_scales.alloc(w->owner, (size_t)count * H * sizeof(float), false) ||
+        raw.alloc(w->owner, (size_t)H * 2 * I, false))
+        return nullptr;
+    for (int e = 0; e < count; ++e) {
+        const auto& x = experts[e];
+        int rc = rkh_h2d(ctx->stream, raw.as<>(), x.gate_up, (size_t)H * 2 * I);
+        if (!rc) rc = rkh_pack_w8(ctx->stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e);
+        if (!rc) rc = rkh_h2d(ctx->stream, raw.as<>(), x.down, (size_t)I * H);
+        if (!rc) rc = rkh_pack_w8(ctx->stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e);
+        if (!rc) rc = rkh_h2d(ctx->stream, w->gate_scales.as<float>() + (size_t)e * 2 * I, x.gate_up_scales, (size_t)2 * I * sizeof(float));
+        if (!rc) rc = rkh_h2d(ctx->stream, w->down_scales.as<float>() + (size_t)e * H, x.down_scales, (size_t)H * sizeof(float));
+        // the staging buffer is reused: finish this expert before the next copy lands
+        if (!rc) rc = rkh_sync(ctx->stream);
+        if (rc) return nullptr;
+    }
+    return w.release();
+}
+
+void rk_npu_moe_w8_weights_free(rk_npu_moe_w8_weights* weights) { delete weights; }
+
+rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* domain,
+                                                        const rk_npu_moe_w8_config* config) {
+    if (!domain || !domain->ctx || !config || !valid(*config)) return nullptr;
+    std::unique_ptr<rk_npu_moe_w8_workspace> ws(new (std::nothrow) rk_npu_moe_w8_workspace());
+    if (!ws) return nullptr;
+    ws->owner.bind(domain);
+    ws->config = *config;
+    const auto& wc = config->weights;
+    const int R = config->max_rows, H = wc.hidden, I = wc.intermediate, top = config->top_k;
+    ws->slots = top + wc.shared_expert;
+    const int routed = R * top;
+    ws->max_blocks = routed / 32 + std::min(wc.routed_experts, routed) + (wc.shared_expert ? (R + 31) / 32 : 0);
+    ws->sorted_rows = ws->max_blocks * 32;
+    const size_t S = (size_t)ws->sorted_rows;
+    std::lock_guard<std::mutex> lock(domain->ctx->submit_mutex);
+    if (ws->input.alloc(ws->owner, (size_t)R * H * 4, false) ||
+        ws->token_scale.alloc(ws->owner, (size_t)R * 4) || ws->ids.alloc(ws->owner, (size_t)routed * 4) ||
+        ws->routes.alloc(ws->owner, (size_t)routed * 4) ||
+        ws->dest_rows.alloc(ws->owner, (size_t)R * ws->slots * 4) ||
+        ws->blk_expert.alloc(ws->owner, (size_t)ws->max_blocks * 4) ||
+        ws->num_blocks.alloc(ws->owner, 16) ||
+        ws->a_tiled.alloc(ws->owner, rkh_tiled_i8_bytes(ws->sorted_rows, H, 32)) ||
+        ws->a_scale.alloc(ws->owner, S * 4) || ws->hidden.alloc(ws->owner, S * I * 4) ||
+        ws->row_max.alloc(ws->owner, S * 4) ||
+        ws->h_tiled.alloc(ws->owner, rkh_tiled_i8_bytes(ws->sorted_rows, I, 32)) ||
+        ws->h_scale.alloc(ws->owner, S * 4) || ws->y.alloc(ws->owner, S * H * 4) ||
+        ws->out.alloc(ws->owner, (size_t)R * H * 4, false) || ws->flag.init(ws->owner))
+        return nullptr;
+    if (rkh_sync(domain->ctx->stream)) return nullptr;
+    return ws.release();
+}
+
+void rk_npu_moe_w8_workspace_free(rk_npu_moe_w8_workspace* workspace) { delete workspace; }
+
+uint64_t rk_npu_moe_w8_weights_device_bytes(const rk_npu_moe_w8_weights* w) {
+    return w ? w->bytes() : 0;
+}
+uint64_t rk_npu_moe_w8_workspace_device_bytes(const rk_npu_moe_w8_workspace* w) {
+    return w ? w->bytes() : 0;
+}
+
+int rk_npu_moe_w8_run_quantized(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w,
+                                int rows, const int8_t* input, const float* row_scales,
+                                const int32_t* ids, const float* routes, float* out,
+                                rk_npu_moe_w8_timings* t) {
+    return moe_run(ws, w, rows, input, false, row_scales, ids, routes, out, t);
+}
+int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int rows,
+                          const float* input, const int32_t* ids, const float* routes, float* out,
+                          rk_npu_moe_w8_timings* t) {
+    return moe_run(ws, w, rows, input, true, nullptr, ids, routes, out, t);
+}
+
+// Device-resident variant: ids / coefficients are trusted to be in range (they
+// cannot be inspected without a copy back); NaN / Inf tokens are still flagged.
+int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w,
+                                 int rows, const float* input, const int32_t* ids,
+                                 const float* routes, float* out) {
+    if (!ws || !w || !input || !ids || !routes || !out || rows < 1 || rows > ws->config.max_rows)
+        return RK_NPU_ERR_PARAM;
+    BusyLock lock(ws->busy);
+    if (!lock) return RK_NPU_ERR_BUSY;
+    int rc = check_handles(ws, w);
+    if (rc) return rc;
+    std::lock_guard<std::mutex> submit(ws->owner.ctx->submit_mutex);
+    note_pending_flag(ws->owner.ctx, ws->flag.device());
+    return enqueue(ws, w, rows, input, true, nullptr, ids, routes, out, nullptr);
+}
+
+} // extern "C"
