@@ -197,6 +197,41 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
     const bool cached = nchunks <= 256 * QR_CACHE;
     const int mode = a.mode;
+    if constexpr (sizeof(T) == 1) {
+        // int8 input is re-tiled byte for byte (the full range -128..127 is legal
+        // for the raw integer operator); scale[] passes through for the MoE path.
+        const int nd = a.dest_rows ? a.dest_stride : 1;
+        if (t == 0 && a.dest_rows) {
+            for (int j = 0; j < nd; ++j) {
+                const int d = a.dest_rows[(size_t)m * nd + j];
+                if (d >= 0) {
+                    if (a.scale_rows && a.scale) a.scale_rows[d] = a.scale[m];
+                    if (a.zero_bits) a.zero_bits[d] = 0u;
+                }
+            }
+        }
+        const int8_t* brow = reinterpret_cast<const int8_t*>(row);
+        for (int c = t; c < nchunks; c += 256) {
+            uint32_t w[4] = {0, 0, 0, 0};
+            if (vec && c * 16 + 16 <= K) {
+                const uint4 v4 = *reinterpret_cast<const uint4*>(brow + c * 16);
+                w[0] = v4.x; w[1] = v4.y; w[2] = v4.z; w[3] = v4.w;
+            } else {
+                for (int j = 0; j < 16; ++j)
+                    if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
+            }
+            const uint4 packed = make_uint4(w[0], w[1], w[2], w[3]);
+            if (!a.dest_rows) {
+                *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            } else {
+                for (int j = 0; j < nd; ++j) {
+                    const int d = a.dest_rows[(size_t)m * nd + j];
+                    if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+                }
+            }
+        }
+        return;
+    }
     const bool need_max = mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
     const bool check = mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
 
@@ -331,8 +366,14 @@ __device__ __forceinline__ float silu_poly(float g) {
     return g < -80.0f ? -0.0f : g / d;
 }
 
+// y = (float(acc) * as) * ws with both products rounded to fp32.  The empty asm
+// makes the value opaque so the compiler cannot merge the second multiply with a
+// following fp16 conversion into one mixed-precision instruction (which would
+// round once instead of twice and differ from the reference on ties).
 __device__ __forceinline__ float dequant(int acc, float as, float ws) {
-    return __fmul_rn(__fmul_rn((float)acc, as), ws);
+    float y = __fmul_rn(__fmul_rn((float)acc, as), ws);
+    asm volatile("" : "+v"(y));
+    return y;
 }
 
 __device__ __forceinline__ void store_out(void* C, int epi, size_t index, int acc, float as,

@@ -1,0 +1,253 @@
+"""GPU parity of the W8A8 operators against the CPU oracle, through the C ABI.
+
+Bars: int8 activations, per-row scales and int32 accumulators bit-exact;
+fp16 / fp32 outputs bit-exact as well (the epilogue is two IEEE multiplies and
+one RNE cast, which the oracle states identically), which is stricter than the
+1e-3 x absmax tolerance the benchmark configuration allows.
+"""
+import numpy as np
+import pytest
+
+from rknpu2_matmul_open_amd import capi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand_i8(rng, shape, lo=-127, hi=127):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+# reference examples/demo.cpp:58-62 runs odd shapes such as 17x40x33, 300x48x33, 1x200x200
+I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96), (17, 40, 33),
+              (33, 130, 70), (64, 256, 256), (65, 257, 129), (128, 512, 384), (300, 48, 33),
+              (200, 1000, 520)]
+
+
+@pytest.mark.parametrize("M,N,K", I32_SHAPES)
+def test_i8i8i32_exact(sess, oracle, M, N, K):
+    rng = np.random.default_rng(M * 1000003 + N * 1009 + K)
+    A = _rand_i8(rng, (M, K), -128, 127)
+    B = _rand_i8(rng, (K, N), -128, 127)
+    op = ops.W8A8Linear(sess, capi.I8I8I32, M, B)
+    try:
+        rc, got = op.run(A)
+        assert rc == 0
+        want = oracle.gemm_i8(A, B)
+        assert np.array_equal(got, want), "M=%d N=%d K=%d first diff at %s" % (
+            M, N, K, np.argwhere(got != want)[:4].tolist())
+        rc, again = op.run(A)
+        assert rc == 0 and np.array_equal(again, got)
+    finally:
+        op.close()
+
+
+def test_i8i8i32_extremes_wrap(sess, oracle):
+    # all -128 x -128 over K=131072+64 stays below 2^31; the wrap rule itself is
+    # exercised with K large enough that +16384 * K crosses 2^31.
+    M, N, K = 2, 64, 131072 + 64
+    A = np.full((M, K), -128, np.int8)
+    B = np.full((K, N), -128, np.int8)
+    op = ops.W8A8Linear(sess, capi.I8I8I32, M, B, k_tile=2048)
+    try:
+        rc, got = op.run(A)
+        assert rc == 0
+        want = np.int64(16384) * K
+        want = ((want + 2 ** 31) % 2 ** 32) - 2 ** 31
+        assert (got == want).all()
+    finally:
+        op.close()
+
+
+F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64, 128),
+              (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", F16_SHAPES)
+def test_f16i8f16_dynamic_bit_exact(sess, oracle, M, N, K):
+    c = workloads.w8a8_case(M, K, N, seed_w=M + N, seed_a=K + 7)
+    A = c["A"].copy()
+    if M > 2:
+        A[1, :] = 0                      # all-zero token: scale 1
+        A[2, : K // 2] = np.float16(0.5).view(np.uint16)  # many exact .5 multiples -> ties
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    try:
+        rc, got = op.run(A)
+        assert rc == 0
+        want = oracle.w8a8(A, c["B"], c["w_scale"])
+        q, s = op.read_quantized()
+        assert np.array_equal(s.view(np.uint32), want["a_scale"].view(np.uint32))
+        assert np.array_equal(q, want["q"])
+        assert np.array_equal(got, want["C"]), "max ulp-ish diff %d" % np.abs(
+            got.astype(np.int32) - want["C"].astype(np.int32)).max()
+    finally:
+        op.close()
+
+
+def test_f32i8f32_dynamic_and_static(sess, oracle):
+    M, N, K = 37, 200, 300
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((M, K)).astype(np.float32) * 3
+    A[0, :8] = [127, -127, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5]
+    B = _rand_i8(rng, (K, N))
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.01
+    op = ops.W8A8Linear(sess, capi.F32I8F32_DYNAMIC, M, B, ws)
+    try:
+        rc, got = op.run(A)
+        want = oracle.w8a8(A, B, ws)
+        assert rc == 0
+        assert np.array_equal(got.view(np.uint32), want["C"].view(np.uint32))
+    finally:
+        op.close()
+    a_scale = (rng.random(M).astype(np.float32) + 0.25) * 0.05
+    a_scale[0] = 1.0  # exact ties at .5 multiples with scale 1
+    for kind, Ain in ((capi.F32I8F32_STATIC, A), (capi.F16I8F16_STATIC, A.astype(np.float16).view(np.uint16))):
+        op = ops.W8A8Linear(sess, kind, M, B, ws)
+        try:
+            rc, got = op.run(Ain, a_scale)
+            want = oracle.w8a8(Ain, B, ws, a_scale_static=a_scale)
+            assert rc == 0
+            q, _ = op.read_quantized()
+            assert np.array_equal(q, want["q"])
+            assert np.array_equal(got, want["C"]) if got.dtype == np.uint16 else np.array_equal(
+                got.view(np.uint32), want["C"].view(np.uint32))
+            bad = a_scale.copy()
+            bad[3] = 0
+            rc, _ = op.run(Ain, bad)
+            assert rc == capi.RK_NPU_ERR_PARAM
+            bad[3] = np.inf
+            rc, _ = op.run(Ain, bad)
+            assert rc == capi.RK_NPU_ERR_PARAM
+        finally:
+            op.close()
+
+
+def test_config0_full(sess, oracle):
+    """BASELINE config 0: M=64, K=2048, N=2048, seeds 0/1."""
+    c = workloads.CONFIGS[0]()
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, c["M"], c["B"], c["w_scale"])
+    try:
+        rc, got = op.run(c["A"])
+        want = oracle.w8a8(c["A"], c["B"], c["w_scale"])
+        assert rc == 0
+        q, s = op.read_quantized()
+        assert np.array_equal(q, want["q"])
+        assert np.array_equal(got, want["C"])
+        # int32 accumulators through the raw-integer operator on the same codes
+        raw = ops.W8A8Linear(sess, capi.I8I8I32, c["M"], c["B"])
+        try:
+            rc, acc = raw.run(want["q"])
+            assert rc == 0 and np.array_equal(acc, want["acc"])
+        finally:
+            raw.close()
+    finally:
+        op.close()
+
+
+def test_config1_full_decode(sess, oracle):
+    """BASELINE config 1: M=1, K=4096, N=14336, seeds 2/3 (GEMV path)."""
+    c = workloads.CONFIGS[1]()
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, 1, c["B"], c["w_scale"])
+    try:
+        rc, got = op.run(c["A"])
+        want = oracle.w8a8(c["A"], c["B"], c["w_scale"])
+        assert rc == 0
+        assert np.array_equal(got, want["C"])
+        err = np.abs(oracle.half_to_float(got) - oracle.half_to_float(want["C"])).max()
+        assert err <= 1e-3 * np.abs(oracle.half_to_float(want["C"])).max()
+        raw = ops.W8A8Linear(sess, capi.I8I8I32, 1, c["B"])
+        try:
+            rc, acc = raw.run(want["q"])
+            assert rc == 0 and np.array_equal(acc, want["acc"])
+        finally:
+            raw.close()
+    finally:
+        op.close()
+
+
+def test_weight_sharing_rebinding_and_errors(sess, oracle):
+    """reference tests/test_quant_matmul.cpp:231-330: one weight serves several M,
+    a workspace can be re-bound to other compatible weights, k_tile mismatch is
+    PARAM, foreign domain is DOMAIN, wrong op kind is PARAM."""
+    lib = sess.lib
+    M, N, K = 8, 96, 96
+    rng = np.random.default_rng(11)
+    A = _rand_i8(rng, (M, K))
+    B0, B1 = _rand_i8(rng, (K, N)), _rand_i8(rng, (K, N))
+    op0 = ops.W8A8Linear(sess, capi.I8I8I32, M, B0, k_tile=32)
+    op1 = ops.W8A8Linear(sess, capi.I8I8I32, M, B1, k_tile=32)
+    opm1 = ops.W8A8Linear(sess, capi.I8I8I32, 1, B0, k_tile=32)
+    full = ops.W8A8Linear(sess, capi.I8I8I32, M, B0)  # k_tile = K
+    try:
+        ref0, ref1 = oracle.gemm_i8(A, B0), oracle.gemm_i8(A, B1)
+        out = np.empty((M, N), np.int32)
+        for w, ref in ((op0.w, ref0), (op1.w, ref1), (op0.w, ref0)):
+            assert lib.rk_npu_i8i8i32_run(op0.ws, w, capi.ptr(A), capi.ptr(out)) == 0
+            assert np.array_equal(out, ref)
+        out1 = np.empty((1, N), np.int32)
+        assert lib.rk_npu_i8i8i32_run(opm1.ws, op0.w, capi.ptr(A), capi.ptr(out1)) == 0
+        assert np.array_equal(out1[0], ref0[0])
+        # incompatible K partition
+        assert lib.rk_npu_i8i8i32_run(full.ws, op0.w, capi.ptr(A), capi.ptr(out)) == capi.RK_NPU_ERR_PARAM
+        # NULL arguments
+        assert lib.rk_npu_i8i8i32_run(op0.ws, op0.w, None, capi.ptr(out)) == capi.RK_NPU_ERR_PARAM
+        assert lib.rk_npu_i8i8i32_run(None, op0.w, capi.ptr(A), capi.ptr(out)) == capi.RK_NPU_ERR_PARAM
+        # wrong op kind for this workspace
+        assert lib.rk_npu_f16i8f16_run_dynamic(op0.ws, op0.w, capi.ptr(A), capi.ptr(out)) == capi.RK_NPU_ERR_PARAM
+        # foreign domain
+        other = lib.rk_npu_iommu_domain_create(sess.ctx, 14)
+        assert other and lib.rk_npu_iommu_domain_id(other) == 14
+        wc = capi.MatmulWeightConfig(K, N, 32)
+        import ctypes as C
+        foreign = lib.rk_npu_i8i8i32_weights_create(other, C.byref(wc), capi.ptr(B0))
+        assert foreign
+        assert lib.rk_npu_i8i8i32_run(op0.ws, foreign, capi.ptr(A), capi.ptr(out)) == capi.RK_NPU_ERR_DOMAIN
+        lib.rk_npu_i8i8i32_weights_free(foreign)
+        lib.rk_npu_iommu_domain_free(other)
+        # invalid scales -> NULL
+        ws = np.ones(N, np.float32)
+        ws[5] = 0
+        assert not lib.rk_npu_f16i8f16_weights_create(sess.domain, C.byref(wc), capi.ptr(B0), capi.ptr(ws))
+        ws[5] = np.nan
+        assert not lib.rk_npu_f16i8f16_weights_create(sess.domain, C.byref(wc), capi.ptr(B0), capi.ptr(ws))
+    finally:
+        for o in (op0, op1, opm1, full):
+            o.close()
+
+
+def test_busy_two_threads(sess):
+    """reference tests/test_quant_matmul.cpp:271-293: two threads hammer one
+    workspace; every call is either OK or BUSY and OK results are correct."""
+    import threading
+    M, N, K = 64, 512, 2048
+    rng = np.random.default_rng(3)
+    A = _rand_i8(rng, (M, K))
+    B = _rand_i8(rng, (K, N))
+    op = ops.W8A8Linear(sess, capi.I8I8I32, M, B)
+    want = A.astype(np.int32) @ B.astype(np.int32)
+    counts = {"ok": 0, "busy": 0, "bad": 0}
+    lock = threading.Lock()
+    go = threading.Event()
+
+    def hammer():
+        out = np.empty((M, N), np.int32)
+        go.wait()
+        for _ in range(64):
+            rc = sess.lib.rk_npu_i8i8i32_run(op.ws, op.w, capi.ptr(A), capi.ptr(out))
+            with lock:
+                if rc == 0:
+                    counts["ok" if np.array_equal(out, want) else "bad"] += 1
+                elif rc == capi.RK_NPU_ERR_BUSY:
+                    counts["busy"] += 1
+                else:
+                    counts["bad"] += 1
+
+    try:
+        ts = [threading.Thread(target=hammer) for _ in range(2)]
+        for t in ts:
+            t.start()
+        go.set()
+        for t in ts:
+            t.join()
+        assert counts["bad"] == 0 and counts["ok"] > 0
+    finally:
+        op.close()
