@@ -541,7 +541,9 @@ __device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i
                                               int col_phys_block, int lane, const float* a_scale,
                                               const float* w_scale, int m_limit) {
     const int n = block_first_col(col_phys_block, g.interleave_F) + (lane & 31);
-    if (n >= g.N) return;
+    // padding blocks beyond the matrix hold zeros; with interleaved columns
+    // their logical index would alias a real column, so test the block itself
+    if (n >= g.N || (g.interleave_F && col_phys_block >= g.N / 32)) return;
     const float ws = EPI == RKH_EPI_I32 ? 1.0f : w_scale[n];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {

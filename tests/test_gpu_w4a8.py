@@ -1,0 +1,330 @@
+"""GPU parity of the W4A8 linear, the fused SwiGLU and the FFN block.
+
+Integer intermediates (int8 activations, int32 accumulators, Down's int8
+re-quantized middle) and all fp32 / fp16 outputs are compared bit-exactly with
+the CPU oracle evaluated with the polynomial exponential (the flavour the
+reference's AArch64 production build runs); the libm flavour is checked within
+the reference's own 7e-7 relative bound.
+Cases follow the reference's tests/test_w4a8.cpp:21-40,71-162 (tails, zero
+row, +-127 extremes, large sums, NaN / -Inf rejection, invalid scale / code,
+foreign domain) and tests/test_w4a8_ffn.cpp:63-117.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from rknpu2_matmul_open_amd import capi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _codes(rng, shape, lo=-8, hi=7):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+def _bits32(x):
+    return np.ascontiguousarray(x, np.float32).view(np.uint32)
+
+
+SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), (9, 200, 96),
+          (40, 130, 257), (64, 256, 1024), (100, 320, 640), (130, 1000, 300)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_w4a8_f32_and_f16_bit_exact(sess, oracle, M, N, K):
+    rng = np.random.default_rng(M * 7919 + N * 31 + K)
+    B = _codes(rng, (K, N))
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.02
+    A = (rng.standard_normal((M, K)) * 2).astype(np.float32)
+    if M >= 3:
+        A[1, :] = 0.0                                   # zero row -> scale 1
+        A[2, : min(K, 8)] = [127, -127, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5][: min(K, 8)]
+        A[2, min(K, 8):] = 0.0                          # max 127 -> scale exactly 1, exact ties
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        want = oracle.w4a8(A, B, ws)
+        rc, acc = wsp.run_i32(w, A)
+        assert rc == 0
+        q, s = wsp.read_quantized()
+        assert np.array_equal(_bits32(s), _bits32(want["a_scale"]))
+        assert np.array_equal(q, want["q"])
+        assert np.array_equal(acc, want["acc"])
+        rc, got = wsp.run_f32(w, A)
+        assert rc == 0 and np.array_equal(_bits32(got), _bits32(want["C"]))
+        A16 = A.astype(np.float16).view(np.uint16)
+        want16 = oracle.w4a8(A16, B, ws)
+        rc, got16 = wsp.run_f16(w, A16)
+        assert rc == 0 and np.array_equal(got16, want16["C"])
+    finally:
+        wsp.close()
+        w.close()
+
+
+def test_w4a8_extremes_and_tiny_scale(sess, oracle):
+    M, N, K = 4, 64, 2048
+    B = np.full((K, N), -8, np.int8)
+    B[:, 1::2] = 7
+    ws = np.full(N, 0.001, np.float32)
+    A = np.zeros((M, K), np.float32)
+    A[0] = 127.0                      # q = 127 everywhere: |sum| = 127*8*2048 > 2^20
+    A[1] = -3.0
+    A[2, 0] = np.float32(1e-40)       # denormal maximum: scale floors at FLT_MIN
+    A[3, 5] = np.float32(2e-36)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        want = oracle.w4a8(A, B, ws)
+        rc, got = wsp.run_f32(w, A)
+        q, s = wsp.read_quantized()
+        assert rc == 0
+        assert np.array_equal(_bits32(s), _bits32(want["a_scale"]))
+        assert s[2] == np.finfo(np.float32).tiny
+        assert np.array_equal(q, want["q"])
+        assert np.array_equal(_bits32(got), _bits32(want["C"]))
+    finally:
+        wsp.close()
+        w.close()
+
+
+def test_w4a8_rejections(sess):
+    lib = sess.lib
+    M, N, K = 3, 65, 33
+    rng = np.random.default_rng(2)
+    B = _codes(rng, (K, N))
+    ws = np.full(N, 0.01, np.float32)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        sentinel = np.full((M, N), 123.0, np.float32)
+        for bad in (np.nan, -np.inf, np.inf):
+            Ab = A.copy()
+            Ab[1, 7] = bad
+            out = sentinel.copy()
+            t = capi.W4A8Timings()
+            rc = lib.rk_npu_w4a8_run_f32(wsp.h, w.h, capi.ptr(Ab), capi.ptr(out), C.byref(t))
+            assert rc == capi.RK_NPU_ERR_PARAM
+            assert (out == 123.0).all() and t.submit_us == 0
+        # the workspace still works afterwards
+        rc, _ = wsp.run_f32(w, A)
+        assert rc == 0
+        # A == C alias
+        buf = np.zeros((M, max(N, K)), np.float32)
+        assert lib.rk_npu_w4a8_run_f32(wsp.h, w.h, capi.ptr(buf), capi.ptr(buf), None) == capi.RK_NPU_ERR_PARAM
+        # invalid scale / code -> NULL
+        cfg = capi.I4WeightConfig(K, N, 480)
+        for v in (0.0, -1.0, np.nan, np.inf):
+            bs = ws.copy()
+            bs[3] = v
+            assert not lib.rk_npu_w4a8_weights_create(sess.domain, C.byref(cfg), capi.ptr(B), capi.ptr(bs))
+        for v in (8, -9):
+            Bb = B.copy()
+            Bb[5, 6] = v
+            assert not lib.rk_npu_w4a8_weights_create(sess.domain, C.byref(cfg), capi.ptr(Bb), capi.ptr(ws))
+        # k_tile mismatch -> PARAM, foreign domain -> DOMAIN
+        w2 = ops.W4A8Weights(sess, B, ws, k_tile=32)
+        rc, _ = wsp.run_f32(w2, A)
+        assert rc == capi.RK_NPU_ERR_PARAM
+        w2.close()
+        other = lib.rk_npu_iommu_domain_create(sess.ctx, 9)
+        foreign = lib.rk_npu_w4a8_weights_create(other, C.byref(cfg), capi.ptr(B), capi.ptr(ws))
+        assert foreign
+        out = np.empty((M, N), np.float32)
+        assert lib.rk_npu_w4a8_run_f32(wsp.h, foreign, capi.ptr(A), capi.ptr(out), None) == capi.RK_NPU_ERR_DOMAIN
+        lib.rk_npu_w4a8_weights_free(foreign)
+        lib.rk_npu_iommu_domain_free(other)
+        # SwiGLU needs N % 64 == 0
+        mid = np.empty((M, N // 2 + 1), np.float32)
+        assert lib.rk_npu_w4a8_run_swiglu_f32(wsp.h, w.h, capi.ptr(A), capi.ptr(mid), None) == capi.RK_NPU_ERR_PARAM
+    finally:
+        wsp.close()
+        w.close()
+
+
+SWIGLU_SHAPES = [(1, 64, 64), (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
+                 (128, 1024, 512)]
+
+
+@pytest.mark.parametrize("M,N,K", SWIGLU_SHAPES)
+def test_swiglu_bit_exact_poly_and_close_to_libm(sess, oracle, M, N, K):
+    rng = np.random.default_rng(N * 13 + K + M)
+    B = _codes(rng, (K, N), -7, 7)
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.01
+    A = (rng.standard_normal((M, K)) * 1.5).astype(np.float32)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        rc, mid = wsp.run_swiglu_f32(w, A)
+        assert rc == 0
+        poly = oracle.w4a8_swiglu(A, B, ws, oracle.EXP_POLY)
+        assert np.array_equal(_bits32(mid), _bits32(poly["middle"]))
+        libm = oracle.w4a8_swiglu(A, B, ws, oracle.EXP_LIBM)["middle"]
+        denom = np.maximum(np.abs(libm), 1e-30)
+        assert (np.abs(mid - libm) / denom).max() <= 7e-7 + 1e-12
+        # the plain run on the same (interleaved) weights must still be in logical column order
+        rc, full = wsp.run_f32(w, A)
+        assert rc == 0 and np.array_equal(_bits32(full), _bits32(oracle.w4a8(A, B, ws)["C"]))
+    finally:
+        wsp.close()
+        w.close()
+
+
+FFN_SHAPES = [(1, 64, 64, 64), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
+              (128, 384, 2048, 256)]
+
+
+@pytest.mark.parametrize("M,H,I,Nout", FFN_SHAPES)
+def test_ffn_bit_exact(sess, oracle, M, H, I, Nout):
+    rng = np.random.default_rng(M + H + I)
+    B_gu = _codes(rng, (H, 2 * I), -7, 7)
+    s_gu = (rng.random(2 * I).astype(np.float32) + 0.5) * 0.01
+    B_dn = _codes(rng, (I, Nout), -7, 7)
+    s_dn = (rng.random(Nout).astype(np.float32) + 0.5) * 0.01
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    if M > 2:
+        x[1] = 0.0  # zero token -> zero middle row -> Down scale 1
+    gw, dw = ops.W4A8Weights(sess, B_gu, s_gu), ops.W4A8Weights(sess, B_dn, s_dn)
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, Nout, I)
+    try:
+        t = capi.W4A8FfnTimings()
+        rc, mid, out = ops.w4a8_ffn(sess, gws, gw, dws, dw, x, t)
+        assert rc == 0
+        want = oracle.w4a8_ffn(x, B_gu, s_gu, B_dn, s_dn, oracle.EXP_POLY)
+        assert want["rc"] == 0
+        assert np.array_equal(_bits32(mid), _bits32(want["middle"]))
+        qd, sd = dws.read_quantized()
+        assert np.array_equal(_bits32(sd), _bits32(want["down_scale"]))
+        assert np.array_equal(qd, want["q_down"])
+        assert np.array_equal(_bits32(out), _bits32(want["C"]))
+        assert t.down.activation_scan_us == 0 and t.total_us > 0
+        # FFN == swiglu followed by run_f32 on the middle, bitwise
+        # (reference tests/test_w4a8_ffn.cpp:153-157)
+        rc, mid2 = gws.run_swiglu_f32(gw, x)
+        rc2, out2 = dws.run_f32(dw, mid2)
+        assert rc == 0 and rc2 == 0
+        assert np.array_equal(_bits32(mid2), _bits32(mid)) and np.array_equal(_bits32(out2), _bits32(out))
+        # end-to-end against the libm flavour within the benchmark tolerance
+        libm = oracle.w4a8_ffn(x, B_gu, s_gu, B_dn, s_dn, oracle.EXP_LIBM)["C"]
+        assert np.abs(out - libm).max() <= 1e-3 * max(np.abs(libm).max(), 1e-30)
+    finally:
+        for o in (gws, dws, gw, dw):
+            o.close()
+
+
+def test_ffn_argument_checks_and_nonfinite_middle(sess):
+    lib = sess.lib
+    M, H, I, Nout = 4, 64, 64, 64
+    rng = np.random.default_rng(1)
+    B_gu, B_dn = _codes(rng, (H, 2 * I)), _codes(rng, (I, Nout))
+    s_gu = np.full(2 * I, 0.01, np.float32)
+    s_dn = np.full(Nout, 0.01, np.float32)
+    gw, dw = ops.W4A8Weights(sess, B_gu, s_gu), ops.W4A8Weights(sess, B_dn, s_dn)
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, Nout, I)
+    dws_m = ops.W4A8Workspace(sess, M + 1, Nout, I)
+    try:
+        x = rng.standard_normal((M, H)).astype(np.float32)
+        mid = np.empty((M, I), np.float32)
+        out = np.empty((M, Nout), np.float32)
+        run = lib.rk_npu_w4a8_run_ffn_f32
+        P = capi.ptr
+        assert run(gws.h, gw.h, gws.h, dw.h, P(x), P(mid), P(out), None) == capi.RK_NPU_ERR_PARAM  # same ws
+        assert run(gws.h, gw.h, dws.h, dw.h, P(x), P(mid), P(mid), None) == capi.RK_NPU_ERR_PARAM  # middle == C
+        assert run(gws.h, gw.h, dws.h, dw.h, P(x), P(mid), P(x), None) == capi.RK_NPU_ERR_PARAM    # A == C
+        assert run(gws.h, gw.h, dws_m.h, dw.h, P(x), P(mid), P(out), None) == capi.RK_NPU_ERR_PARAM  # M differs
+        assert run(gws.h, dw.h, dws.h, dw.h, P(x), P(mid), P(out), None) == capi.RK_NPU_ERR_PARAM  # wrong weights
+        xb = x.copy()
+        xb[0, 0] = np.nan
+        assert run(gws.h, gw.h, dws.h, dw.h, P(xb), P(mid), P(out), None) == capi.RK_NPU_ERR_PARAM
+        assert run(gws.h, gw.h, dws.h, dw.h, P(x), P(mid), P(out), None) == 0
+        # huge gate/up scales overflow the middle to +-Inf: rejected before Down writes C
+        big = ops.W4A8Weights(sess, B_gu, np.full(2 * I, 1e30, np.float32))
+        out[:] = 7.0
+        assert run(gws.h, big.h, dws.h, dw.h, P(x * 1e6), P(mid), P(out), None) == capi.RK_NPU_ERR_PARAM
+        assert (out == 7.0).all()
+        big.close()
+    finally:
+        for o in (gws, dws, dws_m, gw, dw):
+            o.close()
+
+
+def test_weight_info_and_k_tile_resolution(sess):
+    """k_tile = 0 picks the largest partition whose INT16 bound certifies
+    (reference src/rk_npu_i4_bounds.cpp); explicit k_tile > 480 must certify."""
+    K, N = 2048, 64
+    small = np.ones((K, N), np.int8)            # P = 7*K, Q = 8*K: certified up to k with 8k <= 32768 -> 2048? 8*2048=16384 ok
+    w = ops.W4A8Weights(sess, small, np.ones(N, np.float32), k_tile=0)
+    assert w.info.config.k_tile == 2048 and w.info.safe_k_tile == 2048 and w.info.bound_relaxed == 0
+    assert w.info.multiplier == 1.0
+    w.close()
+    heavy = np.full((K, N), -8, np.int8)        # P = 64 per k: tile t certifies iff 64*t <= 32767 -> t <= 511 -> 480
+    w = ops.W4A8Weights(sess, heavy, np.ones(N, np.float32), k_tile=0)
+    assert w.info.config.k_tile == 480 and w.info.safe_k_tile == 480
+    w.close()
+    cfg = capi.I4WeightConfig(K, N, 512)
+    s = np.ones(N, np.float32)
+    assert not sess.lib.rk_npu_w4a8_weights_create(sess.domain, C.byref(cfg), capi.ptr(heavy), capi.ptr(s))
+    h = sess.lib.rk_npu_w4a8_weights_create(sess.domain, C.byref(cfg), capi.ptr(small), capi.ptr(s))
+    assert h
+    sess.lib.rk_npu_w4a8_weights_free(h)
+
+
+def test_config2_sampled_rows_and_properties(sess, oracle):
+    """BASELINE config 2 at full size (M=2048, K=4096, N=4096, seeds 4/5, 0.5% x20
+    outliers): every int8 activation exact, fp16 output exact on a band of rows the
+    oracle can afford, plus a size-independent property on the whole output:
+    scaling a token by a power of two scales its output row exactly (until fp16
+    range limits), because the quantized codes are unchanged."""
+    c = workloads.CONFIGS[2]()
+    M, K, N = c["M"], c["K"], c["N"]
+    w = ops.W4A8Weights(sess, c["B"], c["w_scale"])
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        rc, got = wsp.run_f16(w, c["A"])
+        assert rc == 0
+        q, s = wsp.read_quantized()
+        rcs, s_ref, inv_ref = oracle.w4a8_scales(c["A"])
+        assert rcs == 0 and np.array_equal(_bits32(s), _bits32(s_ref))
+        assert np.array_equal(q, oracle.w4a8_quant(c["A"], inv_ref))
+        rows = np.r_[0:48, 1000:1032, 2016:2048]
+        want = oracle.w4a8(np.ascontiguousarray(c["A"][rows]), c["B"], c["w_scale"])
+        assert np.array_equal(got[rows], want["C"])
+        # int32 accumulators for the same band through the probe entry point
+        small = ops.W4A8Workspace(sess, len(rows), N, K)
+        rc, acc = small.run_i32(w, oracle.half_to_float(c["A"][rows]))
+        small.close()
+        assert rc == 0 and np.array_equal(acc, want["acc"])
+        half = (oracle.half_to_float(c["A"]) * np.float32(0.5)).astype(np.float16).view(np.uint16)
+        rc, got_half = wsp.run_f16(w, half)
+        assert rc == 0
+        f, fh = oracle.half_to_float(got), oracle.half_to_float(got_half)
+        normal = np.abs(f) > 2.0 ** -13   # halves of fp16 normals stay exactly representable
+        assert np.array_equal(fh[normal] * 2, f[normal])
+    finally:
+        wsp.close()
+        w.close()
+
+
+def test_config3_ffn_full(sess, oracle):
+    """BASELINE config 3: M=128, hidden 4096, intermediate 14336, seeds 6-9."""
+    c = workloads.CONFIGS[3]()
+    M, H, I = c["M"], c["H"], c["I"]
+    gw, dw = ops.W4A8Weights(sess, c["B_gu"], c["s_gu"]), ops.W4A8Weights(sess, c["B_down"], c["s_down"])
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, H, I)
+    try:
+        rc, mid, out = ops.w4a8_ffn(sess, gws, gw, dws, dw, c["x"])
+        assert rc == 0
+        want = oracle.w4a8_ffn(c["x"], c["B_gu"], c["s_gu"], c["B_down"], c["s_down"], oracle.EXP_POLY)
+        assert np.array_equal(_bits32(mid), _bits32(want["middle"]))
+        qd, sd = dws.read_quantized()
+        assert np.array_equal(qd, want["q_down"]) and np.array_equal(_bits32(sd), _bits32(want["down_scale"]))
+        assert np.array_equal(_bits32(out), _bits32(want["C"]))
+        rc, acc = dws.run_i32(dw, mid)
+        assert rc == 0 and np.array_equal(acc, want["acc_down"])
+        out16 = oracle.float_to_half(out)
+        ref16 = oracle.half_to_float(oracle.float_to_half(want["C"]))
+        assert np.abs(oracle.half_to_float(out16) - ref16).max() <= 1e-3 * np.abs(ref16).max()
+    finally:
+        for o in (gws, dws, gw, dw):
+            o.close()
