@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1]
+
+A step is one pass of the hot path over one batch of seeded synthetic input,
+with inputs and weights already resident in HBM: per-token quantization +
+GEMV / GEMM with the fused dequant epilogue (+ SwiGLU / re-quantize / Down for
+the FFN, + route / combine for the MoE layer), enqueued through the
+device-pointer entry points of the C ABI and timed with HIP events on the
+context's stream.  The default workload is BASELINE config 1 (w8a8 decode GEMV,
+M=1, K=4096, N=14336), reported as weight GB/s; the line also carries the
+int8 TOPS of config 2 (w4a8 prefill GEMM, M=2048) because the headline metric
+names both.
+
+Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate
+METRIC = "int8 TOPS @M=2048 and GEMV HBM GB/s @M=1 (w8a8/w4a8), % of roofline"
+
+
+def log(msg):
+    sys.stderr.write("[bench] %s\n" % msg)
+    sys.stderr.flush()
+
+
+def _traffic(kernel_key):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE,
+    scaled by a copy kernel of known size), if a summary has been committed."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel_key)
+    except (OSError, ValueError):
+        return None
+
+
+def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
+    """w8a8 decode GEMV, M=1, K=4096, N=14336."""
+    c = workloads.CONFIGS[1]()
+    M, K, N = c["M"], c["K"], c["N"]
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    dA = sess.to_device(c["A"])
+    dC = sess.empty_device(M * N * 2)
+    lib = sess.lib
+
+    def step():
+        rc = op.run_device(dA, dC)
+        if rc:
+            raise RuntimeError("run_device rc=%d" % rc)
+
+    def gemv_only():
+        rc = lib.rk_npu_matmul_workspace_rerun_gemm_device(op.ws, op.w, dC)
+        if rc:
+            raise RuntimeError("rerun rc=%d" % rc)
+
+    step_us = sess.time_us(step, steps, warmup)
+    kernel_us = sess.time_us(gemv_only, max(steps, 50), warmup)
+    got = sess.from_device(dC, (M, N), np.uint16)
+    weight_bytes = K * N
+    # algorithmic bytes of one GEMV launch: weights once + int8 A + fp16 C + scales
+    algo_bytes = weight_bytes + K + N * 2 + N * 4 + 4
+    out = {
+        "value": weight_bytes / step_us / 1e3,  # GB/s (bytes / us / 1e3)
+        "unit": "GB/s",
+        "ms_per_step": step_us / 1e3,
+        "dtype": "int8",
+        "config": {"workload": "c1: w8a8 decode GEMV M=1 K=4096 N=14336, fp16 in/out, seeds 2/3",
+                   "value_is": "int8 weight bytes (58720256) / step time; step = quantize + GEMV kernels"},
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,false>",
+                     "achieved": algo_bytes / kernel_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": algo_bytes / kernel_us / 1e3 / HBM_PEAK_GBS,
+                     "kernel_us": kernel_us, "algorithmic_bytes": algo_bytes,
+                     "traffic": _traffic("gemv_c1")},
+    }
+    if cpu_baseline:
+        from oracle import binding as orc
+        want = orc.w8a8(c["A"], c["B"], c["w_scale"])
+        out["parity"] = bool(np.array_equal(got, want["C"]))
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 10.0:
+            orc.w8a8(c["A"], c["B"], c["w_scale"])
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        out["cpu_baseline"] = {"value": weight_bytes / dt / 1e9, "unit": "GB/s",
+                               "cores": orc.num_threads(), "kind": "port",
+                               "sample": "%d full passes of config 1 (quantize + exact int GEMV + dequant), %.1f ms each"
+                                         % (reps, dt * 1e3)}
+    sess.free_device(dA)
+    sess.free_device(dC)
+    op.close()
+    return out
+
+
+def bench_c2(sess, ops, capi, workloads, steps, warmup):
+    """w4a8 prefill GEMM, M=2048, K=4096, N=4096."""
+    c = workloads.CONFIGS[2]()
+    M, K, N = c["M"], c["K"], c["N"]
+    w = ops.W4A8Weights(sess, c["B"], c["w_scale"])
+    ws = ops.W4A8Workspace(sess, M, N, K)
+    dA = sess.to_device(c["A"])
+    dC = sess.empty_device(M * N * 2)
+    lib = sess.lib
+
+    def step():
+        rc = lib.rk_npu_w4a8_run_f16_device(ws.h, w.h, dA, dC)
+        if rc:
+            raise RuntimeError("run_device rc=%d" % rc)
+
+    def gemm_only():
+        rc = lib.rk_npu_w4a8_workspace_rerun_gemm_device(ws.h, w.h, dC, 1)
+        if rc:
+            raise RuntimeError("rerun rc=%d" % rc)
+
+    step_us = sess.time_us(step, steps, warmup)
+    kernel_us = sess.time_us(gemm_only, steps, warmup)
+    ops_count = 2.0 * M * K * N
+    out = {"workload": "c2: w4a8 prefill GEMM M=2048 K=4096 N=4096, fp16 in/out, seeds 4/5",
+           "tops": ops_count / step_us / 1e6, "ms_per_step": step_us / 1e3,
+           "roofline": {"bound": "mfma", "kernel": "gemm_kernel<2,2,2,4,int4>",
+                        "achieved": ops_count / kernel_us / 1e6, "peak": INT8_PEAK_TOPS,
+                        "unit": "TOP/s", "frac": ops_count / kernel_us / 1e6 / INT8_PEAK_TOPS,
+                        "kernel_us": kernel_us, "traffic": _traffic("gemm_c2")}}
+    sess.free_device(dA)
+    sess.free_device(dC)
+    ws.close()
+    w.close()
+    return out
+
+
+def bench_c3(sess, ops, capi, workloads, steps, warmup):
+    """fused w4a8 FFN block, M=128, hidden 4096, intermediate 14336."""
+    c = workloads.CONFIGS[3]()
+    M, H, I = c["M"], c["H"], c["I"]
+    gw, dw = ops.W4A8Weights(sess, c["B_gu"], c["s_gu"]), ops.W4A8Weights(sess, c["B_down"], c["s_down"])
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, H, I)
+    dA = sess.to_device(c["x"])
+    dmid = sess.empty_device(M * I * 4)
+    dC = sess.empty_device(M * H * 4)
+
+    def step():
+        rc = sess.lib.rk_npu_w4a8_run_ffn_f32_device(gws.h, gw.h, dws.h, dw.h, dA, dmid, dC)
+        if rc:
+            raise RuntimeError("ffn rc=%d" % rc)
+
+    step_us = sess.time_us(step, steps, warmup)
+    ops_count = 2.0 * M * H * 2 * I + 2.0 * M * I * H
+    weight_bytes = (H * 2 * I + I * H) / 2
+    out = {"workload": "c3: fused w4a8 FFN M=128 H=4096 I=14336, seeds 6-9",
+           "tops": ops_count / step_us / 1e6, "weight_GBps": weight_bytes / step_us / 1e3,
+           "ms_per_step": step_us / 1e3}
+    for d in (dA, dmid, dC):
+        sess.free_device(d)
+    for o in (gws, dws, gw, dw):
+        o.close()
+    return out
+
+
+def bench_c4(sess, ops, capi, workloads, steps, warmup):
+    """w8a8 MoE layer, 256 tokens, hidden 2048, 32 experts, top-4, intermediate 1024."""
+    c = workloads.CONFIGS[4]()
+    moe = ops.MoeW8(sess, c["H"], c["I"], c["E"], 0, c["top_k"], 256, c["experts"])
+    dx, dids, drt = sess.to_device(c["x"]), sess.to_device(c["ids"]), sess.to_device(c["routes"])
+    dout = sess.empty_device(c["T"] * c["H"] * 4)
+
+    def step():
+        rc = sess.lib.rk_npu_moe_w8_run_f32_device(moe.ws, moe.w, c["T"], dx, dids, drt, dout)
+        if rc:
+            raise RuntimeError("moe rc=%d" % rc)
+
+    step_us = sess.time_us(step, steps, warmup)
+    assignments = int((c["routes"] != 0).sum())
+    ops_count = assignments * (2.0 * c["H"] * 2 * c["I"] + 2.0 * c["I"] * c["H"])
+    weight_bytes = c["E"] * 3 * c["H"] * c["I"]
+    out = {"workload": "c4: w8a8 MoE T=256 H=2048 E=32 top-4 I=1024, seeds 10-14",
+           "tops": ops_count / step_us / 1e6, "weight_GBps": weight_bytes / step_us / 1e3,
+           "ms_per_step": step_us / 1e3}
+    for d in (dx, dids, drt, dout):
+        sess.free_device(d)
+    moe.close()
+    return out
+
+
+def bench_c0(sess, ops, capi, workloads, steps, warmup):
+    c = workloads.CONFIGS[0]()
+    M, K, N = c["M"], c["K"], c["N"]
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    dA = sess.to_device(c["A"])
+    dC = sess.empty_device(M * N * 2)
+    step_us = sess.time_us(lambda: op.run_device(dA, dC), steps, warmup)
+    out = {"workload": "c0: w8a8 GEMM M=64 K=2048 N=2048", "tops": 2.0 * M * K * N / step_us / 1e6,
+           "weight_GBps": K * N / step_us / 1e3, "ms_per_step": step_us / 1e3}
+    sess.free_device(dA)
+    sess.free_device(dC)
+    op.close()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c1", choices=["c1", "all"],
+                    help="c1: headline line (+ c2 TOPS); all: also time configs 0, 3 and 4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c3", "c4"],
+                    help="profiling aid: run one configuration's loop only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this path runs on one GPU; --gpus %d is not supported "
+                         "(every box of this build has one GPU, no collectives exist)\n" % args.gpus)
+        sys.exit(2)
+
+    from rknpu2_matmul_open_amd import capi, ops, workloads
+    sess = ops.Session()
+    arch, cus, khz = sess.device_info()
+    log("device %s, %d CUs, %d MHz" % (arch, cus, khz // 1000))
+
+    if args.only:
+        fn = {"c0": bench_c0, "c2": bench_c2, "c3": bench_c3, "c4": bench_c4}.get(args.only)
+        res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)
+               if args.only == "c1" else fn(sess, ops, capi, workloads, args.steps, args.warmup))
+        print(json.dumps(res))
+        sess.close()
+        return
+
+    log("config 1 (decode GEMV)")
+    r1 = bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, not args.no_cpu_baseline)
+    log("config 2 (prefill GEMM)")
+    r2 = bench_c2(sess, ops, capi, workloads, max(args.steps // 4, 20), args.warmup)
+    also = {"c2": r2}
+    if args.workload == "all":
+        for name, fn in (("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
+            log("config %s" % name)
+            also[name] = fn(sess, ops, capi, workloads, max(args.steps // 4, 20), args.warmup)
+    line = {
+        "metric": METRIC, "value": r1["value"], "unit": r1["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": r1["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": r1["dtype"],
+        "data": "synthetic (seeded numpy PCG64; weights N(0,0.02) quantized per channel, activations fp16 N(0,1))",
+        "config": r1["config"], "roofline": r1["roofline"],
+        "device": {"arch": arch, "compute_units": cus, "clock_mhz": khz // 1000},
+        "also": also,
+    }
+    if "cpu_baseline" in r1:
+        line["cpu_baseline"] = r1["cpu_baseline"]
+        line["parity_vs_oracle"] = r1["parity"]
+    print(json.dumps(line))
+    sess.close()
+
+
+if __name__ == "__main__":
+    main()

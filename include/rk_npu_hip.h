@@ -80,6 +80,18 @@ int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* workspace,
                                  const float* input_device, const int32_t* expert_ids_device,
                                  const float* route_weights_device, float* output_device);
 
+/* Profiling hooks: launch only the GEMV / GEMM stage of an operator on the
+ * activations its workspace quantized during the previous run, so that the
+ * dominant kernel can be timed by itself with stream events.  `weights` is a
+ * rk_npu_{i8i8i32,f16i8f16,f32i8f32}_weights handle matching the workspace's
+ * op kind; the output element type is the workspace's (W8A8) or fp16 / fp32
+ * as selected by `half` (W4A8). */
+int rk_npu_matmul_workspace_rerun_gemm_device(rk_npu_matmul_workspace* workspace,
+                                              const void* weights, void* C_device);
+int rk_npu_w4a8_workspace_rerun_gemm_device(rk_npu_w4a8_workspace* workspace,
+                                            const rk_npu_w4a8_weights* weights, void* C_device,
+                                            int half);
+
 /* Parity probes: the exact intermediates of the most recent run on a
  * workspace, copied to host.  q is the int8 activation matrix [M, K] in
  * row-major order, a_scale the per-row scales [M].  Blocking. */

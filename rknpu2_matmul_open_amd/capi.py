@@ -215,6 +215,8 @@ _PROTOTYPES = {
     "rk_npu_w4a8_run_f32_device": (C.c_int, [P, P, P, P]),
     "rk_npu_w4a8_run_ffn_f32_device": (C.c_int, [P, P, P, P, P, P, P]),
     "rk_npu_moe_w8_run_f32_device": (C.c_int, [P, P, C.c_int, P, P, P, P]),
+    "rk_npu_matmul_workspace_rerun_gemm_device": (C.c_int, [P, P, P]),
+    "rk_npu_w4a8_workspace_rerun_gemm_device": (C.c_int, [P, P, P, C.c_int]),
     "rk_npu_matmul_workspace_read_quantized": (C.c_int, [P, P, P]),
     "rk_npu_w4a8_workspace_read_quantized": (C.c_int, [P, P, P]),
     "rk_npu_w4a8_run_i32": (C.c_int, [P, P, P, P]),

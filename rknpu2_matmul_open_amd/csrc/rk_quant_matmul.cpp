@@ -126,6 +126,8 @@ namespace {
 
 // Enqueue quantize + GEMM on the context's stream.  dA / dC are device
 // pointers (the workspace's own staging buffers or the caller's).
+int enqueue_gemm(rk_npu_matmul_workspace* ws, const Weights& w, void* dC);
+
 int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA,
             const float* a_scale_static_dev, void* dC) {
     const auto& s = ws->strategy;
@@ -136,10 +138,19 @@ int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA,
     q.mode = ws->t.quant == 0 ? RKH_Q_COPY_I8 : ws->t.quant == 1 ? RKH_Q_W8_DYNAMIC : RKH_Q_W8_STATIC;
     q.M = s.M;
     q.K = s.K;
-    q.scale = ws->t.quant == 2 ? const_cast<float*>(a_scale_static_dev) : ws->a_scale.as<float>();
+    (void)a_scale_static_dev; // static scales are staged in the workspace's a_scale
+    q.scale = ws->t.quant == 0 ? nullptr : ws->a_scale.as<float>();
     q.dst = ws->a_tiled.as<>();
     int rc = rkh_quant_rows(stream, &q);
     if (rc) return map_error(rc);
+    return enqueue_gemm(ws, w, dC);
+}
+
+// GEMV / GEMM stage on the activations already quantized into the workspace.
+int enqueue_gemm(rk_npu_matmul_workspace* ws, const Weights& w, void* dC) {
+    const auto& s = ws->strategy;
+    void* stream = ws->owner.ctx->stream;
+    struct { float* scale; } q{ws->a_scale.as<float>()};
     rkh_gemm_args g{};
     g.A = ws->a_tiled.as<>();
     g.W = w.tiled.as<>();
@@ -394,6 +405,20 @@ int rk_npu_f32i8f32_run_dynamic_device(rk_npu_matmul_workspace* ws,
                                        float* C) {
     return run_device(ws, reinterpret_cast<const Weights*>(weights), RK_NPU_MATMUL_F32I8F32_DYNAMIC,
                       A, C);
+}
+
+// Profiling hook: only the GEMV / GEMM stage, on the activations the previous
+// run left in the workspace.
+int rk_npu_matmul_workspace_rerun_gemm_device(rk_npu_matmul_workspace* ws, const void* weights,
+                                              void* C) {
+    const Weights* w = static_cast<const Weights*>(weights);
+    if (!ws || !w) return RK_NPU_ERR_PARAM;
+    int rc = check_run(ws, w, ws->strategy.op_kind, C, C);
+    if (rc) return rc;
+    BusyLock lock(ws->busy);
+    if (!lock) return RK_NPU_ERR_BUSY;
+    std::lock_guard<std::mutex> submit(ws->owner.ctx->submit_mutex);
+    return enqueue_gemm(ws, *w, C);
 }
 
 // Parity probe: de-tile the int8 activations of the last run.

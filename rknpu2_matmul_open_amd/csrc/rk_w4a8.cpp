@@ -189,6 +189,8 @@ int validate(const rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, cons
 }
 
 enum class Out { F32, F16, I32, SwiGLU };
+int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
+                 bool collect);
 
 // quantize (or re-quantize with reused row maxima) + GEMM.  `scale_source`
 // non-null: A is the fp32 middle of that workspace's SwiGLU run and its
@@ -216,6 +218,16 @@ int enqueue(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void*
     int rc = rkh_quant_rows(stream, &q);
     if (rc) return map_error(rc);
     if (timer) timer->mark();
+    rc = enqueue_gemm(ws, w, dC, out, collect);
+    if (timer) timer->mark();
+    return rc;
+}
+
+// GEMV / GEMM stage on the activations already quantized into the workspace.
+int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
+                 bool collect) {
+    const auto& c = ws->config;
+    void* stream = ws->owner.ctx->stream;
     rkh_gemm_args g{};
     g.A = ws->a_tiled.as<>();
     g.W = w->tiled.as<>();
@@ -238,9 +250,7 @@ int enqueue(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void*
         g.row_max_bits = collect ? ws->row_max.as<uint32_t>() : nullptr;
         break;
     }
-    rc = rkh_gemm(stream, &g);
-    if (timer) timer->mark();
-    return map_error(rc);
+    return map_error(rkh_gemm(stream, &g));
 }
 
 void fill_timings(rk_npu_w4a8_timings* t, StageTimer& timer, int first_mark, bool scanned,
@@ -578,6 +588,18 @@ int rk_npu_w4a8_run_ffn_f32_device(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_
     rc = enqueue(gu, guw, A, false, middle, Out::SwiGLU, true, nullptr, nullptr);
     if (!rc) rc = enqueue(dn, dnw, middle, false, C, Out::F32, false, gu, nullptr);
     return rc;
+}
+
+// Profiling hook: only the GEMV / GEMM stage (fp16 or fp32 output), on the
+// activations the previous run left in the workspace.
+int rk_npu_w4a8_workspace_rerun_gemm_device(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w,
+                                            void* C, int half) {
+    int rc = validate(ws, w, C, ws, false);
+    if (rc) return rc;
+    BusyLock lock(ws->busy);
+    if (!lock) return RK_NPU_ERR_BUSY;
+    std::lock_guard<std::mutex> submit(ws->owner.ctx->submit_mutex);
+    return enqueue_gemm(ws, w, C, half ? Out::F16 : Out::F32, false);
 }
 
 int rk_npu_w4a8_workspace_read_quantized(rk_npu_w4a8_workspace* ws, int8_t* q, float* a_scale) {
