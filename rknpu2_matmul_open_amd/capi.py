@@ -228,7 +228,9 @@ _LIB = None
 
 
 def lib_path():
-    return os.path.join(HERE, "librk_npu_matmul.so")
+    """In-tree library, or the file named by RK_NPU_MATMUL_LIB (to try out a
+    differently built copy without touching the tree)."""
+    return os.environ.get("RK_NPU_MATMUL_LIB") or os.path.join(HERE, "librk_npu_matmul.so")
 
 
 def load_library():

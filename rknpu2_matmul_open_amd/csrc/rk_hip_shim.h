@@ -119,8 +119,8 @@ typedef struct rkh_quant_args {
     float* scale;        /* [M] out (in for STATIC)                                */
     uint8_t* dst;        /* tiled int8, Kp = align64(K)                            */
     int* bad_flag;       /* OR 1: non-finite input (modes with a check), may be NULL */
-    const uint32_t* row_max_bits; /* REUSE modes: max |x| bit pattern per row      */
-    uint32_t* zero_bits; /* if non-NULL, zero_bits[m] = 0 is written for each row  */
+    const uint32_t* row_max_bits; /* REUSE modes: [M][row_max_parts] partial maxima of |x| bits */
+    int row_max_parts;
     /* MoE scatter: when dest_rows != NULL, source row m is written to every
      * tiled row dest_rows[m * dest_stride + j] >= 0, j < dest_stride, and
      * scale_rows[dest row] receives the row's scale. */
@@ -137,7 +137,7 @@ enum rkh_epilogue {
     RKH_EPI_I32 = 0,    /* C int32 = acc                                           */
     RKH_EPI_F16 = 1,    /* C fp16  = rne16((float(acc) * as[m]) * ws[n])           */
     RKH_EPI_F32 = 2,    /* C fp32  = (float(acc) * as[m]) * ws[n]                  */
-    RKH_EPI_SWIGLU = 3  /* C fp32 [M, F] = silu(g) * u, row_max_bits atomicMax     */
+    RKH_EPI_SWIGLU = 3  /* C fp32 [M, F] = silu(g) * u, partial row maxima written  */
 };
 
 typedef struct rkh_gemm_args {
@@ -151,7 +151,7 @@ typedef struct rkh_gemm_args {
     int epilogue;         /* rkh_epilogue                                          */
     void* C;              /* [M, ldc]                                              */
     int ldc;
-    uint32_t* row_max_bits; /* SwiGLU: per-row max |middle| bits (pre-zeroed)      */
+    uint32_t* row_max_bits; /* SwiGLU: [rows][F/32] max |middle| bits per 32 columns */
     int32_t* splitk_acc;  /* scratch [align(M,128) * align(N,256)] int32 for split-K, or NULL */
     /* Grouped (MoE) mode when blk_expert != NULL: row-block b (32 rows of the
      * sorted activation buffer) uses expert blk_expert[b]; blocks at or beyond

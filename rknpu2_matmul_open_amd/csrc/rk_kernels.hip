@@ -12,6 +12,7 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <float.h>
+#include <type_traits>
 
 #include "rk_hip_shim.h"
 
@@ -206,7 +207,6 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
                 const int d = a.dest_rows[(size_t)m * nd + j];
                 if (d >= 0) {
                     if (a.scale_rows && a.scale) a.scale_rows[d] = a.scale[m];
-                    if (a.zero_bits) a.zero_bits[d] = 0u;
                 }
             }
         }
@@ -283,7 +283,17 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     } else if (mode == RKH_Q_W8_STATIC || (mode == RKH_Q_COPY_I8 && a.scale)) {
         scale = a.scale[m];
     } else if (mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) {
-        const uint32_t bits = a.row_max_bits[m];
+        // row maximum = max over the per-32-column partial maxima the SwiGLU
+        // epilogue left behind (unsigned compare of |x| bit patterns)
+        uint32_t bits = 0;
+        for (int i = t; i < a.row_max_parts; i += 256)
+            bits = max(bits, a.row_max_bits[(size_t)m * a.row_max_parts + i]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+        if (lane_id() == 0) wave_bad[wave_id()] = (int)bits;
+        __syncthreads();
+        bits = max(max((uint32_t)wave_bad[0], (uint32_t)wave_bad[1]),
+                   max((uint32_t)wave_bad[2], (uint32_t)wave_bad[3]));
         const float mxv = __uint_as_float(bits);
         if (mode == RKH_Q_REUSE_BITS) {
             if (bits >= 0x7f800000u) {
@@ -304,14 +314,12 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     if (t == 0) {
         if (!a.dest_rows) {
             if (a.scale && mode != RKH_Q_W8_STATIC && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
-            if (a.zero_bits) a.zero_bits[m] = 0u;
         } else {
             if (a.scale && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
             for (int j = 0; j < ndest; ++j) {
                 const int d = a.dest_rows[(size_t)m * ndest + j];
                 if (d >= 0) {
                     a.scale_rows[d] = scale;
-                    if (a.zero_bits) a.zero_bits[d] = 0u;
                 }
             }
         }
@@ -526,8 +534,6 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) 
 // -> LDS as whole 1 KiB tiles, so LDS reads are linear 16 bytes per lane
 // (bank-conflict free) and land directly in MFMA operand order.  Two LDS
 // buffers; the loads of step i+1 are issued before the MFMAs of step i.
-struct TileCoord { int mblk, nblk, kpart; };
-
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
     // contiguous range of logical tiles so neighbours share its L2.
@@ -536,73 +542,170 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
     return xcd * q + min(xcd, r) + idx;
 }
 
-template <int EPI>
-__device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i& acc, int row0,
-                                              int col_phys_block, int lane, const float* a_scale,
-                                              const float* w_scale, int m_limit) {
-    const int n = block_first_col(col_phys_block, g.interleave_F) + (lane & 31);
-    // padding blocks beyond the matrix hold zeros; with interleaved columns
-    // their logical index would alias a real column, so test the block itself
-    if (n >= g.N || (g.interleave_F && col_phys_block >= g.N / 32)) return;
-    const float ws = EPI == RKH_EPI_I32 ? 1.0f : w_scale[n];
+// LDS-only workgroup barrier: waits for this wave's LDS traffic and joins the
+// barrier, but leaves global loads in flight (the K loop keeps prefetches
+// outstanding across it).  The "memory" clobber stops the compiler from moving
+// LDS accesses across it.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// ---- accumulator tile layout ------------------------------------------------
+// The weights are the FIRST MFMA operand and the activations the second, so a
+// 32x32 accumulator tile holds D[n_local][m_local]: lane l owns activation row
+// m_local = l % 32 and the 16 weight columns
+//     n_local(r) = 8 * (r / 4) + 4 * (l / 32) + (r % 4),  r = 0..15,
+// i.e. four runs of four consecutive output columns of ONE output row.  That
+// makes the per-row quantities (a_scale, SwiGLU row maximum) lane-local and the
+// stores row-contiguous.
+__device__ __forceinline__ int tile_col(int r, int lane) {
+    return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+
+// Write one finished 32x32 tile of output elements to C[m0.., n0..] through a
+// wave-private LDS staging area so that global stores are 16 bytes per lane and
+// row-contiguous.  vals[r] is the element for (m0 + lane%32, n0 + tile_col(r)).
+template <typename T>
+__device__ __forceinline__ void store_tile(T* C, int ldc, int m0, int n0, int m_limit, int n_limit,
+                                           const T* vals, uint8_t* stage_lds, int lane) {
+    constexpr int ES = sizeof(T);
+    constexpr int ROW = 32 * ES + 8;            // padded row pitch: conflict-free for b64 / b128
+    constexpr int CHUNKS_PER_ROW = 32 * ES / 16; // 16-byte pieces per row
+    const bool aligned = ((reinterpret_cast<uintptr_t>(C) | ((size_t)ldc * ES) | ((size_t)n0 * ES)) & 15) == 0;
+    if (aligned && n0 + 32 <= n_limit) {
+        const int ml = lane & 31;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        for (int gq = 0; gq < 4; ++gq) {
+            const int col = 8 * gq + 4 * (lane >> 5);
+            T* dst = reinterpret_cast<T*>(stage_lds + ml * ROW + col * ES);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[q] = vals[gq * 4 + q];
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int t = 0; t < CHUNKS_PER_ROW * 32 / 64; ++t) {
+            const int c = lane + 64 * t;
+            const int row = c / CHUNKS_PER_ROW, part = c % CHUNKS_PER_ROW;
+            // rows are 8 bytes past a 16-byte boundary apart, so read as two 8-byte halves
+            const uint2 lo = *reinterpret_cast<const uint2*>(stage_lds + row * ROW + part * 16);
+            const uint2 hi = *reinterpret_cast<const uint2*>(stage_lds + row * ROW + part * 16 + 8);
+            if (m0 + row < m_limit)
+                *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(C) +
+                                          ((size_t)(m0 + row) * ldc + n0) * ES + part * 16) =
+                    make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        const int m = m0 + (lane & 31);
         if (m < m_limit) {
-            const float as = EPI == RKH_EPI_I32 ? 1.0f : a_scale[m];
-            store_out(g.C, EPI, (size_t)m * g.ldc + n, acc[r], as, ws);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int n = n0 + tile_col(r, lane);
+                if (n < n_limit) C[(size_t)m * ldc + n] = vals[r];
+            }
         }
     }
 }
 
-// gate tile / up tile pair -> middle and per-row max bits
+// Dequantize and store one accumulator tile whose physical column block is p.
+template <int EPI>
+__device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i& acc, int m0, int p,
+                                              int lane, const float* a_scale, const float* w_scale,
+                                              int m_limit, uint8_t* stage_lds) {
+    // padding blocks beyond the matrix hold zeros; with interleaved columns their
+    // logical index would alias a real column, so test the block itself
+    if (g.interleave_F ? p >= g.N / 32 : p * 32 >= g.N) return;
+    const int n0 = block_first_col(p, g.interleave_F);
+    const int m = m0 + (lane & 31);
+    if constexpr (EPI == RKH_EPI_I32) {
+        int vals[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) vals[r] = acc[r];
+        store_tile<int>(static_cast<int*>(g.C), g.ldc, m0, n0, m_limit, g.N, vals, stage_lds, lane);
+    } else {
+        const float as = m < m_limit ? a_scale[m] : 0.0f;
+        float y[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = n0 + tile_col(r, lane);
+            y[r] = dequant(acc[r], as, n < g.N ? w_scale[n] : 0.0f);
+        }
+        if constexpr (EPI == RKH_EPI_F16) {
+            __half h[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) h[r] = __float2half_rn(y[r]);
+            store_tile<__half>(static_cast<__half*>(g.C), g.ldc, m0, n0, m_limit, g.N, h, stage_lds, lane);
+        } else {
+            store_tile<float>(static_cast<float*>(g.C), g.ldc, m0, n0, m_limit, g.N, y, stage_lds, lane);
+        }
+    }
+}
+
+// gate tile (physical block p, even) + up tile (p + 1) -> 32 columns of the
+// middle and one partial row maximum per (row, 32-column block).
 __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v16i& gate,
-                                                const v16i& up, int row0, int gate_phys_block,
-                                                int lane, const float* a_scale,
-                                                const float* w_scale, int m_limit) {
+                                                const v16i& up, int m0, int p, int lane,
+                                                const float* a_scale, const float* w_scale,
+                                                int m_limit, uint8_t* stage_lds) {
     const int F = g.interleave_F;
-    const int n = (gate_phys_block >> 1) * 32 + (lane & 31);
-    const bool col_ok = n < F;
-    const float wg = col_ok ? w_scale[n] : 0.0f;
-    const float wu = col_ok ? w_scale[F + n] : 0.0f;
+    const int n0 = (p >> 1) * 32;
+    if (n0 >= F) return;
+    const int m = m0 + (lane & 31);
+    const float as = m < m_limit ? a_scale[m] : 0.0f;
+    float y[16];
+    uint32_t bits = 0;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        uint32_t bits = 0;
-        if (m < m_limit && col_ok) {
-            const float as = a_scale[m];
-            const float gf = dequant(gate[r], as, wg);
-            const float uf = dequant(up[r], as, wu);
-            const float y = __fmul_rn(silu_poly(gf), uf);
-            static_cast<float*>(g.C)[(size_t)m * g.ldc + n] = y;
-            bits = __float_as_uint(y) & 0x7fffffffu;
-        }
-        if (g.row_max_bits) {
-            // max over the 32 lanes that share this row
-#pragma unroll
-            for (int off = 16; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
-            if ((lane & 31) == 0 && m < m_limit && bits) atomicMax(g.row_max_bits + m, bits);
-        }
+        const int n = n0 + tile_col(r, lane);
+        const float gf = dequant(gate[r], as, w_scale[n]);
+        const float uf = dequant(up[r], as, w_scale[F + n]);
+        y[r] = __fmul_rn(silu_poly(gf), uf);
+        bits = max(bits, __float_as_uint(y[r]) & 0x7fffffffu);
+    }
+    store_tile<float>(static_cast<float*>(g.C), g.ldc, m0, n0, m_limit, F, y, stage_lds, lane);
+    if (g.row_max_bits) {
+        bits = max(bits, (uint32_t)__shfl_xor((int)bits, 32));
+        if (lane < 32 && m < m_limit) g.row_max_bits[(size_t)m * (F / 32) + (p >> 1)] = bits;
     }
 }
 
-template <int WM, int WN, int TM, int TN, bool W4, int EPI, bool GROUPED>
+// Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn), each
+// wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is KT 32-deep
+// k-tiles.  Tiles travel global -> registers -> LDS as whole 1 KiB tiles, so LDS
+// reads are linear 16 bytes per lane (bank-conflict free) and land directly in
+// MFMA operand order.
+//
+// Software pipeline (one wave per SIMD, so latency is hidden by ILP only):
+//  - global loads run two K steps ahead in two register stages;
+//  - LDS fragment reads run one k-tile ahead of the MFMAs that use them, the
+//    int4 -> int8 unpack of the next k-tile is interleaved between the MFMAs of
+//    the current one (fragment and operand registers are double buffered);
+//  - the LDS writes of the next step are issued at the start of the step and
+//    the workgroup barrier sits before the LAST k-tile, so the first fragments
+//    of the next step are fetched under that k-tile's MFMAs.
+template <int WM, int WN, int TM, int TN, int KT, bool W4, int EPI, bool GROUPED>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int mblocks,
                                                             int nblocks, int ksplit,
                                                             int ksteps_per_part) {
+    static_assert(KT == 2, "the pipeline below is written for two k-tiles per step");
     constexpr int NW = WM * WN;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int A_CH = BM / 32 * 2;                 // 1 KiB chunks per K step
-    constexpr int B_CH = W4 ? BN / 32 : BN / 32 * 2;
+    constexpr int A_CH = BM / 32 * KT;                // 1 KiB chunks per K step
+    constexpr int B_CH = W4 ? BN / 32 * KT / 2 : BN / 32 * KT;
     constexpr int CH = A_CH + B_CH;
     constexpr int LPW = (CH + NW - 1) / NW;           // chunk loads per wave per step
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][CH * 1024];
+    constexpr int STAGE_BYTES = NW * 32 * (32 * 4 + 8); // epilogue staging, one tile per wave
+    constexpr int LDS_BYTES = 2 * CH * 1024 > STAGE_BYTES ? 2 * CH * 1024 : STAGE_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    uint8_t(*lds)[CH * 1024] = reinterpret_cast<uint8_t(*)[CH * 1024]>(lds_raw);
 
     const int lane = lane_id(), wave = wave_id();
     const int wm = wave / WN, wn = wave % WN;
     const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
     const int KB = Kp / 32;
-    const int ksteps_total = Kp / 64;
+    const int ksteps_total = KB / KT;
 
     // ---- tile assignment
     const int total = mblocks * nblocks * ksplit;
@@ -636,34 +739,28 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
         if (w_scale) w_scale += (size_t)e * g.ws_expert_stride;
     }
 
-    // ---- global -> LDS chunk assignment for this wave
+    // ---- global -> LDS chunk assignment for this wave.  Chunk c of a step:
+    // A chunks first ([row block][k-tile]), then W chunks ([col block][k-tile], or
+    // [col block] for int4 where one chunk covers both k-tiles).
     const uint8_t* src[LPW];
-    int src_step[LPW]; // bytes to advance per K step
-    int lds_off[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-        const int c = wave + i * NW;
+        const int c = min(wave + i * NW, CH - 1); // surplus slots alias the last chunk, unused
         if (c < A_CH) {
-            const int rb = mblk * (BM / 32) + (c >> 1);
-            src[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * 2 + (c & 1)) * 1024 + lane * 16;
-            src_step[i] = 2048;
-        } else if (c < CH) {
+            const int rb = mblk * (BM / 32) + c / KT;
+            src[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * KT + c % KT) * 1024 + lane * 16;
+        } else {
             const int cb = c - A_CH;
             if (W4) {
                 const int pb = nblk * (BN / 32) + cb;
-                src[i] = Wb + ((size_t)pb * (Kp / 64) + kstep0) * 1024 + lane * 16;
-                src_step[i] = 1024;
+                src[i] = Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0) * 1024 + lane * 16;
             } else {
-                const int pb = nblk * (BN / 32) + (cb >> 1);
-                src[i] = Wb + ((size_t)pb * KB + (size_t)kstep0 * 2 + (cb & 1)) * 1024 + lane * 16;
-                src_step[i] = 2048;
+                const int pb = nblk * (BN / 32) + cb / KT;
+                src[i] = Wb + ((size_t)pb * KB + (size_t)kstep0 * KT + cb % KT) * 1024 + lane * 16;
             }
-        } else {
-            src[i] = nullptr;
-            src_step[i] = 0;
         }
-        lds_off[i] = c * 1024 + lane * 16;
     }
+    constexpr int A_STEP = KT * 1024, W_STEP = W4 ? KT * 512 : KT * 1024;
 
     v16i acc[TM][TN];
 #pragma unroll
@@ -673,76 +770,135 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    v4i stage[LPW];
-    auto load_stage = [&]() {
+    v4i stage[2][LPW];  // global prefetch, two steps deep
+    v4i afr[2][TM];     // activation fragments of k-tile 0 / 1
+    v4i wraw[2][TN];    // int4: raw words of a whole step (per step parity); int8: fragments of k-tile 0 / 1
+    v4i wop[2][TN];     // int4 only: unpacked int8 operands of k-tile 0 / 1
+
+    auto load_stage = [&](v4i* regs) {
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
-            if (wave + i * NW < CH) {
-                stage[i] = *reinterpret_cast<const v4i*>(src[i]);
-                src[i] += src_step[i];
-            }
+            if (CH % NW == 0 || wave + i * NW < CH) regs[i] = *reinterpret_cast<const v4i*>(src[i]);
+            src[i] += (wave + i * NW < A_CH) ? A_STEP : W_STEP;
         }
     };
-    auto store_stage = [&](int buf) {
+    auto store_stage = [&](const v4i* regs, int buf) {
 #pragma unroll
         for (int i = 0; i < LPW; ++i)
-            if (wave + i * NW < CH) *reinterpret_cast<v4i*>(&lds[buf][lds_off[i]]) = stage[i];
+            if (CH % NW == 0 || wave + i * NW < CH)
+                *reinterpret_cast<v4i*>(&lds[buf][(wave + i * NW) * 1024 + lane * 16]) = regs[i];
     };
-
-    load_stage();
-    store_stage(0);
-    __syncthreads();
-
-    for (int s = 0; s < ksteps; ++s) {
-        const int buf = s & 1;
-        if (s + 1 < ksteps) load_stage();
-        const uint8_t* la = &lds[buf][0];
+    auto read_a = [&](v4i* dst, int buf, int kt) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            dst[i] = *reinterpret_cast<const v4i*>(&lds[buf][((wm * TM + i) * KT + kt) * 1024 + lane * 16]);
+    };
+    auto read_w = [&](v4i* dst, int buf, int kt) {
         const uint8_t* lb = &lds[buf][A_CH * 1024];
-        if (!W4) {
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
-                v4i af[TM], bf[TN];
+        for (int j = 0; j < TN; ++j)
+            dst[j] = *reinterpret_cast<const v4i*>(
+                lb + (W4 ? (wn * TN + j) : (wn * TN + j) * KT + kt) * 1024 + lane * 16);
+    };
+    auto unpack = [&](v4i* dst, const v4i* raw, int kt) {
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    af[i] = *reinterpret_cast<const v4i*>(la + ((wm * TM + i) * 2 + kt) * 1024 + lane * 16);
+        for (int j = 0; j < TN; ++j) {
+            const int w0 = kt ? raw[j].z : raw[j].x;
+            const int w1 = kt ? raw[j].w : raw[j].y;
+            dst[j].x = (w0 << 4) & 0xF0F0F0F0;
+            dst[j].y = w0 & 0xF0F0F0F0;
+            dst[j].z = (w1 << 4) & 0xF0F0F0F0;
+            dst[j].w = w1 & 0xF0F0F0F0;
+        }
+    };
+    auto mfma_all = [&](const v4i* a, const v4i* w) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    bf[j] = *reinterpret_cast<const v4i*>(lb + ((wn * TN + j) * 2 + kt) * 1024 + lane * 16);
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[j], a[i], acc[i][j], 0, 0, 0);
+    };
+    // One K step.  P = parity (LDS buffer / stage / raw-word buffer of this
+    // step); NEXT: a following step exists; NEXT2: the step after that exists.
+    auto k_step = [&](auto parity, auto next_tag, auto next2_tag) {
+        constexpr int P = decltype(parity)::value;
+        constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+        // ---- k-tile 0
+        if (NEXT2) load_stage(stage[P]);
+        read_a(afr[1], P, 1);
+        if constexpr (!W4) read_w(wraw[1], P, 1);
+        if (NEXT) store_stage(stage[P ^ 1], P ^ 1);
+        if constexpr (W4) {
+            unpack(wop[1], wraw[P], 1);   // operands of k-tile 1, in the shadow of k-tile 0's MFMAs
+            mfma_all(afr[0], wop[0]);
 #pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            for (int q = 0; q < TM * TN; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // 1 MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0); // VALU
+                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);     // 1 LDS op
+                if (NEXT2 && q < LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // 1 global load
             }
         } else {
-            v4i praw[TN];
+            mfma_all(afr[0], wraw[0]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                praw[j] = *reinterpret_cast<const v4i*>(lb + (wn * TN + j) * 1024 + lane * 16);
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
-                v4i af[TM], bf[TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    af[i] = *reinterpret_cast<const v4i*>(la + ((wm * TM + i) * 2 + kt) * 1024 + lane * 16);
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const int w0 = kt ? praw[j].z : praw[j].x;
-                    const int w1 = kt ? praw[j].w : praw[j].y;
-                    bf[j].x = (w0 << 4) & 0xF0F0F0F0;
-                    bf[j].y = w0 & 0xF0F0F0F0;
-                    bf[j].z = (w1 << 4) & 0xF0F0F0F0;
-                    bf[j].w = w1 & 0xF0F0F0F0;
-                }
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            for (int q = 0; q < TM * TN; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (q < TM + TN + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+                if (NEXT2 && q < LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
         }
-        if (s + 1 < ksteps) store_stage(buf ^ 1);
-        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();
+        // ---- k-tile 1: fetch the first fragments of the next step under its MFMAs
+        if (NEXT) {
+            read_a(afr[0], P ^ 1, 0);
+            read_w(W4 ? wraw[P ^ 1] : wraw[0], P ^ 1, 0);
+        }
+        if constexpr (W4) {
+            mfma_all(afr[1], wop[1]);
+            if (NEXT) unpack(wop[0], wraw[P ^ 1], 0);
+#pragma unroll
+            for (int q = 0; q < TM * TN; ++q) {
+                if (q < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS reads first
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (NEXT && q >= TM * TN / 2)
+                    __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN / 2 - 1) / (TM * TN / 2), 0);
+            }
+        } else {
+            mfma_all(afr[1], wraw[1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+
+    // prologue: steps 0 and 1 in flight, step 0 in LDS, its first fragments in registers
+    load_stage(stage[0]);
+    if (ksteps > 1) load_stage(stage[1]);
+    store_stage(stage[0], 0);
+    lds_barrier();
+    read_a(afr[0], 0, 0);
+    read_w(wraw[0], 0, 0);
+    if constexpr (W4) unpack(wop[0], wraw[0], 0);
+
+    int s = 0;
+    for (; s + 3 < ksteps; s += 2) {   // steady state: both steps have a next and a next-next
+        k_step(P0{}, T_{}, T_{});
+        k_step(P1{}, T_{}, T_{});
+    }
+    // tail: at most three steps left, s is even
+    const int left = ksteps - s;
+    if (left == 3) {
+        k_step(P0{}, T_{}, T_{});
+        k_step(P1{}, T_{}, F_{});
+        k_step(P0{}, F_{}, F_{});
+    } else if (left == 2) {
+        k_step(P0{}, T_{}, F_{});
+        k_step(P1{}, F_{}, F_{});
+    } else {
+        k_step(P0{}, F_{}, F_{});
     }
 
     if (W4) {
@@ -764,30 +920,35 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int row0 = mblk * BM + (wm * TM + i) * 32;
-                const int col = (nblk * (BN / 32) + wn * TN + j) * 32 + (lane & 31);
+                const int m = mblk * BM + (wm * TM + i) * 32 + (lane & 31);
+                const int col0 = (nblk * (BN / 32) + wn * TN + j) * 32;
+                if (m < m_limit) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = row0 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                    if (m < m_limit && acc[i][j][r])
-                        atomicAdd(g.splitk_acc + (size_t)m * ld + col, acc[i][j][r]);
+                    for (int r = 0; r < 16; ++r)
+                        if (acc[i][j][r])
+                            atomicAdd(g.splitk_acc + (size_t)m * ld + col0 + tile_col(r, lane), acc[i][j][r]);
                 }
             }
         return;
     }
+    // all waves are past their last LDS fragment read (the barrier of the last
+    // step precedes only register work), so the buffers can be reused as
+    // wave-private staging for the stores
+    lds_barrier();
+    uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int row0 = mblk * BM + (wm * TM + i) * 32;
+        const int m0 = mblk * BM + (wm * TM + i) * 32;
         if constexpr (EPI == RKH_EPI_SWIGLU) {
 #pragma unroll
             for (int j = 0; j < TN; j += 2)
-                epilogue_swiglu(g, acc[i][j], acc[i][j + 1], row0, nblk * (BN / 32) + wn * TN + j,
-                                lane, g.a_scale, w_scale, m_limit);
+                epilogue_swiglu(g, acc[i][j], acc[i][j + 1], m0, nblk * (BN / 32) + wn * TN + j, lane,
+                                g.a_scale, w_scale, m_limit, stage_lds);
         } else {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                epilogue_tile<EPI>(g, acc[i][j], row0, nblk * (BN / 32) + wn * TN + j, lane,
-                                   g.a_scale, w_scale, m_limit);
+                epilogue_tile<EPI>(g, acc[i][j], m0, nblk * (BN / 32) + wn * TN + j, lane,
+                                   g.a_scale, w_scale, m_limit, stage_lds);
         }
     }
 }
@@ -814,8 +975,8 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(rkh_gemm_args g, i
         }
         if (g.row_max_bits) {
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
-            if (lane_id() == 0 && bits) atomicMax(g.row_max_bits + m, bits);
+            for (int off = 16; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+            if ((threadIdx.x & 31) == 0 && n < F) g.row_max_bits[(size_t)m * (F / 32) + (n >> 5)] = bits;
         }
     } else {
         const int pc = blockIdx.x * 256 + threadIdx.x; // physical column
@@ -972,21 +1133,21 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 }
 
 // ------------------------------------------------------------- launchers
-template <int WM, int WN, int TM, int TN>
+template <int WM, int WN, int TM, int TN, int KT>
 int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     const bool grouped = g.blk_expert != nullptr;
     const int mblocks = grouped ? (g.max_blocks + BM / 32 - 1) / (BM / 32) : (g.M + BM - 1) / BM;
     const int cols = g.N;
     const int nblocks = (cols + BN - 1) / BN;
-    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 64);
+    const int ksteps_total = (int)((rkh_align_up(g.K, RKH_K_ALIGN) / 32 + KT - 1) / KT);
     if (ksplit > ksteps_total) ksplit = ksteps_total;
     if (ksplit < 1 || grouped) ksplit = 1;
     const int per = (ksteps_total + ksplit - 1) / ksplit;
     ksplit = (ksteps_total + per - 1) / per;
     const dim3 grid(mblocks * nblocks * ksplit), block(WM * WN * 64);
 #define RK_LAUNCH(W4, EPI, GR)                                                              \
-    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, W4, EPI, GR>), grid, block, 0, st, g,   \
+    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, KT, W4, EPI, GR>), grid, block, 0, st, g,   \
                        mblocks, nblocks, ksplit, per)
 #define RK_BY_EPI(W4, GR)                                                  \
     switch (g.epilogue) {                                                  \
@@ -1219,7 +1380,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
         if (g.M <= 4) return launch_gemv<4>(st, g);
         return launch_gemv<8>(st, g);
     }
-    if (grouped) return launch_gemm_cfg<1, 4, 1, 2>(st, g, 1);
+    if (grouped) return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, 1);
     const DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {
@@ -1227,9 +1388,9 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
         ksplit = 1;
     }
     const int bm = plan.bm;
-    if (bm == 128) return launch_gemm_cfg<2, 2, 2, 4>(st, g, ksplit);
-    if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2>(st, g, ksplit);
-    return launch_gemm_cfg<1, 4, 1, 2>(st, g, ksplit);
+    if (bm == 128) return launch_gemm_cfg<2, 2, 2, 4, 2>(st, g, ksplit);
+    if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2, 2>(st, g, ksplit);
+    return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, ksplit);
 }
 
 int rkh_moe_route(void* stream, const rkh_moe_route_args* args) {

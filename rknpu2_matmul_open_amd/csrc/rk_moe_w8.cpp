@@ -74,7 +74,7 @@ struct rk_npu_moe_w8_workspace {
     DeviceBuffer a_tiled;      // sorted token rows, tiled int8 [sorted_rows x align64(H)]
     DeviceBuffer a_scale;      // [sorted_rows]
     DeviceBuffer hidden;       // [sorted_rows, I] fp32
-    DeviceBuffer row_max;      // [sorted_rows]
+    DeviceBuffer row_max;      // [sorted_rows][I/32] partial row maxima of hidden
     DeviceBuffer h_tiled;      // re-quantized hidden, tiled int8 [sorted_rows x align64(I)]
     DeviceBuffer h_scale;      // [sorted_rows]
     DeviceBuffer y;            // [sorted_rows, H] fp32 expert outputs
@@ -132,7 +132,6 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     q.scale = f32 ? ws->token_scale.as<float>() : const_cast<float*>(d_scales);
     q.dst = ws->a_tiled.as<>();
     q.bad_flag = ws->flag.device();
-    q.zero_bits = ws->row_max.as<uint32_t>();
     q.dest_rows = ws->dest_rows.as<int>();
     q.dest_stride = ws->slots;
     q.scale_rows = ws->a_scale.as<float>();
@@ -171,6 +170,7 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     q2.scale = ws->h_scale.as<float>();
     q2.dst = ws->h_tiled.as<>();
     q2.row_max_bits = ws->row_max.as<uint32_t>();
+    q2.row_max_parts = I / 32;
     q2.active_blocks = ws->num_blocks.as<int>();
     rc = rkh_quant_rows(stream, &q2);
     if (rc) return map_error(rc);
@@ -382,7 +382,7 @@ rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* dom
         ws->num_blocks.alloc(ws->owner, 16) ||
         ws->a_tiled.alloc(ws->owner, rkh_tiled_i8_bytes(ws->sorted_rows, H, 32)) ||
         ws->a_scale.alloc(ws->owner, S * 4) || ws->hidden.alloc(ws->owner, S * I * 4) ||
-        ws->row_max.alloc(ws->owner, S * 4) ||
+        ws->row_max.alloc(ws->owner, S * (size_t)(I / 32) * 4) ||
         ws->h_tiled.alloc(ws->owner, rkh_tiled_i8_bytes(ws->sorted_rows, I, 32)) ||
         ws->h_scale.alloc(ws->owner, S * 4) || ws->y.alloc(ws->owner, S * H * 4) ||
         ws->out.alloc(ws->owner, (size_t)R * H * 4, false) || ws->flag.init(ws->owner))

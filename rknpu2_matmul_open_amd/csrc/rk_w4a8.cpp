@@ -161,7 +161,7 @@ struct rk_npu_w4a8_workspace {
     DeviceBuffer a_tiled;   // quantized activations
     DeviceBuffer a_scale;   // [align128(M)]
     DeviceBuffer c_out;     // [M, N] fp32-sized result staging
-    DeviceBuffer row_max;   // [align128(M)] uint32 row maxima of the SwiGLU middle
+    DeviceBuffer row_max;   // [align128(M)][N/64] partial row maxima of the SwiGLU middle
     DeviceBuffer splitk;
     BadFlag flag;
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
@@ -211,9 +211,9 @@ int enqueue(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void*
     if (scale_source) {
         q.mode = RKH_Q_REUSE_BITS;
         q.row_max_bits = scale_source->row_max.as<uint32_t>();
+        q.row_max_parts = scale_source->config.N / 64; // one partial per 32 middle columns
     } else {
         q.mode = RKH_Q_W4A8;
-        if (collect) q.zero_bits = ws->row_max.as<uint32_t>();
     }
     int rc = rkh_quant_rows(stream, &q);
     if (rc) return map_error(rc);
@@ -485,7 +485,8 @@ rk_npu_w4a8_workspace* rk_npu_w4a8_workspace_create_ex(rk_npu_iommu_domain* doma
         ws->a_tiled.alloc(ws->owner, rkh_tiled_i8_bytes(M, K, RKH_ROW_ALIGN)) ||
         ws->a_scale.alloc(ws->owner, rows * sizeof(float)) ||
         ws->c_out.alloc(ws->owner, (size_t)M * N * 4, false) ||
-        ws->row_max.alloc(ws->owner, rows * sizeof(uint32_t)) || ws->flag.init(ws->owner))
+        ws->row_max.alloc(ws->owner, rows * (size_t)(N / 64 + 1) * sizeof(uint32_t)) ||
+        ws->flag.init(ws->owner))
         return nullptr;
     const size_t scratch = splitk_scratch_bytes(M, N, K, true);
     if (scratch && ws->splitk.alloc(ws->owner, scratch)) return nullptr;
