@@ -12,6 +12,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <float.h>
+#include <stdio.h>
+#include <stdlib.h>
 #include <type_traits>
 
 #include "rk_hip_shim.h"
@@ -28,6 +30,15 @@ namespace {
         if (e_ != hipSuccess) return e_ == hipErrorOutOfMemory ? RKH_ERR_NOMEM \
                                                                : RKH_ERR_RUNTIME; \
     } while (0)
+
+// Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(<N-1>{}).
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
@@ -672,34 +683,38 @@ __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v1
 }
 
 // Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn), each
-// wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is KT 32-deep
-// k-tiles.  Tiles travel global -> registers -> LDS as whole 1 KiB tiles, so LDS
-// reads are linear 16 bytes per lane (bank-conflict free) and land directly in
-// MFMA operand order.
+// wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is two 32-deep
+// k-tiles.
 //
-// Software pipeline (one wave per SIMD, so latency is hidden by ILP only):
-//  - global loads run two K steps ahead in two register stages;
-//  - LDS fragment reads run one k-tile ahead of the MFMAs that use them, the
-//    int4 -> int8 unpack of the next k-tile is interleaved between the MFMAs of
-//    the current one (fragment and operand registers are double buffered);
-//  - the LDS writes of the next step are issued at the start of the step and
-//    the workgroup barrier sits before the LAST k-tile, so the first fragments
-//    of the next step are fetched under that k-tile's MFMAs.
+// Operand delivery.  Both matrices are stored as 1 KiB MFMA-ordered tiles, so a
+// fragment is one 16-byte-per-lane load.  With one wave per SIMD a wave can pull
+// only about 17 B/clk out of LDS, which makes LDS traffic, not MFMA, the limit
+// if both operands are staged there.  Therefore:
+//  - the weight fragments go global -> registers directly (each wave needs its
+//    own columns; the copy of the other wm-row of waves is served by the L1),
+//    through a ring of NS register stages that runs NS-1 K steps ahead;
+//  - only the activation tile, which every wave of the group needs, is staged
+//    through double-buffered LDS (global -> registers -> LDS, two steps ahead).
+// Software pipeline per step: the LDS writes of the next step are issued first,
+// the activation fragments of k-tile 1 are read and the int4 -> int8 unpack of
+// k-tile 1 is interleaved under the MFMAs of k-tile 0; the workgroup barrier
+// sits before k-tile 1 so that the first fragments of the next step are fetched
+// under k-tile 1's MFMAs.
 template <int WM, int WN, int TM, int TN, int KT, bool W4, int EPI, bool GROUPED>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int mblocks,
                                                             int nblocks, int ksplit,
                                                             int ksteps_per_part) {
     static_assert(KT == 2, "the pipeline below is written for two k-tiles per step");
     constexpr int NW = WM * WN;
+    constexpr int NS = 8;                             // register prefetch stages (even)
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int A_CH = BM / 32 * KT;                // 1 KiB chunks per K step
-    constexpr int B_CH = W4 ? BN / 32 * KT / 2 : BN / 32 * KT;
-    constexpr int CH = A_CH + B_CH;
-    constexpr int LPW = (CH + NW - 1) / NW;           // chunk loads per wave per step
+    constexpr int A_CH = BM / 32 * KT;                // 1 KiB activation chunks per K step
+    constexpr int LPW = (A_CH + NW - 1) / NW;         // activation chunk loads per wave per step
+    constexpr int WF = W4 ? TN : TN * KT;             // weight registers (v4i) per step
     constexpr int STAGE_BYTES = NW * 32 * (32 * 4 + 8); // epilogue staging, one tile per wave
-    constexpr int LDS_BYTES = 2 * CH * 1024 > STAGE_BYTES ? 2 * CH * 1024 : STAGE_BYTES;
+    constexpr int LDS_BYTES = 2 * A_CH * 1024 > STAGE_BYTES ? 2 * A_CH * 1024 : STAGE_BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
-    uint8_t(*lds)[CH * 1024] = reinterpret_cast<uint8_t(*)[CH * 1024]>(lds_raw);
+    uint8_t(*lds)[A_CH * 1024] = reinterpret_cast<uint8_t(*)[A_CH * 1024]>(lds_raw);
 
     const int lane = lane_id(), wave = wave_id();
     const int wm = wave / WN, wn = wave % WN;
@@ -739,28 +754,24 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
         if (w_scale) w_scale += (size_t)e * g.ws_expert_stride;
     }
 
-    // ---- global -> LDS chunk assignment for this wave.  Chunk c of a step:
-    // A chunks first ([row block][k-tile]), then W chunks ([col block][k-tile], or
-    // [col block] for int4 where one chunk covers both k-tiles).
-    const uint8_t* src[LPW];
+    // ---- sources.  Activation chunk c of a step = [row block c / KT][k-tile c % KT].
+    const uint8_t* asrc[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-        const int c = min(wave + i * NW, CH - 1); // surplus slots alias the last chunk, unused
-        if (c < A_CH) {
-            const int rb = mblk * (BM / 32) + c / KT;
-            src[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * KT + c % KT) * 1024 + lane * 16;
-        } else {
-            const int cb = c - A_CH;
-            if (W4) {
-                const int pb = nblk * (BN / 32) + cb;
-                src[i] = Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0) * 1024 + lane * 16;
-            } else {
-                const int pb = nblk * (BN / 32) + cb / KT;
-                src[i] = Wb + ((size_t)pb * KB + (size_t)kstep0 * KT + cb % KT) * 1024 + lane * 16;
-            }
-        }
+        const int c = min(wave + i * NW, A_CH - 1); // surplus slots alias the last chunk, unused
+        const int rb = mblk * (BM / 32) + c / KT;
+        asrc[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * KT + c % KT) * 1024 + lane * 16;
     }
-    constexpr int A_STEP = KT * 1024, W_STEP = W4 ? KT * 512 : KT * 1024;
+    // Weight column block j of this wave: int4 = one chunk per step (both
+    // k-tiles), int8 = two consecutive chunks per step.
+    const uint8_t* wsrc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int pb = nblk * (BN / 32) + wn * TN + j;
+        wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0) * 1024 + lane * 16
+                     : Wb + ((size_t)pb * KB + (size_t)kstep0 * KT) * 1024 + lane * 16;
+    }
+    constexpr int A_STEP = KT * 1024, W_STEP = W4 ? 1024 : KT * 1024;
 
     v16i acc[TM][TN];
 #pragma unroll
@@ -770,35 +781,40 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    v4i stage[2][LPW];  // global prefetch, two steps deep
+    v4i stage[NS][LPW]; // activation prefetch ring (same depth as the weight ring)
     v4i afr[2][TM];     // activation fragments of k-tile 0 / 1
-    v4i wraw[2][TN];    // int4: raw words of a whole step (per step parity); int8: fragments of k-tile 0 / 1
+    v4i wring[NS][WF];  // weights: raw int4 words of a step, or int8 fragments [j * KT + kt]
     v4i wop[2][TN];     // int4 only: unpacked int8 operands of k-tile 0 / 1
 
-    auto load_stage = [&](v4i* regs) {
+    auto load_a = [&](v4i* regs) {
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
-            if (CH % NW == 0 || wave + i * NW < CH) regs[i] = *reinterpret_cast<const v4i*>(src[i]);
-            src[i] += (wave + i * NW < A_CH) ? A_STEP : W_STEP;
+            if (A_CH % NW == 0 || wave + i * NW < A_CH) regs[i] = *reinterpret_cast<const v4i*>(asrc[i]);
+            asrc[i] += A_STEP;
         }
     };
-    auto store_stage = [&](const v4i* regs, int buf) {
+    auto store_a = [&](const v4i* regs, int buf) {
 #pragma unroll
         for (int i = 0; i < LPW; ++i)
-            if (CH % NW == 0 || wave + i * NW < CH)
+            if (A_CH % NW == 0 || wave + i * NW < A_CH)
                 *reinterpret_cast<v4i*>(&lds[buf][(wave + i * NW) * 1024 + lane * 16]) = regs[i];
+    };
+    auto load_w = [&](v4i* regs) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (W4) {
+                regs[j] = *reinterpret_cast<const v4i*>(wsrc[j]);
+            } else {
+                regs[j * KT] = *reinterpret_cast<const v4i*>(wsrc[j]);
+                regs[j * KT + 1] = *reinterpret_cast<const v4i*>(wsrc[j] + 1024);
+            }
+            wsrc[j] += W_STEP;
+        }
     };
     auto read_a = [&](v4i* dst, int buf, int kt) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
             dst[i] = *reinterpret_cast<const v4i*>(&lds[buf][((wm * TM + i) * KT + kt) * 1024 + lane * 16]);
-    };
-    auto read_w = [&](v4i* dst, int buf, int kt) {
-        const uint8_t* lb = &lds[buf][A_CH * 1024];
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-            dst[j] = *reinterpret_cast<const v4i*>(
-                lb + (W4 ? (wn * TN + j) : (wn * TN + j) * KT + kt) * 1024 + lane * 16);
     };
     auto unpack = [&](v4i* dst, const v4i* raw, int kt) {
 #pragma unroll
@@ -811,95 +827,92 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
             dst[j].w = w1 & 0xF0F0F0F0;
         }
     };
-    auto mfma_all = [&](const v4i* a, const v4i* w) {
+    // MFMAs of one k-tile; weights are the first operand (see tile_col()).
+    auto mfma_all = [&](const v4i* a, const v4i* w, int wstride, int woff) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[j], a[i], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[j * wstride + woff], a[i], acc[i][j], 0, 0, 0);
     };
-    // One K step.  P = parity (LDS buffer / stage / raw-word buffer of this
-    // step); NEXT: a following step exists; NEXT2: the step after that exists.
-    auto k_step = [&](auto parity, auto next_tag, auto next2_tag) {
-        constexpr int P = decltype(parity)::value;
-        constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+
+    // One K step.  SLOT = s % NS selects the register stage, SLOT % 2 the LDS
+    // buffer.  n1 / n3: step s+1 / s+(NS-1) exists (compile-time true in the
+    // steady state, run-time flags in the tail).
+    auto k_step = [&](auto slot_tag, auto n1, auto n3) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        constexpr int P = SLOT & 1;
         // ---- k-tile 0
-        if (NEXT2) load_stage(stage[P]);
+        // Loads complete in issue order: the activations go first so that waiting
+        // for them (for the LDS write two steps later) leaves the weight loads of
+        // the same and later steps in flight.
+        if (n3) load_a(stage[(SLOT + NS - 1) % NS]);
+        if (n3) load_w(wring[(SLOT + NS - 1) % NS]);
         read_a(afr[1], P, 1);
-        if constexpr (!W4) read_w(wraw[1], P, 1);
-        if (NEXT) store_stage(stage[P ^ 1], P ^ 1);
+        if (n1) store_a(stage[(SLOT + 1) % NS], P ^ 1);
         if constexpr (W4) {
-            unpack(wop[1], wraw[P], 1);   // operands of k-tile 1, in the shadow of k-tile 0's MFMAs
-            mfma_all(afr[0], wop[0]);
+            unpack(wop[1], wring[SLOT], 1);
+            mfma_all(afr[0], wop[0], 1, 0);
 #pragma unroll
             for (int q = 0; q < TM * TN; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // 1 MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0); // VALU
-                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);     // 1 LDS op
-                if (NEXT2 && q < LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // 1 global load
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // 1 MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0);
+                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // 1 LDS op
+                if (q < TN + LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // 1 global load
             }
         } else {
-            mfma_all(afr[0], wraw[0]);
+            mfma_all(afr[0], wring[SLOT], KT, 0);
 #pragma unroll
             for (int q = 0; q < TM * TN; ++q) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (q < TM + TN + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
-                if (NEXT2 && q < LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+                if (q < TN * KT + LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
         // ---- k-tile 1: fetch the first fragments of the next step under its MFMAs
-        if (NEXT) {
-            read_a(afr[0], P ^ 1, 0);
-            read_w(W4 ? wraw[P ^ 1] : wraw[0], P ^ 1, 0);
-        }
+        if (n1) read_a(afr[0], P ^ 1, 0);
         if constexpr (W4) {
-            mfma_all(afr[1], wop[1]);
-            if (NEXT) unpack(wop[0], wraw[P ^ 1], 0);
+            mfma_all(afr[1], wop[1], 1, 0);
+            if (n1) unpack(wop[0], wring[(SLOT + 1) % NS], 0);
 #pragma unroll
             for (int q = 0; q < TM * TN; ++q) {
-                if (q < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS reads first
+                if (q < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // LDS reads first
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (NEXT && q >= TM * TN / 2)
-                    __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN / 2 - 1) / (TM * TN / 2), 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0);
             }
         } else {
-            mfma_all(afr[1], wraw[1]);
+            mfma_all(afr[1], wring[SLOT], KT, 1);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
     using T_ = std::true_type;
-    using F_ = std::false_type;
-    using P0 = std::integral_constant<int, 0>;
-    using P1 = std::integral_constant<int, 1>;
 
-    // prologue: steps 0 and 1 in flight, step 0 in LDS, its first fragments in registers
-    load_stage(stage[0]);
-    if (ksteps > 1) load_stage(stage[1]);
-    store_stage(stage[0], 0);
+    // prologue: weights of steps 0..NS-2 and activations of steps 0, 1 in flight;
+    // step 0 in LDS, its first fragments in registers
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i) {
+        if (i < ksteps) {
+            load_a(stage[i]);
+            load_w(wring[i]);
+        }
+    }
+    store_a(stage[0], 0);
     lds_barrier();
     read_a(afr[0], 0, 0);
-    read_w(wraw[0], 0, 0);
-    if constexpr (W4) unpack(wop[0], wraw[0], 0);
+    if constexpr (W4) unpack(wop[0], wring[0], 0);
 
     int s = 0;
-    for (; s + 3 < ksteps; s += 2) {   // steady state: both steps have a next and a next-next
-        k_step(P0{}, T_{}, T_{});
-        k_step(P1{}, T_{}, T_{});
-    }
-    // tail: at most three steps left, s is even
-    const int left = ksteps - s;
-    if (left == 3) {
-        k_step(P0{}, T_{}, T_{});
-        k_step(P1{}, T_{}, F_{});
-        k_step(P0{}, F_{}, F_{});
-    } else if (left == 2) {
-        k_step(P0{}, T_{}, F_{});
-        k_step(P1{}, F_{}, F_{});
-    } else {
-        k_step(P0{}, F_{}, F_{});
-    }
+    // steady state: NS steps per trip, every look-ahead exists
+    for (; s + 2 * NS - 2 < ksteps; s += NS)
+        static_for<NS>([&](auto slot) { k_step(slot, T_{}, T_{}); });
+    // tail: run-time look-ahead flags
+    for (; s < ksteps; s += NS)
+        static_for<NS>([&](auto slot) {
+            constexpr int SL = decltype(slot)::value;
+            if (s + SL < ksteps) k_step(slot, s + SL + 1 < ksteps, s + SL + NS - 1 < ksteps);
+        });
 
     if (W4) {
 #pragma unroll
@@ -1381,14 +1394,24 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
         return launch_gemv<8>(st, g);
     }
     if (grouped) return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, 1);
-    const DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
+    DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
+    // Tuning aid: RK_NPU_HIP_GEMM_PLAN="rows:ksplit" forces the workgroup tile
+    // rows (32 / 64 / 128) and the K split of dense launches.
+    static const char* forced = getenv("RK_NPU_HIP_GEMM_PLAN");
+    if (forced) {
+        int rows = 0, split = 0;
+        if (sscanf(forced, "%d:%d", &rows, &split) == 2 && (rows == 32 || rows == 64 || rows == 128) && split >= 1) {
+            plan.bm = rows;
+            plan.ksplit = split > min_ksplit(g.K, g.w_int4) ? split : min_ksplit(g.K, g.w_int4);
+        }
+    }
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {
         if (min_ksplit(g.K, g.w_int4) > 1) return RKH_ERR_RUNTIME;
         ksplit = 1;
     }
     const int bm = plan.bm;
-    if (bm == 128) return launch_gemm_cfg<2, 2, 2, 4, 2>(st, g, ksplit);
+    if (bm == 128) return launch_gemm_cfg<2, 4, 2, 2, 2>(st, g, ksplit);
     if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2, 2>(st, g, ksplit);
     return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, ksplit);
 }
