@@ -1,0 +1,236 @@
+"""The C-ABI boundary without a GPU: headers are valid C99, the shared library
+loads and exports every function the headers declare, struct layouts seen by a
+C compiler equal the ctypes mirror, defaults and the CPU-only queries return
+the numbers the reference's own tests pin, and opening a context on a machine
+without a device fails cleanly (no compute path is entered)."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from rknpu2_matmul_open_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INC = os.path.join(ROOT, "include")
+HEADERS = ["rk_npu_common.h", "rk_npu_quant_matmul.h", "rk_npu_matmul_i4.h", "rk_npu_w4a8.h",
+           "rk_npu_moe_w8.h", "rk_npu_hip.h"]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return capi.load_library()
+
+
+def _declared_functions():
+    names = set()
+    for h in HEADERS:
+        text = open(os.path.join(INC, h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        for m in re.finditer(r"\b(rk_npu_[a-z0-9_]+)\s*\(", text):
+            names.add(m.group(1))
+    return names
+
+
+def test_headers_compile_as_c99(tmp_path):
+    """reference tests/test_quant_header.c, test_w4a8_header.c, test_moe_w8_header.c:
+    plain-C translation units keep the headers valid C."""
+    for h in HEADERS:
+        src = tmp_path / (h + ".c")
+        src.write_text('#include "%s"\nint main(void) { return 0; }\n' % h)
+        subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", INC, "-c", str(src),
+                               "-o", str(tmp_path / "o.o")])
+
+
+def test_library_exports_every_declared_function(lib):
+    declared = _declared_functions()
+    assert len(declared) > 60
+    missing = [n for n in sorted(declared) if not hasattr(lib, n)]
+    assert not missing, missing
+    # and the ctypes mirror binds exactly those
+    assert set(capi.EXPORTED_SYMBOLS) == declared
+
+
+def test_struct_layouts_match_the_c_compiler(tmp_path):
+    pairs = [("rk_npu_matmul_strategy", capi.MatmulStrategy), ("rk_npu_matmul_autotune_config", capi.MatmulAutotuneConfig),
+             ("rk_npu_matmul_weight_config", capi.MatmulWeightConfig),
+             ("rk_npu_matmul_workspace_requirements", capi.WorkspaceRequirements),
+             ("rk_npu_matmul_weight_requirements", capi.WeightRequirements),
+             ("rk_npu_i4_weight_config", capi.I4WeightConfig), ("rk_npu_i4_memory_info", capi.I4MemoryInfo),
+             ("rk_npu_w4a8_config", capi.W4A8Config), ("rk_npu_w4a8_memory_info", capi.W4A8MemoryInfo),
+             ("rk_npu_w4a8_options", capi.W4A8Options), ("rk_npu_w4a8_memory_info_ex", capi.W4A8MemoryInfoEx),
+             ("rk_npu_w4a8_timings", capi.W4A8Timings), ("rk_npu_w4a8_weight_info", capi.W4A8WeightInfo),
+             ("rk_npu_w4a8_ffn_timings", capi.W4A8FfnTimings),
+             ("rk_npu_moe_w8_weight_config", capi.MoeWeightConfig), ("rk_npu_moe_w8_config", capi.MoeConfig),
+             ("rk_npu_moe_w8_expert", capi.MoeExpert), ("rk_npu_moe_w8_timings", capi.MoeTimings),
+             ("rk_npu_domain_memory_stats", capi.DomainMemoryStats)]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rk_npu_hip.h"', "int main(void) {"]
+    for cname, ct in pairs:
+        lines.append('printf("%s %%zu", sizeof(%s));' % (cname, cname))
+        for fname, _ in ct._fields_:
+            lines.append('printf(" %%zu", offsetof(%s, %s));' % (cname, fname))
+        lines.append('printf("\\n");')
+    lines.append("return 0; }")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c99", "-I", INC, str(src), "-o", str(exe)])
+    out = subprocess.check_output([str(exe)]).decode().splitlines()
+    for line, (cname, ct) in zip(out, pairs):
+        parts = line.split()
+        assert parts[0] == cname
+        assert int(parts[1]) == C.sizeof(ct), cname
+        for off, (fname, _) in zip(parts[2:], ct._fields_):
+            assert int(off) == getattr(ct, fname).offset, (cname, fname)
+
+
+def test_error_codes_and_strings(lib):
+    assert (capi.RK_NPU_OK, capi.RK_NPU_ERR_OPEN, capi.RK_NPU_ERR_IOCTL, capi.RK_NPU_ERR_PARAM,
+            capi.RK_NPU_ERR_NOMEM, capi.RK_NPU_ERR_SUBMIT, capi.RK_NPU_ERR_BUSY, capi.RK_NPU_ERR_DOMAIN,
+            capi.RK_NPU_ERR_IO, capi.RK_NPU_ERR_CACHE_MISS) == (0, -1, -2, -3, -4, -5, -6, -7, -8, -9)
+    assert lib.rk_npu_strerror(0) == b"ok"
+    assert lib.rk_npu_strerror(-3) == b"bad argument"
+    assert lib.rk_npu_strerror(-6) == b"workspace is already running"
+    assert lib.rk_npu_strerror(-9) == b"tuning cache miss"
+    assert lib.rk_npu_strerror(-77) == b"unknown error"
+    assert len({lib.rk_npu_strerror(c) for c in range(0, -10, -1)}) == 10
+
+
+def test_defaults_of_config_init(lib):
+    """reference src/rk_npu_w4a8.cpp:162-168, src/rk_npu_moe_w8.cpp:824-826,
+    src/rk_npu_quant_matmul.cpp:1522-1535."""
+    w = capi.W4A8Config()
+    lib.rk_npu_w4a8_config_init(C.byref(w), 7, 65, 513)
+    assert (w.M, w.N, w.K, w.m_tile, w.k_tile, w.n_tile, w.npu_core_mask, w.timeout_ms, w.pipeline,
+            w.cpu_threads) == (7, 65, 513, 64, 480, 1024, 1, 500, 1, 1)
+    o = capi.W4A8Options()
+    lib.rk_npu_w4a8_options_init(C.byref(o))
+    assert (o.struct_size, o.input_layout, o.reduce_backend) == (C.sizeof(capi.W4A8Options), 0, 0)
+    m = capi.MoeConfig()
+    lib.rk_npu_moe_w8_config_init(C.byref(m), 2048, 512, 64, 1, 8, 256)
+    assert (m.struct_size, m.weights.hidden, m.weights.intermediate, m.weights.routed_experts,
+            m.weights.shared_expert, m.max_rows, m.top_k, m.npu_cores, m.cpu_threads, m.native_input,
+            m.middle, m.timeout_ms) == (C.sizeof(capi.MoeConfig), 2048, 512, 64, 1, 256, 8, 3, 4, 0, 0, 1000)
+    a = capi.MatmulAutotuneConfig()
+    lib.rk_npu_matmul_autotune_config_init(C.byref(a), 3, 4, 5)
+    assert (a.M, a.N, a.K, a.allowed_npu_core_mask, a.allowed_cpu_core_mask, a.warmup, a.loops, a.repeats,
+            a.timeout_ms, a.verbose, a.required_k_tile) == (3, 4, 5, 7, 0, 2, 8, 3, 500, 0, 0)
+    lib.rk_npu_w4a8_config_init(None, 1, 1, 1)   # NULL is ignored
+    lib.rk_npu_moe_w8_config_init(None, 1, 1, 1, 0, 1, 1)
+
+
+def test_w4a8_memory_query_pins(lib):
+    """reference tests/test_w4a8_cpu.cpp:143-152 and tests/test_w4a8_reduction.cpp:112-119."""
+    cfg = capi.W4A8Config()
+    lib.rk_npu_w4a8_config_init(C.byref(cfg), 3, 65, 513)
+    mem = capi.W4A8MemoryInfo()
+    assert lib.rk_npu_w4a8_memory_query(C.byref(cfg), C.byref(mem)) == 0
+    assert mem.weight_metadata_bytes == 65 * 8 == 520
+    assert mem.cpu_scratch_bytes == 3 * 128 * 4 + 3 * 8 == 1560
+    assert mem.backend.wave_count == 2 and mem.backend.packed_weight_bytes == 544 * 128 // 2
+    cfg.m_tile = 65
+    assert lib.rk_npu_w4a8_memory_query(C.byref(cfg), C.byref(mem)) == capi.RK_NPU_ERR_PARAM
+    cfg.m_tile = 64
+    cfg.K = (2 ** 31 - 1) // 1024 + 1
+    assert lib.rk_npu_w4a8_memory_query(C.byref(cfg), C.byref(mem)) == capi.RK_NPU_ERR_PARAM
+    lib.rk_npu_w4a8_config_init(C.byref(cfg), 128, 4096, 11008)
+    ex = capi.W4A8MemoryInfoEx()
+    assert lib.rk_npu_w4a8_memory_query_ex(C.byref(cfg), None, C.byref(ex)) == 0
+    assert ex.base.backend.partial_bytes == 2 * 256 * 4096 * 2 == 4194304
+    assert ex.effective_reduce_backend == capi.W4A8_REDUCE_CPU
+    # option handling: NPU reduce is effective only for M > 16; CHAIN + NPU reduce is rejected
+    opt = capi.W4A8Options()
+    lib.rk_npu_w4a8_options_init(C.byref(opt))
+    opt.reduce_backend = capi.W4A8_REDUCE_NPU
+    assert lib.rk_npu_w4a8_memory_query_ex(C.byref(cfg), C.byref(opt), C.byref(ex)) == 0
+    assert ex.effective_reduce_backend == capi.W4A8_REDUCE_NPU
+    cfg.pipeline = capi.W4A8_CHAIN
+    assert lib.rk_npu_w4a8_memory_query_ex(C.byref(cfg), C.byref(opt), C.byref(ex)) == capi.RK_NPU_ERR_PARAM
+    cfg.pipeline = capi.W4A8_PIPELINED
+    cfg.M = 16
+    assert lib.rk_npu_w4a8_memory_query_ex(C.byref(cfg), C.byref(opt), C.byref(ex)) == 0
+    assert ex.effective_reduce_backend == capi.W4A8_REDUCE_CPU
+    opt.struct_size = 3
+    assert lib.rk_npu_w4a8_memory_query_ex(C.byref(cfg), C.byref(opt), C.byref(ex)) == capi.RK_NPU_ERR_PARAM
+    for field, bad in (("k_tile", 0), ("k_tile", 48), ("k_tile", 2080), ("n_tile", 32), ("n_tile", 100),
+                       ("n_tile", 8192), ("npu_core_mask", 5), ("npu_core_mask", 0), ("timeout_ms", 0),
+                       ("cpu_threads", 0), ("cpu_threads", 5), ("pipeline", 3), ("M", 0), ("N", 0)):
+        lib.rk_npu_w4a8_config_init(C.byref(cfg), 8, 256, 512)
+        setattr(cfg, field, bad)
+        assert lib.rk_npu_w4a8_memory_query(C.byref(cfg), C.byref(mem)) == capi.RK_NPU_ERR_PARAM, (field, bad)
+    lib.rk_npu_w4a8_config_init(C.byref(cfg), 8, 64, 512)
+    cfg.npu_core_mask = 3     # two cores need two 64-column blocks
+    assert lib.rk_npu_w4a8_memory_query(C.byref(cfg), C.byref(mem)) == capi.RK_NPU_ERR_PARAM
+
+
+def test_w8_memory_queries_and_k_partition(lib):
+    """reference tests/test_quant_matmul.cpp:239-254 (M=8, N=K=96) and
+    src/rk_npu_quant_matmul.cpp:1131-1142 (partition policy)."""
+    from rknpu2_matmul_open_amd.ops import default_strategy
+    M, N, K = 8, 96, 96
+    for k_tile, waves in ((K, 1), (32, 3)):
+        s = default_strategy(capi.I8I8I32, M, N, K, k_tile=k_tile, n_tile=32 if k_tile == 32 else N)
+        if k_tile == 32:
+            s.npu_core_mask = 7
+        req = capi.WorkspaceRequirements()
+        assert lib.rk_npu_matmul_workspace_memory_query(C.byref(s), C.byref(req)) == 0
+        assert req.wave_count == waves
+        assert req.input_bytes == min(waves, 2) * M * ((min(k_tile, K) + 31) // 32 * 32)
+        assert req.output_bytes == min(waves, 3) * M * N * 4
+        assert req.buffer_count == 2 * waves + min(waves, 2) + min(waves, 3)
+        wc = capi.MatmulWeightConfig(K, N, k_tile)
+        wr = capi.WeightRequirements()
+        assert lib.rk_npu_i8i8i32_weights_memory_query(C.byref(wc), C.byref(wr)) == 0
+        assert (wr.packed_b_bytes, wr.scale_bytes, wr.buffer_count, wr.wave_count) == (K * N, 0, 1, waves)
+        assert lib.rk_npu_f16i8f16_weights_memory_query(C.byref(wc), C.byref(wr)) == 0
+        assert wr.scale_bytes == N * 4 and wr.bytes == K * N + N * 4
+    bad = default_strategy(capi.I8I8I32, M, N, K)
+    for field, v in (("k_tile", 0), ("k_tile", K + 1), ("n_tile", 3073), ("npu_core_mask", 5),
+                     ("cpu_threads", 2), ("cpu_core_mask", 0), ("a_layout", 4), ("c_layout", 3), ("op_kind", 9)):
+        s = default_strategy(capi.I8I8I32, M, N, K)
+        setattr(s, field, v)
+        req = capi.WorkspaceRequirements()
+        assert lib.rk_npu_matmul_workspace_memory_query(C.byref(s), C.byref(req)) == capi.RK_NPU_ERR_PARAM, field
+    q = lib.rk_npu_matmul_k_partition_query
+    assert q(0, 10, 10) == q(1, 0, 1) == q(1, 10, 11) == capi.RK_NPU_ERR_PARAM
+    assert q(4, 8192, 3100) == 0                          # M <= 4 always eligible
+    assert q(8, 8192, 2560) == capi.RK_NPU_ERR_PARAM      # split with a tile > 2048 not 1024-aligned
+    assert q(8, 8192, 3072) == 0
+    assert q(8, 3500, 3500) == capi.RK_NPU_ERR_PARAM      # a wave in (3072, 4096)
+    assert q(8, 4096, 4096) == 0 and q(128, 4096, 2048) == 0
+
+
+def test_open_without_device_fails_cleanly(lib):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    assert not lib.rk_npu_open(None)
+    assert not lib.rk_npu_open(b"/dev/dri/renderD128")
+    assert not lib.rk_npu_open(b"hip:")
+    # NULL handles are tolerated by every free / close
+    lib.rk_npu_close(None)
+    lib.rk_npu_iommu_domain_free(None)
+    lib.rk_npu_matmul_workspace_free(None)
+    lib.rk_npu_i8i8i32_weights_free(None)
+    lib.rk_npu_f16i8f16_weights_free(None)
+    lib.rk_npu_f32i8f32_weights_free(None)
+    lib.rk_npu_w4a8_weights_free(None)
+    lib.rk_npu_w4a8_workspace_free(None)
+    lib.rk_npu_moe_w8_weights_free(None)
+    lib.rk_npu_moe_w8_workspace_free(None)
+    assert lib.rk_npu_iommu_domain_id(None) == 0xFFFFFFFF
+    assert not lib.rk_npu_iommu_domain_create(None, 0)
+    assert lib.rk_npu_moe_w8_weights_device_bytes(None) == 0
+    # NULL handles in run calls are argument errors, not crashes
+    assert lib.rk_npu_i8i8i32_run(None, None, None, None) == capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_w4a8_run_f32(None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_moe_w8_run_f32(None, None, 1, None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
+
+
+def test_package_fails_loudly_without_the_library(monkeypatch, tmp_path):
+    monkeypatch.setenv("RK_NPU_MATMUL_LIB", str(tmp_path / "missing.so"))
+    monkeypatch.setattr(capi, "_LIB", None)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        capi.load_library()

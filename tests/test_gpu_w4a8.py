@@ -328,3 +328,29 @@ def test_config3_ffn_full(sess, oracle):
     finally:
         for o in (gws, dws, gw, dw):
             o.close()
+
+
+def test_k_tile_resolution_against_reference_golden(sess):
+    """tests/golden/i4_bounds.json holds what the reference's bound_i4_weights
+    answers for seeded code matrices (written by tests/golden/make_golden.py from
+    the compiled reference); weights_create must resolve the same tiles."""
+    import json
+    import os
+    from tests.golden.make_golden import i4_matrix
+    with open(os.path.join(os.path.dirname(__file__), "golden", "i4_bounds.json")) as f:
+        cases = json.load(f)
+    for case in cases:
+        B = i4_matrix(**case["recipe"])
+        K, N = B.shape
+        scale = np.ones(N, np.float32)
+        if case["auto_k_tile"] > 0:
+            w = ops.W4A8Weights(sess, B, scale, k_tile=0)
+            assert w.info.safe_k_tile == case["auto_k_tile"], case["recipe"]
+            assert w.info.config.k_tile == min(case["auto_k_tile"], 2048, (K + 31) // 32 * 32)
+            w.close()
+        for tile, ok in case["explicit"].items():
+            cfg = capi.I4WeightConfig(K, N, int(tile))
+            h = sess.lib.rk_npu_w4a8_weights_create(sess.domain, C.byref(cfg), capi.ptr(B), capi.ptr(scale))
+            assert bool(h) == bool(ok), (case["recipe"], tile)
+            if h:
+                sess.lib.rk_npu_w4a8_weights_free(h)
