@@ -210,6 +210,18 @@ def bench_c0(sess, ops, capi, workloads, steps, warmup):
     return out
 
 
+def bench_copy(sess, steps):
+    """Calibration for the rocprofv3 --pmc traffic figures: a plain device-to-device
+    copy of a known size (256 MiB read + 256 MiB written per launch)."""
+    nbytes = 256 << 20
+    src, dst = sess.empty_device(nbytes), sess.empty_device(nbytes)
+    us = sess.time_us(lambda: sess.lib.rk_npu_hip_copy(sess.ctx, dst, src, nbytes), steps, 2)
+    sess.free_device(src)
+    sess.free_device(dst)
+    return {"workload": "device-to-device copy, 268435456 B read + 268435456 B written per launch",
+            "GBps_read_plus_write": 2 * nbytes / us / 1e3}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -218,7 +230,7 @@ def main():
     ap.add_argument("--workload", default="c1", choices=["c1", "all"],
                     help="c1: headline line (+ c2 TOPS); all: also time configs 0, 3 and 4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c3", "c4"],
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c3", "c4", "copy"],
                     help="profiling aid: run one configuration's loop only")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -231,6 +243,10 @@ def main():
     arch, cus, khz = sess.device_info()
     log("device %s, %d CUs, %d MHz" % (arch, cus, khz // 1000))
 
+    if args.only == "copy":
+        print(json.dumps(bench_copy(sess, min(args.steps, 10))))
+        sess.close()
+        return
     if args.only:
         fn = {"c0": bench_c0, "c2": bench_c2, "c3": bench_c3, "c4": bench_c4}.get(args.only)
         res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)

@@ -45,6 +45,8 @@ void* rk_npu_hip_malloc(rk_npu_ctx* ctx, size_t bytes);
 void rk_npu_hip_free(rk_npu_ctx* ctx, void* ptr);
 int rk_npu_hip_upload(rk_npu_ctx* ctx, void* dst_device, const void* src_host, size_t bytes);
 int rk_npu_hip_download(rk_npu_ctx* ctx, void* dst_host, const void* src_device, size_t bytes);
+/* Device-to-device copy enqueued on the context's stream (not waited for). */
+int rk_npu_hip_copy(rk_npu_ctx* ctx, void* dst_device, const void* src_device, size_t bytes);
 
 /* Stream timing (HIP events on the context's stream). */
 typedef struct rk_npu_hip_event rk_npu_hip_event;

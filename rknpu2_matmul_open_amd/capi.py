@@ -204,6 +204,7 @@ _PROTOTYPES = {
     "rk_npu_hip_free": (None, [P, P]),
     "rk_npu_hip_upload": (C.c_int, [P, P, P, C.c_size_t]),
     "rk_npu_hip_download": (C.c_int, [P, P, P, C.c_size_t]),
+    "rk_npu_hip_copy": (C.c_int, [P, P, P, C.c_size_t]),
     "rk_npu_hip_event_create": (P, []),
     "rk_npu_hip_event_free": (None, [P]),
     "rk_npu_hip_event_record": (C.c_int, [P, P]),

@@ -255,6 +255,11 @@ int rk_npu_hip_download(rk_npu_ctx* ctx, void* dst_host, const void* src_device,
     return rkhost::map_error(rc);
 }
 
+int rk_npu_hip_copy(rk_npu_ctx* ctx, void* dst_device, const void* src_device, size_t bytes) {
+    if (!ctx || !dst_device || !src_device) return RK_NPU_ERR_PARAM;
+    return rkhost::map_error(rkh_d2d(ctx->stream, dst_device, src_device, bytes));
+}
+
 struct rk_npu_hip_event {
     void* handle = nullptr;
 };
