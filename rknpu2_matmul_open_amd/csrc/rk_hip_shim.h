@@ -163,6 +163,10 @@ typedef struct rkh_gemm_args {
     size_t ws_expert_stride; /* floats between experts in w_scale                 */
 } rkh_gemm_args;
 int rkh_gemm(void* stream, const rkh_gemm_args* args);
+/* quantize + GEMM as one request: for decode-sized M the quantization is fused
+ * into the GEMV kernel (one launch); otherwise the two kernels run back to back.
+ * Either way qargs->dst / qargs->scale end up holding the quantized rows. */
+int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_args* gargs);
 /* Bytes of split-K scratch rkh_gemm may use for a dense problem of this shape
  * (0 when it never splits K); the caller passes a zero-filled buffer of at
  * least this size in splitk_acc. */

@@ -416,10 +416,19 @@ constexpr int GEMV_WAVES = 8;
 constexpr int GEMV_UNROLL = 4;
 constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
 
-template <int MR, bool W4>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) {
+constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
+
+// QT: 0 = activations come quantized from the tiled buffer g.A;
+//     1 / 2 = fused per-token quantization of fp16 / fp32 rows q.src (every
+//     workgroup quantizes the few rows itself -- they are L2 hits after the first
+//     -- which saves a kernel launch per decode step; workgroup 0 also writes the
+//     scales and the tiled int8 copy that the two-kernel path would have left).
+template <int MR, bool W4, int QT>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
+    __shared__ uint32_t row_max[MR];
+    __shared__ float row_scale[MR];
     const int lane = lane_id(), wave = wave_id();
     const int half = lane >> 5;
     const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
@@ -433,15 +442,82 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) 
 
     const uint8_t* wbase = g.W + (W4 ? (size_t)p * (Kp / 64) * 1024 : (size_t)p * KB * 1024);
 
+    // Fused path: put the first batch of weight loads in flight before the
+    // quantization prologue so that its latency hides behind them.
+    v4i wpre[GEMV_UNROLL];
+    if constexpr (QT != 0) {
+        const int tiles = W4 ? Kp >> 6 : Kp >> 5;
+#pragma unroll
+        for (int u = 0; u < GEMV_UNROLL; ++u) {
+            const int tt = wave + u * GEMV_WAVES;
+            wpre[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                       wbase + (size_t)tt * 1024 + lane * 16))
+                                 : v4i{0, 0, 0, 0};
+        }
+    }
+    if constexpr (QT != 0) {
+        using T = typename std::conditional<QT == 1, uint16_t, float>::type;
+        const int t = threadIdx.x;
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+        if (t < MR) row_max[t] = 0u;
+        __syncthreads();
+        float v[GEMV_QCHUNKS][16];
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const T* row = static_cast<const T*>(q.src) + (size_t)m * K;
+                RowLoader<T>::load16(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0, v[i]);
+                float mx = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    mx = fmaxf(mx, fabsf(v[i][j]));
+                    bad |= not_finite(v[i][j]);
+                }
+                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
+            }
+        }
+        __syncthreads();
+        if (t < g.M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            if (p == 0 && q.scale) q.scale[t] = sc;
+        }
+        if (p == 0 && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
+        // zero the K padding of the staged rows
+        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) {
+            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const uint4 packed = quantize16<false>(v[i], 1.0f / row_scale[m]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
+                if (p == 0 && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            }
+        }
+        // a_scale of the epilogue comes from LDS in this path
+    }
+
     for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
         const int kc = min(kc_max, Kp - kc0);
         // stage activations: row-major [MR][kc] in LDS from the tiled buffer
         const int chunks = kc >> 4;
         if (kc0) __syncthreads();
-        for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
-            const int m = idx / chunks, c = idx - m * chunks;
-            const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-            *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+        if constexpr (QT == 0) {
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks;
+                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+            }
         }
         __syncthreads();
 
@@ -452,10 +528,14 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) 
 #pragma unroll
                 for (int u = 0; u < GEMV_UNROLL; ++u) {
                     const int tt = tb + u * GEMV_WAVES;
-                    w[u] = tt < tiles
-                               ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                     wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
-                               : v4i{0, 0, 0, 0};
+                    if (QT != 0 && tb == wave) {
+                        w[u] = wpre[u];
+                    } else {
+                        w[u] = tt < tiles
+                                   ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                         wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
+                                   : v4i{0, 0, 0, 0};
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < GEMV_UNROLL; ++u) {
@@ -479,10 +559,14 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) 
 #pragma unroll
                 for (int u = 0; u < GEMV_UNROLL; ++u) {
                     const int tt = tb + u * GEMV_WAVES;
-                    w[u] = tt < tiles
-                               ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                     wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
-                               : v4i{0, 0, 0, 0};
+                    if (QT != 0 && tb == wave) {
+                        w[u] = wpre[u];
+                    } else {
+                        w[u] = tt < tiles
+                                   ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                         wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
+                                   : v4i{0, 0, 0, 0};
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < GEMV_UNROLL; ++u) {
@@ -533,7 +617,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g) 
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
         const int n = block_first_col(p, g.interleave_F) + j;
         if (n < g.N)
-            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum, g.a_scale ? g.a_scale[m] : 1.0f,
+            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
+                      QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
                       g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
@@ -1195,13 +1280,40 @@ int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
 }
 
 template <int MR>
-int launch_gemv(hipStream_t st, const rkh_gemm_args& g) {
+int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
     const int pblocks = (int)(rkh_align_up(g.N, 32) / 32);
     const dim3 grid(pblocks), block(GEMV_WAVES * 64);
-    if (g.w_int4) hipLaunchKernelGGL((gemv_kernel<MR, true>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemv_kernel<MR, false>), grid, block, 0, st, g);
+    const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
+    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+#define RK_GEMV(W4, QT) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT>), grid, block, 0, st, g, q)
+    if (g.w_int4) {
+        if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
+    } else {
+        if (qt == 0) RK_GEMV(false, 0); else if (qt == 1) RK_GEMV(false, 1); else RK_GEMV(false, 2);
+    }
+#undef RK_GEMV
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
+}
+
+int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    if (g.M == 1) return launch_gemv<1>(st, g, fuse);
+    if (g.M == 2) return launch_gemv<2>(st, g, fuse);
+    if (g.M <= 4) return launch_gemv<4>(st, g, fuse);
+    return launch_gemv<8>(st, g, fuse);
+}
+
+// The decode path can quantize inside the GEMV when the rows fit the kernel's
+// LDS staging and per-thread register cache.
+bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g) {
+    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU || q.dest_rows) return false;
+    if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
+    if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
+    const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
+    const long kp = (long)rkh_align_up(g.K, RKH_K_ALIGN);
+    if (kp * mr > GEMV_LDS_BYTES) return false;
+    const long chunks = (long)g.M * ((g.K + 15) / 16);
+    return chunks <= (long)GEMV_QCHUNKS * GEMV_WAVES * 64;
 }
 
 int g_fail_malloc_after = 0;
@@ -1387,12 +1499,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     const rkh_gemm_args& g = *args;
     hipStream_t st = (hipStream_t)stream;
     const bool grouped = g.blk_expert != nullptr;
-    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) {
-        if (g.M == 1) return launch_gemv<1>(st, g);
-        if (g.M == 2) return launch_gemv<2>(st, g);
-        if (g.M <= 4) return launch_gemv<4>(st, g);
-        return launch_gemv<8>(st, g);
-    }
+    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) return dispatch_gemv(st, g, nullptr);
     if (grouped) return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, 1);
     DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
     // Tuning aid: RK_NPU_HIP_GEMM_PLAN="rows:ksplit" forces the workgroup tile
@@ -1414,6 +1521,12 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     if (bm == 128) return launch_gemm_cfg<2, 4, 2, 2, 2>(st, g, ksplit);
     if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2, 2>(st, g, ksplit);
     return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, ksplit);
+}
+
+int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_args* gargs) {
+    if (gemv_can_fuse(*qargs, *gargs)) return dispatch_gemv((hipStream_t)stream, *gargs, qargs);
+    const int rc = rkh_quant_rows(stream, qargs);
+    return rc ? rc : rkh_gemm(stream, gargs);
 }
 
 int rkh_moe_route(void* stream, const rkh_moe_route_args* args) {

@@ -124,46 +124,44 @@ struct rk_npu_matmul_workspace {
 
 namespace {
 
-// Enqueue quantize + GEMM on the context's stream.  dA / dC are device
-// pointers (the workspace's own staging buffers or the caller's).
-int enqueue_gemm(rk_npu_matmul_workspace* ws, const Weights& w, void* dC);
-
-int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA,
-            const float* a_scale_static_dev, void* dC) {
+rkh_gemm_args gemm_args(rk_npu_matmul_workspace* ws, const Weights& w, void* dC) {
     const auto& s = ws->strategy;
-    void* stream = ws->owner.ctx->stream;
-    rkh_quant_args q{};
-    q.src = dA;
-    q.in_dtype = ws->t.in_dtype;
-    q.mode = ws->t.quant == 0 ? RKH_Q_COPY_I8 : ws->t.quant == 1 ? RKH_Q_W8_DYNAMIC : RKH_Q_W8_STATIC;
-    q.M = s.M;
-    q.K = s.K;
-    (void)a_scale_static_dev; // static scales are staged in the workspace's a_scale
-    q.scale = ws->t.quant == 0 ? nullptr : ws->a_scale.as<float>();
-    q.dst = ws->a_tiled.as<>();
-    int rc = rkh_quant_rows(stream, &q);
-    if (rc) return map_error(rc);
-    return enqueue_gemm(ws, w, dC);
-}
-
-// GEMV / GEMM stage on the activations already quantized into the workspace.
-int enqueue_gemm(rk_npu_matmul_workspace* ws, const Weights& w, void* dC) {
-    const auto& s = ws->strategy;
-    void* stream = ws->owner.ctx->stream;
-    struct { float* scale; } q{ws->a_scale.as<float>()};
     rkh_gemm_args g{};
     g.A = ws->a_tiled.as<>();
     g.W = w.tiled.as<>();
     g.M = s.M;
     g.N = s.N;
     g.K = s.K;
-    g.a_scale = q.scale;
+    g.a_scale = ws->a_scale.as<float>();
     g.w_scale = w.w_scale.as<float>();
     g.epilogue = ws->t.out_epi;
     g.C = dC;
     g.ldc = s.N;
     g.splitk_acc = ws->splitk ? ws->splitk.as<int32_t>() : nullptr;
-    return map_error(rkh_gemm(stream, &g));
+    return g;
+}
+
+// Enqueue quantize + GEMM on the context's stream (one fused kernel for
+// decode-sized M).  dA / dC are device pointers; static scales are expected in
+// the workspace's a_scale buffer.
+int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA, void* dC) {
+    const auto& s = ws->strategy;
+    rkh_quant_args q{};
+    q.src = dA;
+    q.in_dtype = ws->t.in_dtype;
+    q.mode = ws->t.quant == 0 ? RKH_Q_COPY_I8 : ws->t.quant == 1 ? RKH_Q_W8_DYNAMIC : RKH_Q_W8_STATIC;
+    q.M = s.M;
+    q.K = s.K;
+    q.scale = ws->t.quant == 0 ? nullptr : ws->a_scale.as<float>();
+    q.dst = ws->a_tiled.as<>();
+    const rkh_gemm_args g = gemm_args(ws, w, dC);
+    return map_error(rkh_quant_gemm(ws->owner.ctx->stream, &q, &g));
+}
+
+// GEMV / GEMM stage on the activations already quantized into the workspace.
+int enqueue_gemm(rk_npu_matmul_workspace* ws, const Weights& w, void* dC) {
+    const rkh_gemm_args g = gemm_args(ws, w, dC);
+    return map_error(rkh_gemm(ws->owner.ctx->stream, &g));
 }
 
 int check_run(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kind kind,
@@ -191,7 +189,7 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
         rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         if (!rc && ws->t.quant == 2)
             rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(), a_scale, (size_t)s.M * sizeof(float)));
-        if (!rc) rc = enqueue(ws, *w, ws->a_raw.as<>(), ws->a_scale.as<float>(), ws->c_out.as<>());
+        if (!rc) rc = enqueue(ws, *w, ws->a_raw.as<>(), ws->c_out.as<>());
         if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }
     const int wait = map_error(rkh_sync(ctx->stream));
@@ -205,7 +203,7 @@ int run_device(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_k
     BusyLock lock(ws->busy);
     if (!lock) return RK_NPU_ERR_BUSY;
     std::lock_guard<std::mutex> submit(ws->owner.ctx->submit_mutex);
-    return enqueue(ws, *w, dA, nullptr, dC);
+    return enqueue(ws, *w, dA, dC);
 }
 
 // reference src/rk_npu_kn_plan.cpp:43-116 (logical RK3588 payload sizes)

@@ -191,6 +191,8 @@ int validate(const rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, cons
 enum class Out { F32, F16, I32, SwiGLU };
 int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
                  bool collect);
+rkh_gemm_args gemm_args(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
+                        bool collect);
 
 // quantize (or re-quantize with reused row maxima) + GEMM.  `scale_source`
 // non-null: A is the fp32 middle of that workspace's SwiGLU run and its
@@ -215,19 +217,23 @@ int enqueue(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void*
     } else {
         q.mode = RKH_Q_W4A8;
     }
-    int rc = rkh_quant_rows(stream, &q);
-    if (rc) return map_error(rc);
-    if (timer) timer->mark();
-    rc = enqueue_gemm(ws, w, dC, out, collect);
-    if (timer) timer->mark();
-    return rc;
+    const rkh_gemm_args g = gemm_args(ws, w, dC, out, collect);
+    int rc;
+    if (timer) {
+        // separate launches so the stage timer can tell the two apart
+        rc = rkh_quant_rows(stream, &q);
+        timer->mark();
+        if (!rc) rc = rkh_gemm(stream, &g);
+        timer->mark();
+    } else {
+        rc = rkh_quant_gemm(stream, &q, &g);
+    }
+    return map_error(rc);
 }
 
-// GEMV / GEMM stage on the activations already quantized into the workspace.
-int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
-                 bool collect) {
+rkh_gemm_args gemm_args(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
+                        bool collect) {
     const auto& c = ws->config;
-    void* stream = ws->owner.ctx->stream;
     rkh_gemm_args g{};
     g.A = ws->a_tiled.as<>();
     g.W = w->tiled.as<>();
@@ -250,7 +256,14 @@ int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* 
         g.row_max_bits = collect ? ws->row_max.as<uint32_t>() : nullptr;
         break;
     }
-    return map_error(rkh_gemm(stream, &g));
+    return g;
+}
+
+// GEMV / GEMM stage on the activations already quantized into the workspace.
+int enqueue_gemm(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, void* dC, Out out,
+                 bool collect) {
+    const rkh_gemm_args g = gemm_args(ws, w, dC, out, collect);
+    return map_error(rkh_gemm(ws->owner.ctx->stream, &g));
 }
 
 void fill_timings(rk_npu_w4a8_timings* t, StageTimer& timer, int first_mark, bool scanned,
