@@ -624,12 +624,6 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
 }
 
 // ------------------------------------------------------------------ GEMM
-// Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn),
-// each wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is 64 deep:
-// the step's A tiles (BM/32 x 2 KiB) and W tiles are copied global -> register
-// -> LDS as whole 1 KiB tiles, so LDS reads are linear 16 bytes per lane
-// (bank-conflict free) and land directly in MFMA operand order.  Two LDS
-// buffers; the loads of step i+1 are issued before the MFMAs of step i.
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
     // contiguous range of logical tiles so neighbours share its L2.
@@ -705,29 +699,36 @@ __device__ __forceinline__ void store_tile(T* C, int ldc, int m0, int n0, int m_
     }
 }
 
-// Dequantize and store one accumulator tile whose physical column block is p.
+// Weight scales of the 16 columns a lane owns in the tile whose first logical
+// column is n0 (zero beyond the matrix).
+__device__ __forceinline__ void load_col_scales(float* ws, const float* w_scale, int n0, int n_limit,
+                                                int lane) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int n = n0 + tile_col(r, lane);
+        ws[r] = n < n_limit ? w_scale[n] : 0.0f;
+    }
+}
+
+// Dequantize and store one accumulator tile whose physical column block is p;
+// as / ws are the lane's row scale and its 16 column scales.
 template <int EPI>
-__device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i& acc, int m0, int p,
-                                              int lane, const float* a_scale, const float* w_scale,
-                                              int m_limit, uint8_t* stage_lds) {
+__device__ __forceinline__ void epilogue_tile_scaled(const rkh_gemm_args& g, const v16i& acc, int m0,
+                                                     int p, int lane, float as, const float* ws,
+                                                     int m_limit, uint8_t* stage_lds) {
     // padding blocks beyond the matrix hold zeros; with interleaved columns their
     // logical index would alias a real column, so test the block itself
     if (g.interleave_F ? p >= g.N / 32 : p * 32 >= g.N) return;
     const int n0 = block_first_col(p, g.interleave_F);
-    const int m = m0 + (lane & 31);
     if constexpr (EPI == RKH_EPI_I32) {
         int vals[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) vals[r] = acc[r];
         store_tile<int>(static_cast<int*>(g.C), g.ldc, m0, n0, m_limit, g.N, vals, stage_lds, lane);
     } else {
-        const float as = m < m_limit ? a_scale[m] : 0.0f;
         float y[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int n = n0 + tile_col(r, lane);
-            y[r] = dequant(acc[r], as, n < g.N ? w_scale[n] : 0.0f);
-        }
+        for (int r = 0; r < 16; ++r) y[r] = dequant(acc[r], as, ws[r]);
         if constexpr (EPI == RKH_EPI_F16) {
             __half h[16];
 #pragma unroll
@@ -739,8 +740,47 @@ __device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i
     }
 }
 
+template <int EPI>
+__device__ __forceinline__ void epilogue_tile(const rkh_gemm_args& g, const v16i& acc, int m0, int p,
+                                              int lane, const float* a_scale, const float* w_scale,
+                                              int m_limit, uint8_t* stage_lds) {
+    if (g.interleave_F ? p >= g.N / 32 : p * 32 >= g.N) return;
+    float as = 0.0f, ws[16];
+    if constexpr (EPI != RKH_EPI_I32) {
+        const int m = m0 + (lane & 31);
+        as = m < m_limit ? a_scale[m] : 0.0f;
+        load_col_scales(ws, w_scale, block_first_col(p, g.interleave_F), g.N, lane);
+    }
+    epilogue_tile_scaled<EPI>(g, acc, m0, p, lane, as, ws, m_limit, stage_lds);
+}
+
 // gate tile (physical block p, even) + up tile (p + 1) -> 32 columns of the
-// middle and one partial row maximum per (row, 32-column block).
+// middle and one partial row maximum per (row, 32-column block).  wsg / wsu are
+// the lane's gate and up column scales.
+__device__ __forceinline__ void epilogue_swiglu_scaled(const rkh_gemm_args& g, const v16i& gate,
+                                                       const v16i& up, int m0, int p, int lane,
+                                                       float as, const float* wsg, const float* wsu,
+                                                       int m_limit, uint8_t* stage_lds) {
+    const int F = g.interleave_F;
+    const int n0 = (p >> 1) * 32;
+    if (n0 >= F) return;
+    const int m = m0 + (lane & 31);
+    float y[16];
+    uint32_t bits = 0;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float gf = dequant(gate[r], as, wsg[r]);
+        const float uf = dequant(up[r], as, wsu[r]);
+        y[r] = __fmul_rn(silu_poly(gf), uf);
+        bits = max(bits, __float_as_uint(y[r]) & 0x7fffffffu);
+    }
+    store_tile<float>(static_cast<float*>(g.C), g.ldc, m0, n0, m_limit, F, y, stage_lds, lane);
+    if (g.row_max_bits) {
+        bits = max(bits, (uint32_t)__shfl_xor((int)bits, 32));
+        if (lane < 32 && m < m_limit) g.row_max_bits[(size_t)m * (F / 32) + (p >> 1)] = bits;
+    }
+}
+
 __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v16i& gate,
                                                 const v16i& up, int m0, int p, int lane,
                                                 const float* a_scale, const float* w_scale,
@@ -750,21 +790,10 @@ __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v1
     if (n0 >= F) return;
     const int m = m0 + (lane & 31);
     const float as = m < m_limit ? a_scale[m] : 0.0f;
-    float y[16];
-    uint32_t bits = 0;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int n = n0 + tile_col(r, lane);
-        const float gf = dequant(gate[r], as, w_scale[n]);
-        const float uf = dequant(up[r], as, w_scale[F + n]);
-        y[r] = __fmul_rn(silu_poly(gf), uf);
-        bits = max(bits, __float_as_uint(y[r]) & 0x7fffffffu);
-    }
-    store_tile<float>(static_cast<float*>(g.C), g.ldc, m0, n0, m_limit, F, y, stage_lds, lane);
-    if (g.row_max_bits) {
-        bits = max(bits, (uint32_t)__shfl_xor((int)bits, 32));
-        if (lane < 32 && m < m_limit) g.row_max_bits[(size_t)m * (F / 32) + (p >> 1)] = bits;
-    }
+    float wsg[16], wsu[16];
+    load_col_scales(wsg, w_scale, n0, F, lane);
+    load_col_scales(wsu, w_scale + F, n0, F, lane);
+    epilogue_swiglu_scaled(g, gate, up, m0, p, lane, as, wsg, wsu, m_limit, stage_lds);
 }
 
 // Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn), each
@@ -1051,6 +1080,253 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
     }
 }
 
+// ---- 128 x 256 tile, waves split K ------------------------------------------
+// The large dense tile.  Eight waves = 4 column groups (wn) x 2 k-halves (wk):
+// wave (wn, wk) accumulates the whole 128 x 64 strip of column group wn, but
+// only over k-tile wk of every 64-deep K step; the two halves are summed once,
+// through LDS, before the epilogue.  Compared with splitting the rows between
+// the two waves that share a SIMD, no weight byte is loaded (or unpacked) by
+// two waves, which takes a third off the traffic through the vector memory
+// path -- the resource this kernel runs out of first -- and halves the int4
+// unpack work, at the price of 128 accumulator registers per lane.
+//
+// Per K step a wave issues: its 1 KiB share of the step's activation tile
+// (global -> registers, NS-1 steps ahead; registers -> LDS two steps ahead),
+// the weight words of its k-tile for its two column blocks (global ->
+// registers, NS-1 steps ahead: 8 bytes per lane for int4, 16 for int8), four
+// 16-byte LDS fragment reads for the NEXT step, eight MFMAs of THIS step and,
+// for int4, the unpack of the next step's operands in the MFMA shadow.  Three
+// LDS buffers and one workgroup barrier per step: step s+2 is written while
+// step s+1 is read and step s is multiplied.
+template <bool W4, int EPI>
+__global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
+    constexpr int NW = 8, TM = 4, TN = 2, NS = 6, NB = 3;
+    constexpr int BM = 128, BN = 256;
+    constexpr int BUF = 8 * 1024;                         // one step of activations
+    constexpr int XCH = NW * 2 * 16 * 64 * 4;             // k-half exchange, one round
+    constexpr int LDS_BYTES = XCH > NB * BUF ? XCH : NB * BUF;
+    static_assert(NS % NB == 0 && NS % 2 == 0, "slot -> buffer / fragment parity must be compile-time");
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int wn = wave & 3, wk = wave >> 2;
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int ksteps = KB / 2;
+
+    // ---- tile assignment: XCD-contiguous ranges, 4 row blocks per column sweep
+    const int total = mblocks * nblocks;
+    const int tile = xcd_remap(blockIdx.x, total);
+    constexpr int GM = 4;
+    const int per_group = GM * nblocks;
+    const int group = tile / per_group;
+    const int first_m = group * GM;
+    const int gm = min(mblocks - first_m, GM);
+    const int in_group = tile - group * per_group;
+    const int mblk = first_m + in_group % gm;
+    const int nblk = in_group / gm;
+
+    // ---- sources
+    // activation chunk of this wave: row block wave / 2, k-tile wave % 2
+    // (wave-uniform base pointers advance on the scalar unit; lanes add a constant offset)
+    const uint8_t* asrc = g.A + ((size_t)(mblk * 4 + (wave >> 1)) * KB + (wave & 1)) * 1024;
+    const uint8_t* wsrc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int pb = nblk * 8 + wn * TN + j;
+        wsrc[j] = W4 ? g.W + (size_t)pb * (KB / 2) * 1024 + wk * 8 : g.W + ((size_t)pb * KB + wk) * 1024;
+    }
+    const unsigned lane_off = lane * 16;
+    constexpr int A_STEP = 2048, W_STEP = W4 ? 1024 : 2048;
+    using wraw_t = typename std::conditional<W4, v2i, v4i>::type;
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    v4i stage[NS];        // activation prefetch ring
+    wraw_t wring[NS][TN]; // weight prefetch ring
+    v4i afr[2][TM];       // activation fragments, this step / next step
+    v4i wop[2][TN];       // int4 only: unpacked operands, this step / next step
+
+    auto load_a = [&](v4i& reg) {
+        reg = *reinterpret_cast<const v4i*>(asrc + lane_off);
+        asrc += A_STEP;
+    };
+    auto load_w = [&](wraw_t* regs) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            regs[j] = *reinterpret_cast<const wraw_t*>(wsrc[j] + lane_off);
+            wsrc[j] += W_STEP;
+        }
+    };
+    auto store_a = [&](const v4i& reg, int buf) {
+        *reinterpret_cast<v4i*>(lds_raw + buf * BUF + wave * 1024 + lane * 16) = reg;
+    };
+    auto read_a = [&](v4i* dst, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            dst[i] = *reinterpret_cast<const v4i*>(lds_raw + buf * BUF + (i * 2 + wk) * 1024 + lane * 16);
+    };
+    auto unpack = [&](v4i* dst, const wraw_t* raw) {
+        if constexpr (W4) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                dst[j].x = (raw[j].x << 4) & 0xF0F0F0F0;
+                dst[j].y = raw[j].x & 0xF0F0F0F0;
+                dst[j].z = (raw[j].y << 4) & 0xF0F0F0F0;
+                dst[j].w = raw[j].y & 0xF0F0F0F0;
+            }
+        }
+    };
+
+    // SLOT = s % NS: ring stage, LDS buffer SLOT % NB, fragment set SLOT % 2.
+    // n1 / n2 / nf: steps s+1 / s+2 / s+NS-1 exist.
+    auto k_step = [&](auto slot_tag, auto n1, auto n2, auto nf) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        constexpr int F = SLOT & 1;
+        if (nf) load_a(stage[(SLOT + NS - 1) % NS]);
+        if (nf) load_w(wring[(SLOT + NS - 1) % NS]);
+        if (n1) read_a(afr[F ^ 1], (SLOT + 1) % NB);
+        if (n2) store_a(stage[(SLOT + 2) % NS], (SLOT + 2) % NB);
+        if constexpr (W4) {
+            if (n1) unpack(wop[F ^ 1], wring[(SLOT + 1) % NS]);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                if constexpr (W4)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop[F][j], afr[F][i], acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[SLOT][j], afr[F][i], acc[i][j], 0, 0, 0);
+            }
+#pragma unroll
+        for (int q = 0; q < TM * TN; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
+            if (W4) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);         // unpack in its shadow
+            if (q < 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // global loads
+            if (q < 5) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // LDS reads / write
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();
+    };
+    using T_ = std::true_type;
+
+    // prologue: NS-1 steps in flight; steps 0 and 1 in LDS; step 0 in registers
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i) {
+        if (i < ksteps) {
+            load_a(stage[i]);
+            load_w(wring[i]);
+        }
+    }
+    store_a(stage[0], 0);
+    if (ksteps > 1) store_a(stage[1], 1);
+    lds_barrier();
+    read_a(afr[0], 0);
+    unpack(wop[0], wring[0]);
+
+    int s = 0;
+    for (; s + 2 * NS - 2 < ksteps; s += NS)
+        static_for<NS>([&](auto slot) { k_step(slot, T_{}, T_{}, T_{}); });
+    for (; s < ksteps; s += NS)
+        static_for<NS>([&](auto slot) {
+            constexpr int SL = decltype(slot)::value;
+            if (s + SL < ksteps)
+                k_step(slot, s + SL + 1 < ksteps, s + SL + 2 < ksteps, s + SL + NS - 1 < ksteps);
+        });
+
+    // ---- epilogue.  Scales first (their latency hides behind the exchange):
+    // after the exchange this wave owns row blocks 2*wk, 2*wk+1 of its strip.
+    const int m_limit = g.M;
+    float as[2] = {0.0f, 0.0f}, ws[TN][16];
+    if constexpr (EPI != RKH_EPI_I32) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) {
+            const int m = mblk * BM + (wk * 2 + ii) * 32 + (lane & 31);
+            as[ii] = m < m_limit ? g.a_scale[m] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int pb = nblk * 8 + wn * TN + j;
+            if constexpr (EPI == RKH_EPI_SWIGLU) {
+                // pb even = gate, odd = up block of middle columns (pb / 2) * 32
+                const int F = g.interleave_F;
+                load_col_scales(ws[j], g.w_scale + (j ? F : 0), (pb >> 1) * 32, F, lane);
+            } else {
+                const bool live = g.interleave_F ? pb < g.N / 32 : pb * 32 < g.N;
+                load_col_scales(ws[j], g.w_scale, block_first_col(pb, g.interleave_F), live ? g.N : 0, lane);
+            }
+        }
+    }
+    // Sum the two k-halves: each wave hands the partner's row blocks over and
+    // adds what it receives, one column block per round.  All fragment reads of
+    // the K loop completed before its last barrier, so LDS is free.  The half
+    // index is a template tag so that accumulator registers are indexed with
+    // constants.
+    auto finish = [&](auto wk_tag) {
+        constexpr int WK = decltype(wk_tag)::value;
+        int* xch = reinterpret_cast<int*>(lds_raw);
+        const int partner = wave ^ 4;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii) {
+                const v16i& give = acc[(WK ^ 1) * 2 + ii][j];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<v4i*>(xch + (((wave * 2 + ii) * 4 + q) * 64 + lane) * 4) =
+                        v4i{give[q * 4], give[q * 4 + 1], give[q * 4 + 2], give[q * 4 + 3]};
+            }
+            lds_barrier();
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii) {
+                v16i& keep = acc[WK * 2 + ii][j];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const v4i got =
+                        *reinterpret_cast<const v4i*>(xch + (((partner * 2 + ii) * 4 + q) * 64 + lane) * 4);
+                    keep[q * 4] += got.x;
+                    keep[q * 4 + 1] += got.y;
+                    keep[q * 4 + 2] += got.z;
+                    keep[q * 4 + 3] += got.w;
+                }
+            }
+            lds_barrier();
+        }
+        uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) {
+            constexpr int i0 = WK * 2;
+            const int m0 = mblk * BM + (i0 + ii) * 32;
+            if constexpr (W4) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i0 + ii][j][r] >>= 4;
+            }
+            const int pb0 = nblk * 8 + wn * TN;
+            if constexpr (EPI == RKH_EPI_SWIGLU) {
+                epilogue_swiglu_scaled(g, acc[i0 + ii][0], acc[i0 + ii][1], m0, pb0, lane, as[ii], ws[0], ws[1],
+                                       m_limit, stage_lds);
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    epilogue_tile_scaled<EPI>(g, acc[i0 + ii][j], m0, pb0 + j, lane, as[ii], ws[j], m_limit,
+                                              stage_lds);
+            }
+        }
+    };
+    if (wk == 0) finish(std::integral_constant<int, 0>{});
+    else finish(std::integral_constant<int, 1>{});
+}
+
 // Epilogue over the split-K scratch matrix; re-zeroes what it consumed so the
 // scratch is clean for the next call.
 __global__ __launch_bounds__(256) void splitk_epilogue_kernel(rkh_gemm_args g, int ld) {
@@ -1276,6 +1552,25 @@ int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
         hipLaunchKernelGGL(splitk_epilogue_kernel, egrid, dim3(256), 0, st, g, ld);
         RKH_CHECK(hipGetLastError());
     }
+    return RKH_OK;
+}
+
+int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g) {
+    const int mblocks = (g.M + 127) / 128, nblocks = (g.N + 255) / 256;
+    const dim3 grid(mblocks * nblocks), block(512);
+#define RK_WK(W4, EPI) hipLaunchKernelGGL((gemm_wk_kernel<W4, EPI>), grid, block, 0, st, g, mblocks, nblocks)
+#define RK_WK_EPI(W4)                                           \
+    switch (g.epilogue) {                                       \
+    case RKH_EPI_I32: RK_WK(W4, RKH_EPI_I32); break;            \
+    case RKH_EPI_F16: RK_WK(W4, RKH_EPI_F16); break;            \
+    case RKH_EPI_F32: RK_WK(W4, RKH_EPI_F32); break;            \
+    case RKH_EPI_SWIGLU: RK_WK(W4, RKH_EPI_SWIGLU); break;      \
+    default: return RKH_ERR_RUNTIME;                            \
+    }
+    if (g.w_int4) { RK_WK_EPI(true) } else { RK_WK_EPI(false) }
+#undef RK_WK_EPI
+#undef RK_WK
+    RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
 
@@ -1518,6 +1813,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
         ksplit = 1;
     }
     const int bm = plan.bm;
+    if (bm == 128 && ksplit == 1) return launch_gemm_wk(st, g);
     if (bm == 128) return launch_gemm_cfg<2, 4, 2, 2, 2>(st, g, ksplit);
     if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2, 2>(st, g, ksplit);
     return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, ksplit);
