@@ -136,7 +136,7 @@ def bench_c2(sess, ops, capi, workloads, steps, warmup):
     ops_count = 2.0 * M * K * N
     out = {"workload": "c2: w4a8 prefill GEMM M=2048 K=4096 N=4096, fp16 in/out, seeds 4/5",
            "tops": ops_count / step_us / 1e6, "ms_per_step": step_us / 1e3,
-           "roofline": {"bound": "mfma", "kernel": "gemm_kernel<2,2,2,4,int4>",
+           "roofline": {"bound": "mfma", "kernel": "gemm_wk_kernel<int4,f16> (128x256 tile, waves split K)",
                         "achieved": ops_count / kernel_us / 1e6, "peak": INT8_PEAK_TOPS,
                         "unit": "TOP/s", "frac": ops_count / kernel_us / 1e6 / INT8_PEAK_TOPS,
                         "kernel_us": kernel_us, "traffic": _traffic("gemm_c2")}}

@@ -1083,30 +1083,57 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 // ---- 128 x 256 tile, waves split K ------------------------------------------
 // The large dense tile.  Eight waves = 4 column groups (wn) x 2 k-halves (wk):
 // wave (wn, wk) accumulates the whole 128 x 64 strip of column group wn, but
-// only over k-tile wk of every 64-deep K step; the two halves are summed once,
-// through LDS, before the epilogue.  Compared with splitting the rows between
-// the two waves that share a SIMD, no weight byte is loaded (or unpacked) by
-// two waves, which takes a third off the traffic through the vector memory
-// path -- the resource this kernel runs out of first -- and halves the int4
-// unpack work, at the price of 128 accumulator registers per lane.
+// only over k-tile wk of every 64-deep K sub-step; the two halves are summed
+// once, through LDS, before the epilogue.  Compared with splitting the rows
+// between the two waves that share a SIMD, no weight byte is loaded (or
+// unpacked) by two waves, which takes a third off the traffic through the
+// vector memory path and halves the int4 unpack work, at the price of 128
+// accumulator registers per lane.
 //
-// Per K step a wave issues: its 1 KiB share of the step's activation tile
-// (global -> registers, NS-1 steps ahead; registers -> LDS two steps ahead),
-// the weight words of its k-tile for its two column blocks (global ->
-// registers, NS-1 steps ahead: 8 bytes per lane for int4, 16 for int8), four
-// 16-byte LDS fragment reads for the NEXT step, eight MFMAs of THIS step and,
-// for int4, the unpack of the next step's operands in the MFMA shadow.  Three
-// LDS buffers and one workgroup barrier per step: step s+2 is written while
-// step s+1 is read and step s is multiplied.
+// Activations: every wave copies its 1 KiB share of a sub-step's 128 x 64 tile
+// global -> LDS directly (no registers), WK_D sub-steps ahead, into a ring of
+// WK_NBUF buffers.  Weights: global -> registers, WK_NSW-1 sub-steps ahead (8
+// bytes per lane for int4, 16 for int8).  Each sub-step a wave also reads the
+// four 16-byte activation fragments of the NEXT sub-step and issues eight
+// MFMAs, with the int4 unpack of the next operands in their shadow.
+//
+// A workgroup barrier costs roughly a third of a sub-step's MFMA time (the
+// matrix pipes drain while the waves meet), so there is only one every WK_G
+// sub-steps.
+//
+// All loads of the loop are inline assembly and every wait is explicit.  (The
+// compiler's own bookkeeping orders each LDS read and each register load after
+// ALL outstanding global -> LDS copies, which would undo the prefetch.)  The
+// waits rely on vector memory loads completing in issue order and on every
+// sub-step issuing exactly 1 + TN loads -- copy first, then weights -- also
+// beyond the end of K, where the source pointers simply stop advancing (those
+// loads hit the L1 and their results are never used).  With that:
+//  * weights of sub-step s+1 were issued at s+1-(NSW-1); (NSW-2) * (1+TN)
+//    loads have been issued since, hence vmcnt((NSW-2) * (1+TN));
+//  * publication: the fragments read during sub-steps B+1..B+G (B = last
+//    sub-step before a barrier) belong to sub-steps <= B+G+1; their copies
+//    were issued at sub-steps <= B+G+1-D, before the weights a wave waits for
+//    during sub-step B, so they have landed when it reaches the barrier
+//    (needs D >= NSW + G - 1);
+//  * reuse: the copy issued at sub-step s overwrites the buffer that held
+//    sub-step s+D-NBUF, last read at sub-step s+D-NBUF-1 <= s-G-1, which is
+//    before the latest barrier (needs NBUF >= D + G).
+constexpr int WK_NSW = 8, WK_NBUF = 16, WK_G = 4, WK_D = 12, WK_BUF = 8 * 1024;
+constexpr int WK_LDS_BYTES = WK_NBUF * WK_BUF;
+static_assert(WK_D >= WK_NSW + WK_G - 1 && WK_NBUF >= WK_D + WK_G, "see the ordering rules above");
+
+typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm" // m0 is set and clobbered on purpose below
 template <bool W4, int EPI>
 __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
-    constexpr int NW = 8, TM = 4, TN = 2, NS = 6, NB = 3;
-    constexpr int BM = 128, BN = 256;
-    constexpr int BUF = 8 * 1024;                         // one step of activations
-    constexpr int XCH = NW * 2 * 16 * 64 * 4;             // k-half exchange, one round
-    constexpr int LDS_BYTES = XCH > NB * BUF ? XCH : NB * BUF;
-    static_assert(NS % NB == 0 && NS % 2 == 0, "slot -> buffer / fragment parity must be compile-time");
-    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    constexpr int TM = 4, TN = 2, NSW = WK_NSW, NBUF = WK_NBUF, G = WK_G, D = WK_D;
+    constexpr int BM = 128, BUF = WK_BUF;
+    constexpr int UNR = 16; // sub-steps per unrolled trip: multiple of NSW, NBUF, G and 2
+    constexpr int LPS = 1 + TN; // loads per sub-step and wave
+    static_assert(UNR % NSW == 0 && UNR % NBUF == 0 && UNR % G == 0, "slot arithmetic must be compile-time");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[]; // WK_LDS_BYTES
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
@@ -1127,9 +1154,8 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     const int mblk = first_m + in_group % gm;
     const int nblk = in_group / gm;
 
-    // ---- sources
+    // ---- sources: wave-uniform base pointers (scalar registers) + a constant lane offset.
     // activation chunk of this wave: row block wave / 2, k-tile wave % 2
-    // (wave-uniform base pointers advance on the scalar unit; lanes add a constant offset)
     const uint8_t* asrc = g.A + ((size_t)(mblk * 4 + (wave >> 1)) * KB + (wave & 1)) * 1024;
     const uint8_t* wsrc[TN];
 #pragma unroll
@@ -1140,6 +1166,12 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     const unsigned lane_off = lane * 16;
     constexpr int A_STEP = 2048, W_STEP = W4 ? 1024 : 2048;
     using wraw_t = typename std::conditional<W4, v2i, v4i>::type;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds_raw;
+    const uint32_t copy_dst = lds_base + wave * 1024; // this wave's chunk inside buffer 0
+    // LDS byte addresses of this lane's fragment of row block 0 in buffers 0 and 8
+    uint32_t frag_lo = lds_base + wk * 1024 + lane * 16;
+    uint32_t frag_hi = frag_lo + 8 * BUF;
+    int a_left = ksteps - 1, w_left = ksteps - 1; // how often the sources may still advance
 
     v16i acc[TM][TN];
 #pragma unroll
@@ -1149,101 +1181,98 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    v4i stage[NS];        // activation prefetch ring
-    wraw_t wring[NS][TN]; // weight prefetch ring
-    v4i afr[2][TM];       // activation fragments, this step / next step
-    v4i wop[2][TN];       // int4 only: unpacked operands, this step / next step
+    wraw_t wring[NSW][TN]; // weight prefetch ring
+    v4i afr[2][TM];        // activation fragments, this sub-step / next
+    v4i wop[2][TN];        // int4 only: unpacked operands, this sub-step / next
 
-    auto load_a = [&](v4i& reg) {
-        reg = *reinterpret_cast<const v4i*>(asrc + lane_off);
-        asrc += A_STEP;
+    auto copy_a = [&](int buf) { // global -> LDS, 16 bytes per lane, lane-contiguous
+        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(asrc),
+                     "s"(copy_dst + buf * BUF)
+                     : "memory", "m0");
+        asrc += a_left > 0 ? A_STEP : 0;
+        --a_left;
     };
     auto load_w = [&](wraw_t* regs) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            regs[j] = *reinterpret_cast<const wraw_t*>(wsrc[j] + lane_off);
-            wsrc[j] += W_STEP;
+            if constexpr (W4) asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(regs[j]) : "v"(lane_off), "s"(wsrc[j]));
+            else asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(regs[j]) : "v"(lane_off), "s"(wsrc[j]));
+            wsrc[j] += w_left > 0 ? W_STEP : 0;
         }
+        --w_left;
     };
-    auto store_a = [&](const v4i& reg, int buf) {
-        *reinterpret_cast<v4i*>(lds_raw + buf * BUF + wave * 1024 + lane * 16) = reg;
+    // wait until at most N of this wave's loads are outstanding; regs become valid
+    auto w_wait = [&](auto n_tag, wraw_t* regs) {
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(regs[0]), "+v"(regs[1]) : "n"(decltype(n_tag)::value) : "memory");
     };
-    auto read_a = [&](v4i* dst, int buf) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-            dst[i] = *reinterpret_cast<const v4i*>(lds_raw + buf * BUF + (i * 2 + wk) * 1024 + lane * 16);
+    // one fragment read (row block i of buffer buf); completion is awaited by frags_wait()
+    auto read_frag = [&](v4i& dst, auto buf_tag, auto i_tag) {
+        constexpr int BUFI = decltype(buf_tag)::value, I = decltype(i_tag)::value;
+        constexpr int OFF = (BUFI % 8) * BUF + I * 2048;
+        static_assert(OFF < 65536, "ds_read offset field");
+        const uint32_t addr = BUFI < 8 ? frag_lo : frag_hi;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
     };
-    auto unpack = [&](v4i* dst, const wraw_t* raw) {
+    auto frags_wait = [&](v4i* f) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3])::"memory");
+    };
+    auto unpack_one = [&](v4i& dst, const wraw_t& raw) {
         if constexpr (W4) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                dst[j].x = (raw[j].x << 4) & 0xF0F0F0F0;
-                dst[j].y = raw[j].x & 0xF0F0F0F0;
-                dst[j].z = (raw[j].y << 4) & 0xF0F0F0F0;
-                dst[j].w = raw[j].y & 0xF0F0F0F0;
-            }
+            dst.x = (raw.x << 4) & 0xF0F0F0F0;
+            dst.y = raw.x & 0xF0F0F0F0;
+            dst.z = (raw.y << 4) & 0xF0F0F0F0;
+            dst.w = raw.y & 0xF0F0F0F0;
         }
     };
+    using WaitW = std::integral_constant<int, (NSW - 2) * LPS>;
 
-    // SLOT = s % NS: ring stage, LDS buffer SLOT % NB, fragment set SLOT % 2.
-    // n1 / n2 / nf: steps s+1 / s+2 / s+NS-1 exist.
-    auto k_step = [&](auto slot_tag, auto n1, auto n2, auto nf) {
+    // Sub-step s; SLOT = s % UNR.
+    auto k_step = [&](auto slot_tag) {
         constexpr int SLOT = decltype(slot_tag)::value;
         constexpr int F = SLOT & 1;
-        if (nf) load_a(stage[(SLOT + NS - 1) % NS]);
-        if (nf) load_w(wring[(SLOT + NS - 1) % NS]);
-        if (n1) read_a(afr[F ^ 1], (SLOT + 1) % NB);
-        if (n2) store_a(stage[(SLOT + 2) % NS], (SLOT + 2) % NB);
-        if constexpr (W4) {
-            if (n1) unpack(wop[F ^ 1], wring[(SLOT + 1) % NS]);
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                if constexpr (W4)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop[F][j], afr[F][i], acc[i][j], 0, 0, 0);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[SLOT][j], afr[F][i], acc[i][j], 0, 0, 0);
-            }
-#pragma unroll
-        for (int q = 0; q < TM * TN; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
-            if (W4) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);         // unpack in its shadow
-            if (q < 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // global loads
-            if (q < 5) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // LDS reads / write
-        }
+        using NextBuf = std::integral_constant<int, (SLOT + 1) % NBUF>;
+        copy_a((SLOT + D) % NBUF);
+        load_w(wring[(SLOT + NSW - 1) % NSW]);
         __builtin_amdgcn_sched_barrier(0);
-        lds_barrier();
+        static_for<TM * TN>([&](auto q_tag) {
+            constexpr int Q = decltype(q_tag)::value;
+            constexpr int J = Q / TM, I = Q % TM;
+            if constexpr (W4)
+                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop[F][J], afr[F][I], acc[I][J], 0, 0, 0);
+            else
+                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[SLOT % NSW][J], afr[F][I], acc[I][J], 0, 0, 0);
+            // in the MFMA's shadow: one fragment read of the next sub-step, part of its unpack
+            if constexpr (Q < TM) read_frag(afr[F ^ 1][Q], NextBuf{}, std::integral_constant<int, Q>{});
+            if constexpr (Q == 1) w_wait(WaitW{}, wring[(SLOT + 1) % NSW]);
+            if constexpr (W4 && Q >= 2 && Q < 2 + TN) unpack_one(wop[F ^ 1][Q - 2], wring[(SLOT + 1) % NSW][Q - 2]);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        frags_wait(afr[F ^ 1]);
+        if constexpr ((SLOT + 1) % G == 0) asm volatile("s_barrier" ::: "memory");
     };
-    using T_ = std::true_type;
 
-    // prologue: NS-1 steps in flight; steps 0 and 1 in LDS; step 0 in registers
+    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
 #pragma unroll
-    for (int i = 0; i < NS - 1; ++i) {
-        if (i < ksteps) {
-            load_a(stage[i]);
-            load_w(wring[i]);
-        }
+    for (int t = -D; t < 0; ++t) {
+        copy_a(t + D);
+        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
     }
-    store_a(stage[0], 0);
-    if (ksteps > 1) store_a(stage[1], 1);
-    lds_barrier();
-    read_a(afr[0], 0);
-    unpack(wop[0], wring[0]);
+    w_wait(WaitW{}, wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
+    asm volatile("s_barrier" ::: "memory");
+    static_for<TM>([&](auto i_tag) { read_frag(afr[0][decltype(i_tag)::value], std::integral_constant<int, 0>{}, i_tag); });
+#pragma unroll
+    for (int j = 0; j < TN; ++j) unpack_one(wop[0][j], wring[0][j]);
+    frags_wait(afr[0]);
 
     int s = 0;
-    for (; s + 2 * NS - 2 < ksteps; s += NS)
-        static_for<NS>([&](auto slot) { k_step(slot, T_{}, T_{}, T_{}); });
-    for (; s < ksteps; s += NS)
-        static_for<NS>([&](auto slot) {
-            constexpr int SL = decltype(slot)::value;
-            if (s + SL < ksteps)
-                k_step(slot, s + SL + 1 < ksteps, s + SL + 2 < ksteps, s + SL + NS - 1 < ksteps);
+    for (; s + UNR <= ksteps; s += UNR) static_for<UNR>([&](auto slot) { k_step(slot); });
+    if (s < ksteps)
+        static_for<UNR>([&](auto slot) {
+            if (s + decltype(slot)::value < ksteps) k_step(slot);
         });
-
-    // ---- epilogue.  Scales first (their latency hides behind the exchange):
-    // after the exchange this wave owns row blocks 2*wk, 2*wk+1 of its strip.
+    // ---- epilogue.  Scale loads first: their latency hides behind the drain
+    // and the exchange.  After the exchange this wave owns row blocks 2*wk,
+    // 2*wk+1 of its strip.
     const int m_limit = g.M;
     float as[2] = {0.0f, 0.0f}, ws[TN][16];
     if constexpr (EPI != RKH_EPI_I32) {
@@ -1265,41 +1294,42 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             }
         }
     }
-    // Sum the two k-halves: each wave hands the partner's row blocks over and
-    // adds what it receives, one column block per round.  All fragment reads of
-    // the K loop completed before its last barrier, so LDS is free.  The half
-    // index is a template tag so that accumulator registers are indexed with
-    // constants.
+    // drain the look-ahead copies (they write LDS); then every wave is past its
+    // last fragment read and LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+
+    // Sum the two k-halves: each wave hands the partner's two row blocks over
+    // (4 tiles, 16 KiB per wave, the whole ring) and adds what it receives.  The
+    // half index is a template tag so that accumulator registers are indexed
+    // with constants.
     auto finish = [&](auto wk_tag) {
         constexpr int WK = decltype(wk_tag)::value;
         int* xch = reinterpret_cast<int*>(lds_raw);
         const int partner = wave ^ 4;
+        static_assert(8 * 4 * 16 * 64 * 4 <= WK_LDS_BYTES, "exchange area");
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int t = 0; t < 4; ++t) {
+            const v16i& give = acc[(WK ^ 1) * 2 + (t >> 1)][t & 1];
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii) {
-                const v16i& give = acc[(WK ^ 1) * 2 + ii][j];
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<v4i*>(xch + (((wave * 2 + ii) * 4 + q) * 64 + lane) * 4) =
-                        v4i{give[q * 4], give[q * 4 + 1], give[q * 4 + 2], give[q * 4 + 3]};
-            }
-            lds_barrier();
-#pragma unroll
-            for (int ii = 0; ii < 2; ++ii) {
-                v16i& keep = acc[WK * 2 + ii][j];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const v4i got =
-                        *reinterpret_cast<const v4i*>(xch + (((partner * 2 + ii) * 4 + q) * 64 + lane) * 4);
-                    keep[q * 4] += got.x;
-                    keep[q * 4 + 1] += got.y;
-                    keep[q * 4 + 2] += got.z;
-                    keep[q * 4 + 3] += got.w;
-                }
-            }
-            lds_barrier();
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<v4i*>(xch + (((wave * 4 + t) * 4 + q) * 64 + lane) * 4) =
+                    v4i{give[q * 4], give[q * 4 + 1], give[q * 4 + 2], give[q * 4 + 3]};
         }
+        lds_barrier();
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            v16i& keep = acc[WK * 2 + (t >> 1)][t & 1];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4i got = *reinterpret_cast<const v4i*>(xch + (((partner * 4 + t) * 4 + q) * 64 + lane) * 4);
+                keep[q * 4] += got.x;
+                keep[q * 4 + 1] += got.y;
+                keep[q * 4 + 2] += got.z;
+                keep[q * 4 + 3] += got.w;
+            }
+        }
+        lds_barrier();
         uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii) {
@@ -1326,6 +1356,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     if (wk == 0) finish(std::integral_constant<int, 0>{});
     else finish(std::integral_constant<int, 1>{});
 }
+#pragma clang diagnostic pop
 
 // Epilogue over the split-K scratch matrix; re-zeroes what it consumed so the
 // scratch is clean for the next call.
@@ -1558,7 +1589,14 @@ int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
 int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g) {
     const int mblocks = (g.M + 127) / 128, nblocks = (g.N + 255) / 256;
     const dim3 grid(mblocks * nblocks), block(512);
-#define RK_WK(W4, EPI) hipLaunchKernelGGL((gemm_wk_kernel<W4, EPI>), grid, block, 0, st, g, mblocks, nblocks)
+#define RK_WK(W4, EPI)                                                                              \
+    do {                                                                                            \
+        static const hipError_t attr = hipFuncSetAttribute(                                         \
+            reinterpret_cast<const void*>(&gemm_wk_kernel<W4, EPI>),                                \
+            hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES);                              \
+        RKH_CHECK(attr);                                                                            \
+        hipLaunchKernelGGL((gemm_wk_kernel<W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, nblocks); \
+    } while (0)
 #define RK_WK_EPI(W4)                                           \
     switch (g.epilogue) {                                       \
     case RKH_EPI_I32: RK_WK(W4, RKH_EPI_I32); break;            \
