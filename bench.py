@@ -147,6 +147,40 @@ def bench_c2(sess, ops, capi, workloads, steps, warmup):
     return out
 
 
+def bench_c2w8(sess, ops, capi, workloads, steps, warmup):
+    """w8a8 prefill GEMM at the same shape as config 2 (M=2048, K=4096, N=4096), int8 weights."""
+    M, K, N = 2048, 4096, 4096
+    c = workloads.w8a8_case(M, K, N, seed_w=4, seed_a=5)
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    dA = sess.to_device(c["A"])
+    dC = sess.empty_device(M * N * 2)
+    lib = sess.lib
+
+    def step():
+        rc = op.run_device(dA, dC)
+        if rc:
+            raise RuntimeError("run_device rc=%d" % rc)
+
+    def gemm_only():
+        rc = lib.rk_npu_matmul_workspace_rerun_gemm_device(op.ws, op.w, dC)
+        if rc:
+            raise RuntimeError("rerun rc=%d" % rc)
+
+    step_us = sess.time_us(step, steps, warmup)
+    kernel_us = sess.time_us(gemm_only, steps, warmup)
+    ops_count = 2.0 * M * K * N
+    out = {"workload": "w8a8 prefill GEMM M=2048 K=4096 N=4096, fp16 in/out, seeds 4/5",
+           "tops": ops_count / step_us / 1e6, "ms_per_step": step_us / 1e3,
+           "roofline": {"bound": "mfma", "kernel": "gemm_wk_kernel<int8,f16> (128x256 tile, waves split K)",
+                        "achieved": ops_count / kernel_us / 1e6, "peak": INT8_PEAK_TOPS,
+                        "unit": "TOP/s", "frac": ops_count / kernel_us / 1e6 / INT8_PEAK_TOPS,
+                        "kernel_us": kernel_us, "traffic": None}}
+    sess.free_device(dA)
+    sess.free_device(dC)
+    op.close()
+    return out
+
+
 def bench_c3(sess, ops, capi, workloads, steps, warmup):
     """fused w4a8 FFN block, M=128, hidden 4096, intermediate 14336."""
     c = workloads.CONFIGS[3]()
@@ -235,7 +269,7 @@ def main():
     ap.add_argument("--workload", default="c1", choices=["c1", "all"],
                     help="c1: headline line (+ c2 TOPS); all: also time configs 0, 3 and 4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c3", "c4", "copy"],
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c2w8", "c3", "c4", "copy"],
                     help="profiling aid: run one configuration's loop only")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -253,7 +287,7 @@ def main():
         sess.close()
         return
     if args.only:
-        fn = {"c0": bench_c0, "c2": bench_c2, "c3": bench_c3, "c4": bench_c4}.get(args.only)
+        fn = {"c0": bench_c0, "c2": bench_c2, "c2w8": bench_c2w8, "c3": bench_c3, "c4": bench_c4}.get(args.only)
         res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)
                if args.only == "c1" else fn(sess, ops, capi, workloads, args.steps, args.warmup))
         print(json.dumps(res))
@@ -266,7 +300,7 @@ def main():
     r2 = bench_c2(sess, ops, capi, workloads, max(args.steps // 4, 20), args.warmup)
     also = {"c2": r2}
     if args.workload == "all":
-        for name, fn in (("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
+        for name, fn in (("c2w8", bench_c2w8), ("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
             log("config %s" % name)
             also[name] = fn(sess, ops, capi, workloads, max(args.steps // 4, 20), args.warmup)
     line = {

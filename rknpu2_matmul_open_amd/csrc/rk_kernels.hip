@@ -362,6 +362,100 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     }
 }
 
+// Dense quantization of many rows: one workgroup per 8 consecutive rows, so
+// that every store instruction writes whole 128-byte lines of the tiled int8
+// matrix (for a fixed 16-element chunk, 8 consecutive rows are 8 consecutive
+// 16-byte slots of a tile).  Lane = (row r = lane % 8, chunk column lane / 8 +
+// 8 * wave): a row's loads are 8 consecutive chunks per wave instruction.  Rows
+// of up to 32 * Q8_CACHE chunks are held in registers between the maximum and
+// the quantization (all loads of a thread in flight at once); longer rows are
+// read twice, the second time from L2.
+// Modes: dynamic W8 / W4A8 maxima or a given static scale; rows written in place.
+constexpr int Q8_CACHE = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
+    __shared__ float part_max[4][8];
+    __shared__ int part_bad[4];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int r = lane & 7, cl = (lane >> 3) + 8 * wave;
+    const int m = blockIdx.x * 8 + r;
+    const bool live = m < a.M;
+    const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
+    const int nchunks = (K + 15) >> 4;
+    const T* row = static_cast<const T*>(a.src) + (size_t)(live ? m : a.M - 1) * K;
+    const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    const int mode = a.mode;
+    const bool need_max = mode != RKH_Q_W8_STATIC;
+    const bool check = mode == RKH_Q_W4A8;
+    const bool cached = nchunks <= 32 * Q8_CACHE;
+
+    float v[Q8_CACHE][16];
+    float mx = 0.0f;
+    bool bad = false;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < Q8_CACHE; ++i) {
+            const int c = cl + 32 * i;
+            if (c < nchunks) RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
+        }
+        if (need_max) {
+#pragma unroll
+            for (int i = 0; i < Q8_CACHE; ++i) {
+                if (cl + 32 * i < nchunks) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        mx = fmaxf(mx, fabsf(v[i][j]));
+                        bad |= not_finite(v[i][j]);
+                    }
+                }
+            }
+        }
+    } else if (need_max) {
+        for (int c = cl; c < nchunks; c += 32) {
+            float tmp[16];
+            RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                mx = fmaxf(mx, fabsf(tmp[j]));
+                bad |= not_finite(tmp[j]);
+            }
+        }
+    }
+    float scale = 1.0f;
+    if (need_max) {
+#pragma unroll
+        for (int off = 8; off < 64; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        const unsigned long long bad_mask = __ballot(bad && check && live);
+        if (lane < 8) part_max[wave][lane] = mx;
+        if (lane == 0) part_bad[wave] = bad_mask != 0ull;
+        __syncthreads();
+        mx = fmaxf(fmaxf(part_max[0][r], part_max[1][r]), fmaxf(part_max[2][r], part_max[3][r]));
+        if (t == 0 && a.bad_flag && (part_bad[0] | part_bad[1] | part_bad[2] | part_bad[3])) atomicOr(a.bad_flag, 1);
+        if (mode == RKH_Q_W4A8) scale = mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN);
+        else scale = mx > 0.0f ? mx / 127.0f : 1.0f;
+        if (t < 8 && live && a.scale) a.scale[m] = scale;
+    } else {
+        scale = a.scale[live ? m : a.M - 1];
+    }
+    if (!live) return;
+    const float inv = 1.0f / scale;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < Q8_CACHE; ++i) {
+            const int c = cl + 32 * i;
+            if (c < nchunks)
+                *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(v[i], inv);
+        }
+    } else {
+        for (int c = cl; c < nchunks; c += 32) {
+            float tmp[16];
+            RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(tmp, inv);
+        }
+    }
+}
+
 // ------------------------------------------------------------- epilogues
 // Degree-7 fp32 exponential SiLU, step for step the sequence of the reference
 // (src/rk_npu_swiglu_fp32_neon.h:13-51): every fused step is an explicit fmaf.
@@ -1231,6 +1325,10 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         constexpr int SLOT = decltype(slot_tag)::value;
         constexpr int F = SLOT & 1;
         using NextBuf = std::integral_constant<int, (SLOT + 1) % NBUF>;
+        // The two waves of a SIMD drift apart between barriers (the older one wins
+        // every issue conflict) and the one left behind cannot keep the matrix pipe
+        // busy alone; the wave that is further into the barrier interval yields.
+        __builtin_amdgcn_s_setprio(G - 1 - SLOT % G);
         copy_a((SLOT + D) % NBUF);
         load_w(wring[(SLOT + NSW - 1) % NSW]);
         __builtin_amdgcn_sched_barrier(0);
@@ -1786,7 +1884,19 @@ int rkh_pack_w4(void* stream, const int8_t* src, int K, int N, int interleave_F,
 
 int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     if (args->M <= 0) return RKH_OK;
-    const dim3 grid(args->M), block(256);
+    const dim3 block(256);
+    const int mode = args->mode;
+    if (args->M >= 256 && !args->dest_rows && !args->active_blocks && args->in_dtype != RKH_I8 &&
+        (mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_W8_STATIC)) {
+        const dim3 grid8((args->M + 7) / 8);
+        if (args->in_dtype == RKH_F16)
+            hipLaunchKernelGGL(quant_rows8_kernel<uint16_t>, grid8, block, 0, (hipStream_t)stream, *args);
+        else
+            hipLaunchKernelGGL(quant_rows8_kernel<float>, grid8, block, 0, (hipStream_t)stream, *args);
+        RKH_CHECK(hipGetLastError());
+        return RKH_OK;
+    }
+    const dim3 grid(args->M);
     switch (args->in_dtype) {
     case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args); break;
     case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args); break;
@@ -1813,7 +1923,7 @@ static DensePlan dense_plan(int M, int N, int K, int w_int4) {
     while (bm > 32 && tiles_of(bm) < 160) bm >>= 1;
     const long tiles = tiles_of(bm);
     int s = 1;
-    if (tiles < 192) {
+    if (tiles < 192 && bm < 128) { // 128-row tiles are only chosen when they fill most of the chip
         s = (int)((256 + tiles - 1) / tiles);
         const int max_s = ksteps / 8 > 0 ? ksteps / 8 : 1; // at least 512 k per part
         if (s > max_s) s = max_s;

@@ -20,7 +20,9 @@ def _rand_i8(rng, shape, lo=-127, hi=127):
 # reference examples/demo.cpp:58-62 runs odd shapes such as 17x40x33, 300x48x33, 1x200x200
 I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96), (17, 40, 33),
               (33, 130, 70), (64, 256, 256), (65, 257, 129), (128, 512, 384), (300, 48, 33),
-              (200, 1000, 520)]
+              (200, 1000, 520),
+              # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
+              (641, 6900, 200), (700, 6900, 1100)]
 
 
 @pytest.mark.parametrize("M,N,K", I32_SHAPES)
@@ -59,7 +61,8 @@ def test_i8i8i32_extremes_wrap(sess, oracle):
 
 
 F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64, 128),
-              (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024)]
+              (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024),
+              (650, 7000, 1100)]  # large-tile kernel
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
@@ -83,8 +86,8 @@ def test_f16i8f16_dynamic_bit_exact(sess, oracle, M, N, K):
         op.close()
 
 
-def test_f32i8f32_dynamic_and_static(sess, oracle):
-    M, N, K = 37, 200, 300
+@pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203)])  # second: many-row quantization path
+def test_f32i8f32_dynamic_and_static(sess, oracle, M, N, K):
     rng = np.random.default_rng(5)
     A = rng.standard_normal((M, K)).astype(np.float32) * 3
     A[0, :8] = [127, -127, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5]
