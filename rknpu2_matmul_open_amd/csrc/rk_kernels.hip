@@ -1213,7 +1213,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 //    sub-step s+D-NBUF, last read at sub-step s+D-NBUF-1 <= s-G-1, which is
 //    before the latest barrier (needs NBUF >= D + G).
 constexpr int WK_NSW = 8, WK_NBUF = 16, WK_G = 4, WK_D = 12, WK_BUF = 8 * 1024;
-constexpr int WK_LDS_BYTES = WK_NBUF * WK_BUF;
+constexpr int WK_SCALES_OFF = WK_NBUF * WK_BUF;            // fp32 scales of the tile: 128 rows, then 256 columns
+constexpr int WK_LDS_BYTES = WK_SCALES_OFF + (128 + 256) * 4;
 static_assert(WK_D >= WK_NSW + WK_G - 1 && WK_NBUF >= WK_D + WK_G, "see the ordering rules above");
 
 typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
@@ -1349,6 +1350,35 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         if constexpr ((SLOT + 1) % G == 0) asm volatile("s_barrier" ::: "memory");
     };
 
+    // The tile's scales are fetched before anything else and parked in LDS, so
+    // the epilogue does not start with a round trip to memory: thread t holds the
+    // row scale of row t (t < 128) and the column scale of physical column t
+    // (t < 256).  They are the oldest loads in flight, so the prologue's wait
+    // below covers them.
+    float my_as = 0.0f, my_ws = 0.0f;
+    bool as_valid = false, ws_valid = false;
+    if constexpr (EPI != RKH_EPI_I32) {
+        const int t = threadIdx.x;
+        const int m = mblk * BM + (t & 127);
+        const int pb = nblk * 8 + ((t & 255) >> 5);
+        int n;
+        if constexpr (EPI == RKH_EPI_SWIGLU) {
+            // pb even = gate, odd = up block of middle columns (pb / 2) * 32
+            const int F = g.interleave_F;
+            const int nl = (pb >> 1) * 32 + (t & 31);
+            n = (pb & 1 ? F : 0) + nl;
+            ws_valid = nl < F;
+        } else {
+            const bool live = g.interleave_F ? pb < g.N / 32 : pb * 32 < g.N;
+            n = block_first_col(pb, g.interleave_F) + (t & 31);
+            ws_valid = live && n < g.N;
+        }
+        as_valid = m < g.M;
+        const float* pa = g.a_scale + (as_valid ? m : 0);
+        const float* pw = g.w_scale + (ws_valid ? n : 0);
+        asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
+        asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
+    }
     // prologue: the same issue order as if the loop had run for sub-steps -D..-1
 #pragma unroll
     for (int t = -D; t < 0; ++t) {
@@ -1356,7 +1386,14 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
     }
     w_wait(WaitW{}, wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
-    asm volatile("s_barrier" ::: "memory");
+    if constexpr (EPI != RKH_EPI_I32) {
+        asm volatile("" : "+v"(my_as), "+v"(my_ws)); // valid from here on
+        float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
+        const int t = threadIdx.x;
+        if (t < 128) sc[t] = as_valid ? my_as : 0.0f;
+        if (t < 256) sc[128 + t] = ws_valid ? my_ws : 0.0f;
+    }
+    lds_barrier();
     static_for<TM>([&](auto i_tag) { read_frag(afr[0][decltype(i_tag)::value], std::integral_constant<int, 0>{}, i_tag); });
 #pragma unroll
     for (int j = 0; j < TN; ++j) unpack_one(wop[0][j], wring[0][j]);
@@ -1368,29 +1405,18 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         static_for<UNR>([&](auto slot) {
             if (s + decltype(slot)::value < ksteps) k_step(slot);
         });
-    // ---- epilogue.  Scale loads first: their latency hides behind the drain
-    // and the exchange.  After the exchange this wave owns row blocks 2*wk,
-    // 2*wk+1 of its strip.
+    // ---- epilogue.  After the exchange this wave owns row blocks 2*wk, 2*wk+1
+    // of its strip; its scales come from the LDS copy made in the prologue.
     const int m_limit = g.M;
     float as[2] = {0.0f, 0.0f}, ws[TN][16];
     if constexpr (EPI != RKH_EPI_I32) {
+        const float* sc = reinterpret_cast<const float*>(lds_raw + WK_SCALES_OFF);
 #pragma unroll
-        for (int ii = 0; ii < 2; ++ii) {
-            const int m = mblk * BM + (wk * 2 + ii) * 32 + (lane & 31);
-            as[ii] = m < m_limit ? g.a_scale[m] : 0.0f;
-        }
+        for (int ii = 0; ii < 2; ++ii) as[ii] = sc[(wk * 2 + ii) * 32 + (lane & 31)];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int pb = nblk * 8 + wn * TN + j;
-            if constexpr (EPI == RKH_EPI_SWIGLU) {
-                // pb even = gate, odd = up block of middle columns (pb / 2) * 32
-                const int F = g.interleave_F;
-                load_col_scales(ws[j], g.w_scale + (j ? F : 0), (pb >> 1) * 32, F, lane);
-            } else {
-                const bool live = g.interleave_F ? pb < g.N / 32 : pb * 32 < g.N;
-                load_col_scales(ws[j], g.w_scale, block_first_col(pb, g.interleave_F), live ? g.N : 0, lane);
-            }
-        }
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ws[j][r] = sc[128 + (wn * TN + j) * 32 + tile_col(r, lane)];
     }
     // drain the look-ahead copies (they write LDS); then every wave is past its
     // last fragment read and LDS is reused
@@ -1405,7 +1431,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         constexpr int WK = decltype(wk_tag)::value;
         int* xch = reinterpret_cast<int*>(lds_raw);
         const int partner = wave ^ 4;
-        static_assert(8 * 4 * 16 * 64 * 4 <= WK_LDS_BYTES, "exchange area");
+        static_assert(8 * 4 * 16 * 64 * 4 <= WK_SCALES_OFF, "exchange area");
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const v16i& give = acc[(WK ^ 1) * 2 + (t >> 1)][t & 1];
