@@ -1350,11 +1350,17 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         if constexpr ((SLOT + 1) % G == 0) asm volatile("s_barrier" ::: "memory");
     };
 
-    // The tile's scales are fetched before anything else and parked in LDS, so
-    // the epilogue does not start with a round trip to memory: thread t holds the
-    // row scale of row t (t < 128) and the column scale of physical column t
-    // (t < 256).  They are the oldest loads in flight, so the prologue's wait
-    // below covers them.
+    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
+#pragma unroll
+    for (int t = -D; t < 0; ++t) {
+        copy_a(t + D);
+        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
+    }
+    // The tile's scales are fetched now, behind the prologue's loads, and handed
+    // to the epilogue through LDS after the loop, so the epilogue does not start
+    // with a round trip to memory: thread t holds the row scale of row t
+    // (t < 128) and the column scale of physical column t (t < 256).  (Two more
+    // loads in the queue only make the first sub-steps' waits stricter.)
     float my_as = 0.0f, my_ws = 0.0f;
     bool as_valid = false, ws_valid = false;
     if constexpr (EPI != RKH_EPI_I32) {
@@ -1379,21 +1385,8 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
     }
-    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
-#pragma unroll
-    for (int t = -D; t < 0; ++t) {
-        copy_a(t + D);
-        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
-    }
     w_wait(WaitW{}, wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
-    if constexpr (EPI != RKH_EPI_I32) {
-        asm volatile("" : "+v"(my_as), "+v"(my_ws)); // valid from here on
-        float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
-        const int t = threadIdx.x;
-        if (t < 128) sc[t] = as_valid ? my_as : 0.0f;
-        if (t < 256) sc[128 + t] = ws_valid ? my_ws : 0.0f;
-    }
-    lds_barrier();
+    asm volatile("s_barrier" ::: "memory");
     static_for<TM>([&](auto i_tag) { read_frag(afr[0][decltype(i_tag)::value], std::integral_constant<int, 0>{}, i_tag); });
 #pragma unroll
     for (int j = 0; j < TN; ++j) unpack_one(wop[0][j], wring[0][j]);
@@ -1405,10 +1398,19 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         static_for<UNR>([&](auto slot) {
             if (s + decltype(slot)::value < ksteps) k_step(slot);
         });
-    // ---- epilogue.  After the exchange this wave owns row blocks 2*wk, 2*wk+1
-    // of its strip; its scales come from the LDS copy made in the prologue.
+    // ---- epilogue.  Drain the look-ahead copies (they write LDS) and the scale
+    // loads; then every wave is past its last fragment read and LDS is reused.
+    // After the exchange this wave owns row blocks 2*wk, 2*wk+1 of its strip.
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(my_as), "+v"(my_ws)::"memory");
     const int m_limit = g.M;
     float as[2] = {0.0f, 0.0f}, ws[TN][16];
+    if constexpr (EPI != RKH_EPI_I32) {
+        float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
+        const int t = threadIdx.x;
+        if (t < 128) sc[t] = as_valid ? my_as : 0.0f;
+        if (t < 256) sc[128 + t] = ws_valid ? my_ws : 0.0f;
+    }
+    lds_barrier();
     if constexpr (EPI != RKH_EPI_I32) {
         const float* sc = reinterpret_cast<const float*>(lds_raw + WK_SCALES_OFF);
 #pragma unroll
@@ -1418,10 +1420,6 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 #pragma unroll
             for (int r = 0; r < 16; ++r) ws[j][r] = sc[128 + (wn * TN + j) * 32 + tile_col(r, lane)];
     }
-    // drain the look-ahead copies (they write LDS); then every wave is past its
-    // last fragment read and LDS is reused
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    lds_barrier();
 
     // Sum the two k-halves: each wave hands the partner's two row blocks over
     // (4 tiles, 16 KiB per wave, the whole ring) and adds what it receives.  The
