@@ -47,7 +47,7 @@ extern "C" {
 #define RKH_ERR_NOMEM (-4)
 #define RKH_ERR_RUNTIME (-5)
 
-enum { RKH_ROW_ALIGN = 128, RKH_COL_ALIGN = 256, RKH_K_ALIGN = 64 };
+enum { RKH_ROW_ALIGN = 128, RKH_COL_ALIGN = 256, RKH_K_ALIGN = 256 };
 
 #if defined(__HIPCC__)
 #define RKH_HD __host__ __device__

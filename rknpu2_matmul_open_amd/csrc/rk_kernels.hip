@@ -1133,25 +1133,6 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 
     // ---- epilogue
     const int m_limit = GROUPED ? g.num_blocks[0] * 32 : g.M;
-    if (ksplit > 1) {
-        // exact integer partial sums: accumulate into the zeroed scratch matrix
-        // (physical column order); a second kernel applies the epilogue.
-        const int ld = nblocks * BN;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int m = mblk * BM + (wm * TM + i) * 32 + (lane & 31);
-                const int col0 = (nblk * (BN / 32) + wn * TN + j) * 32;
-                if (m < m_limit) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (acc[i][j][r])
-                            atomicAdd(g.splitk_acc + (size_t)m * ld + col0 + tile_col(r, lane), acc[i][j][r]);
-                }
-            }
-        return;
-    }
     // all waves are past their last LDS fragment read (the barrier of the last
     // step precedes only register work), so the buffers can be reused as
     // wave-private staging for the stores
@@ -1174,36 +1155,40 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
     }
 }
 
-// ---- 128 x 256 tile, waves split K ------------------------------------------
-// The large dense tile.  Eight waves = 4 column groups (wn) x 2 k-halves (wk):
-// wave (wn, wk) accumulates the whole 128 x 64 strip of column group wn, but
-// only over k-tile wk of every 64-deep K sub-step; the two halves are summed
+// ---- tiles of (32 * TM) rows x 256 columns, waves split K --------------------
+// Eight waves = 4 column groups (wn) x 2 k-halves (wk): wave (wn, wk)
+// accumulates the whole (32*TM) x 64 strip of column group wn, but only over
+// every second 32-deep k-tile (k-tile % 2 == wk); the two halves are summed
 // once, through LDS, before the epilogue.  Compared with splitting the rows
 // between the two waves that share a SIMD, no weight byte is loaded (or
 // unpacked) by two waves, which takes a third off the traffic through the
-// vector memory path and halves the int4 unpack work, at the price of 128
-// accumulator registers per lane.
+// vector memory path and halves the int4 unpack work.
 //
-// Activations: every wave copies its 1 KiB share of a sub-step's 128 x 64 tile
-// global -> LDS directly (no registers), WK_D sub-steps ahead, into a ring of
-// WK_NBUF buffers.  Weights: global -> registers, WK_NSW-1 sub-steps ahead (8
-// bytes per lane for int4, 16 for int8).  Each sub-step a wave also reads the
-// four 16-byte activation fragments of the NEXT sub-step and issues eight
-// MFMAs, with the int4 unpack of the next operands in their shadow.
+// A sub-step always covers 8 KiB of activations = (32*TM) rows x (8/TM)
+// k-tiles, i.e. 64 / 128 / 256 k for TM = 4 / 2 / 1, so that whatever the tile
+// height a wave issues per sub-step one 1 KiB activation copy, four 16-byte
+// fragment reads and eight MFMAs.
 //
-// A workgroup barrier costs roughly a third of a sub-step's MFMA time (the
-// matrix pipes drain while the waves meet), so there is only one every WK_G
+// Activations: every wave copies its 1 KiB share of a sub-step global -> LDS
+// directly (no registers), WK_D sub-steps ahead, into a ring of WK_NBUF
+// buffers.  Weights: global -> registers, NSW-1 sub-steps ahead (8 bytes per
+// lane and k-tile pair for int4, 16 per k-tile for int8).  The fragments of
+// the NEXT sub-step are read and, for int4, its operands unpacked in the
+// shadow of this sub-step's MFMAs.
+//
+// A workgroup barrier costs a good part of a sub-step's MFMA time (the matrix
+// pipes drain while the waves meet), so there is only one every WK_G
 // sub-steps.
 //
 // All loads of the loop are inline assembly and every wait is explicit.  (The
 // compiler's own bookkeeping orders each LDS read and each register load after
 // ALL outstanding global -> LDS copies, which would undo the prefetch.)  The
 // waits rely on vector memory loads completing in issue order and on every
-// sub-step issuing exactly 1 + TN loads -- copy first, then weights -- also
+// sub-step issuing exactly LPS loads -- copy first, then weights -- also
 // beyond the end of K, where the source pointers simply stop advancing (those
 // loads hit the L1 and their results are never used).  With that:
-//  * weights of sub-step s+1 were issued at s+1-(NSW-1); (NSW-2) * (1+TN)
-//    loads have been issued since, hence vmcnt((NSW-2) * (1+TN));
+//  * weights of sub-step s+1 were issued at s+1-(NSW-1); (NSW-2) * LPS loads
+//    have been issued since, hence vmcnt((NSW-2) * LPS);
 //  * publication: the fragments read during sub-steps B+1..B+G (B = last
 //    sub-step before a barrier) belong to sub-steps <= B+G+1; their copies
 //    were issued at sub-steps <= B+G+1-D, before the weights a wave waits for
@@ -1212,22 +1197,46 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int
 //  * reuse: the copy issued at sub-step s overwrites the buffer that held
 //    sub-step s+D-NBUF, last read at sub-step s+D-NBUF-1 <= s-G-1, which is
 //    before the latest barrier (needs NBUF >= D + G).
-constexpr int WK_NSW = 8, WK_NBUF = 16, WK_G = 4, WK_D = 12, WK_BUF = 8 * 1024;
-constexpr int WK_SCALES_OFF = WK_NBUF * WK_BUF;            // fp32 scales of the tile: 128 rows, then 256 columns
+//
+// Split K over workgroups (ksplit > 1, small M): every part stores its int32
+// tile in accumulator order to scratch and gemm_wk_reduce_kernel, launched
+// behind it, adds the parts and runs the epilogue.  (Summing inside this
+// kernel, in the part that arrives last, needs a device-scope release per
+// workgroup; on this multi-die part each one walks the die's L2, and 32
+// workgroups per die queueing for that cost more than the second launch.)
+constexpr int WK_NBUF = 16, WK_G = 4, WK_D = 12, WK_BUF = 8 * 1024;
+constexpr int WK_SCALES_OFF = WK_NBUF * WK_BUF;                   // fp32 scales of the tile: 128 rows, then 256 columns
 constexpr int WK_LDS_BYTES = WK_SCALES_OFF + (128 + 256) * 4;
-static_assert(WK_D >= WK_NSW + WK_G - 1 && WK_NBUF >= WK_D + WK_G, "see the ordering rules above");
 
 typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
+// Row / column block of logical dense tile `tile`: column sweeps over groups of
+// 4 row blocks, so that concurrently running tiles share weight columns in L2.
+__device__ __forceinline__ void wk_tile_coords(int tile, int mblocks, int nblocks, int& mblk, int& nblk) {
+    constexpr int GM = 4;
+    const int per_group = GM * nblocks;
+    const int group = tile / per_group;
+    const int first_m = group * GM;
+    const int gm = min(mblocks - first_m, GM);
+    const int in_group = tile - group * per_group;
+    mblk = first_m + in_group % gm;
+    nblk = in_group / gm;
+}
+
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm" // m0 is set and clobbered on purpose below
-template <bool W4, int EPI>
-__global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
-    constexpr int TM = 4, TN = 2, NSW = WK_NSW, NBUF = WK_NBUF, G = WK_G, D = WK_D;
-    constexpr int BM = 128, BUF = WK_BUF;
-    constexpr int UNR = 16; // sub-steps per unrolled trip: multiple of NSW, NBUF, G and 2
-    constexpr int LPS = 1 + TN; // loads per sub-step and wave
+template <int TM, bool W4, int EPI>
+__global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mblocks, int nblocks, int ksplit,
+                                                      int ksteps_per_part) {
+    constexpr int TN = 2, KTS = 8 / TM, KTW = KTS / 2; // k-tiles per sub-step: all / this wave's
+    constexpr int NSW = (TM == 4 || (TM == 2 && W4)) ? 8 : 4;
+    constexpr int NBUF = WK_NBUF, G = WK_G, D = WK_D, BM = 32 * TM, BUF = WK_BUF;
+    constexpr int UNR = 16;            // sub-steps per unrolled trip: multiple of NSW, NBUF, G and 2
+    constexpr int LPS = 1 + KTW * TN;  // loads per sub-step and wave
+    constexpr int NWREG = KTW * TN;    // weight registers (and unpack items) per sub-step
     static_assert(UNR % NSW == 0 && UNR % NBUF == 0 && UNR % G == 0, "slot arithmetic must be compile-time");
+    static_assert(D >= NSW + G - 1 && NBUF >= D + G, "see the ordering rules above");
+    static_assert((NSW - 2) * LPS <= 63, "vmcnt field");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[]; // WK_LDS_BYTES
 
     const int lane = lane_id();
@@ -1235,35 +1244,41 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     const int wn = wave & 3, wk = wave >> 2;
     const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
     const int KB = Kp / 32;
-    const int ksteps = KB / 2;
+    const int ksteps_total = KB / KTS;
 
     // ---- tile assignment: XCD-contiguous ranges, 4 row blocks per column sweep
-    const int total = mblocks * nblocks;
-    const int tile = xcd_remap(blockIdx.x, total);
-    constexpr int GM = 4;
-    const int per_group = GM * nblocks;
-    const int group = tile / per_group;
-    const int first_m = group * GM;
-    const int gm = min(mblocks - first_m, GM);
-    const int in_group = tile - group * per_group;
-    const int mblk = first_m + in_group % gm;
-    const int nblk = in_group / gm;
+    const int tiles = mblocks * nblocks;
+    const int logical = xcd_remap(blockIdx.x, tiles * ksplit);
+    const int kpart = logical / tiles;
+    const int tile = logical - kpart * tiles;
+    int mblk, nblk;
+    wk_tile_coords(tile, mblocks, nblocks, mblk, nblk);
+    const int kstep0 = kpart * ksteps_per_part;
+    const int ksteps = min(ksteps_per_part, ksteps_total - kstep0); // >= 1 by construction of the launch
+
+    const uint8_t* Wb = g.W;
+    const float* w_scale = g.w_scale;
+    const int m_limit = g.M;
 
     // ---- sources: wave-uniform base pointers (scalar registers) + a constant lane offset.
-    // activation chunk of this wave: row block wave / 2, k-tile wave % 2
-    const uint8_t* asrc = g.A + ((size_t)(mblk * 4 + (wave >> 1)) * KB + (wave & 1)) * 1024;
+    // activation chunk of this wave: row block wave / KTS, k-tile wave % KTS of the sub-step
+    const uint8_t* asrc = g.A + ((size_t)(mblk * TM + wave / KTS) * KB + (size_t)kstep0 * KTS + wave % KTS) * 1024;
+    // int8 weights of a wave with four k-tiles per sub-step span 6 KiB; the base
+    // sits in the middle so that the 13-bit signed instruction offset reaches all
+    constexpr int W_BIAS = (!W4 && KTW > 2) ? 4096 : 0;
     const uint8_t* wsrc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int pb = nblk * 8 + wn * TN + j;
-        wsrc[j] = W4 ? g.W + (size_t)pb * (KB / 2) * 1024 + wk * 8 : g.W + ((size_t)pb * KB + wk) * 1024;
+        wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0 * KTW) * 1024 + wk * 8
+                     : Wb + ((size_t)pb * KB + (size_t)kstep0 * KTS + wk) * 1024 + W_BIAS;
     }
     const unsigned lane_off = lane * 16;
-    constexpr int A_STEP = 2048, W_STEP = W4 ? 1024 : 2048;
+    constexpr int A_STEP = KTS * 1024, W_STEP = W4 ? KTW * 1024 : KTS * 1024;
     using wraw_t = typename std::conditional<W4, v2i, v4i>::type;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds_raw;
     const uint32_t copy_dst = lds_base + wave * 1024; // this wave's chunk inside buffer 0
-    // LDS byte addresses of this lane's fragment of row block 0 in buffers 0 and 8
+    // LDS byte addresses of this lane's fragment (row block 0, this wave's first k-tile) in buffers 0 and 8
     uint32_t frag_lo = lds_base + wk * 1024 + lane * 16;
     uint32_t frag_hi = frag_lo + 8 * BUF;
     int a_left = ksteps - 1, w_left = ksteps - 1; // how often the sources may still advance
@@ -1276,9 +1291,9 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    wraw_t wring[NSW][TN]; // weight prefetch ring
-    v4i afr[2][TM];        // activation fragments, this sub-step / next
-    v4i wop[2][TN];        // int4 only: unpacked operands, this sub-step / next
+    wraw_t wring[NSW][NWREG]; // weight prefetch ring, index u * TN + j
+    v4i afr[2][4];            // activation fragments (index u * TM + i), this sub-step / next
+    v4i wop[2][NWREG];        // int4 only: unpacked operands, this sub-step / next
 
     auto copy_a = [&](int buf) { // global -> LDS, 16 bytes per lane, lane-contiguous
         asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(asrc),
@@ -1288,22 +1303,32 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         --a_left;
     };
     auto load_w = [&](wraw_t* regs) {
+        static_for<NWREG>([&](auto e_tag) {
+            constexpr int E = decltype(e_tag)::value, U = E / TN, J = E % TN;
+            const unsigned off = lane_off; // (locals: asm operands cannot name captures of an enclosing lambda)
+            const uint8_t* base = wsrc[J];
+            wraw_t r;
+            if constexpr (W4)
+                asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(r) : "v"(off), "s"(base), "n"(U * 1024));
+            else
+                asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(r) : "v"(off), "s"(base), "n"(U * 2048 - W_BIAS));
+            regs[E] = r;
+        });
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if constexpr (W4) asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(regs[j]) : "v"(lane_off), "s"(wsrc[j]));
-            else asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(regs[j]) : "v"(lane_off), "s"(wsrc[j]));
-            wsrc[j] += w_left > 0 ? W_STEP : 0;
-        }
+        for (int j = 0; j < TN; ++j) wsrc[j] += w_left > 0 ? W_STEP : 0;
         --w_left;
     };
-    // wait until at most N of this wave's loads are outstanding; regs become valid
-    auto w_wait = [&](auto n_tag, wraw_t* regs) {
-        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(regs[0]), "+v"(regs[1]) : "n"(decltype(n_tag)::value) : "memory");
+    // wait until at most (NSW-2)*LPS of this wave's loads are outstanding; regs become valid
+    auto w_wait = [&](wraw_t* regs) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSW - 2) * LPS) : "memory");
+#pragma unroll
+        for (int e = 0; e < NWREG; ++e) asm volatile("" : "+v"(regs[e]));
     };
-    // one fragment read (row block i of buffer buf); completion is awaited by frags_wait()
-    auto read_frag = [&](v4i& dst, auto buf_tag, auto i_tag) {
-        constexpr int BUFI = decltype(buf_tag)::value, I = decltype(i_tag)::value;
-        constexpr int OFF = (BUFI % 8) * BUF + I * 2048;
+    // fragment f = u * TM + i of buffer buf; completion is awaited by frags_wait()
+    auto read_frag = [&](v4i& dst, auto buf_tag, auto f_tag) {
+        constexpr int BUFI = decltype(buf_tag)::value, FI = decltype(f_tag)::value;
+        constexpr int U = FI / TM, I = FI % TM;
+        constexpr int OFF = (BUFI % 8) * BUF + (I * KTS + 2 * U) * 1024;
         static_assert(OFF < 65536, "ds_read offset field");
         const uint32_t addr = BUFI < 8 ? frag_lo : frag_hi;
         asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
@@ -1319,13 +1344,13 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             dst.w = raw.y & 0xF0F0F0F0;
         }
     };
-    using WaitW = std::integral_constant<int, (NSW - 2) * LPS>;
 
     // Sub-step s; SLOT = s % UNR.
     auto k_step = [&](auto slot_tag) {
         constexpr int SLOT = decltype(slot_tag)::value;
         constexpr int F = SLOT & 1;
         using NextBuf = std::integral_constant<int, (SLOT + 1) % NBUF>;
+        constexpr int UPS = (NWREG + 3) / 4; // unpack items per MFMA slot (slots 2..5)
         // The two waves of a SIMD drift apart between barriers (the older one wins
         // every issue conflict) and the one left behind cannot keep the matrix pipe
         // busy alone; the wave that is further into the barrier interval yields.
@@ -1333,17 +1358,22 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         copy_a((SLOT + D) % NBUF);
         load_w(wring[(SLOT + NSW - 1) % NSW]);
         __builtin_amdgcn_sched_barrier(0);
-        static_for<TM * TN>([&](auto q_tag) {
+        static_for<8>([&](auto q_tag) {
             constexpr int Q = decltype(q_tag)::value;
-            constexpr int J = Q / TM, I = Q % TM;
+            constexpr int U = Q / (TN * TM), J = Q % (TN * TM) / TM, I = Q % TM;
             if constexpr (W4)
-                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop[F][J], afr[F][I], acc[I][J], 0, 0, 0);
+                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop[F][U * TN + J], afr[F][U * TM + I], acc[I][J], 0, 0, 0);
             else
-                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[SLOT % NSW][J], afr[F][I], acc[I][J], 0, 0, 0);
+                acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[SLOT % NSW][U * TN + J], afr[F][U * TM + I],
+                                                                  acc[I][J], 0, 0, 0);
             // in the MFMA's shadow: one fragment read of the next sub-step, part of its unpack
-            if constexpr (Q < TM) read_frag(afr[F ^ 1][Q], NextBuf{}, std::integral_constant<int, Q>{});
-            if constexpr (Q == 1) w_wait(WaitW{}, wring[(SLOT + 1) % NSW]);
-            if constexpr (W4 && Q >= 2 && Q < 2 + TN) unpack_one(wop[F ^ 1][Q - 2], wring[(SLOT + 1) % NSW][Q - 2]);
+            if constexpr (Q < 4) read_frag(afr[F ^ 1][Q], NextBuf{}, std::integral_constant<int, Q>{});
+            if constexpr (Q == 1) w_wait(wring[(SLOT + 1) % NSW]);
+            if constexpr (W4 && Q >= 2 && Q < 6) {
+#pragma unroll
+                for (int e = (Q - 2) * UPS; e < (Q - 1) * UPS; ++e)
+                    if (e < NWREG) unpack_one(wop[F ^ 1][e], wring[(SLOT + 1) % NSW][e]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
         frags_wait(afr[F ^ 1]);
@@ -1359,13 +1389,13 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     // The tile's scales are fetched now, behind the prologue's loads, and handed
     // to the epilogue through LDS after the loop, so the epilogue does not start
     // with a round trip to memory: thread t holds the row scale of row t
-    // (t < 128) and the column scale of physical column t (t < 256).  (Two more
+    // (t < BM) and the column scale of physical column t (t < 256).  (Two more
     // loads in the queue only make the first sub-steps' waits stricter.)
     float my_as = 0.0f, my_ws = 0.0f;
     bool as_valid = false, ws_valid = false;
     if constexpr (EPI != RKH_EPI_I32) {
         const int t = threadIdx.x;
-        const int m = mblk * BM + (t & 127);
+        const int m = mblk * BM + (t & (BM - 1));
         const int pb = nblk * 8 + ((t & 255) >> 5);
         int n;
         if constexpr (EPI == RKH_EPI_SWIGLU) {
@@ -1379,17 +1409,17 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             n = block_first_col(pb, g.interleave_F) + (t & 31);
             ws_valid = live && n < g.N;
         }
-        as_valid = m < g.M;
+        as_valid = m < m_limit;
         const float* pa = g.a_scale + (as_valid ? m : 0);
-        const float* pw = g.w_scale + (ws_valid ? n : 0);
+        const float* pw = w_scale + (ws_valid ? n : 0);
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
     }
-    w_wait(WaitW{}, wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
+    w_wait(wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
     asm volatile("s_barrier" ::: "memory");
-    static_for<TM>([&](auto i_tag) { read_frag(afr[0][decltype(i_tag)::value], std::integral_constant<int, 0>{}, i_tag); });
+    static_for<4>([&](auto f_tag) { read_frag(afr[0][decltype(f_tag)::value], std::integral_constant<int, 0>{}, f_tag); });
 #pragma unroll
-    for (int j = 0; j < TN; ++j) unpack_one(wop[0][j], wring[0][j]);
+    for (int e = 0; e < NWREG; ++e) unpack_one(wop[0][e], wring[0][e]);
     frags_wait(afr[0]);
 
     int s = 0;
@@ -1398,53 +1428,48 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
         static_for<UNR>([&](auto slot) {
             if (s + decltype(slot)::value < ksteps) k_step(slot);
         });
+    __builtin_amdgcn_s_setprio(0);
+
     // ---- epilogue.  Drain the look-ahead copies (they write LDS) and the scale
     // loads; then every wave is past its last fragment read and LDS is reused.
-    // After the exchange this wave owns row blocks 2*wk, 2*wk+1 of its strip.
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(my_as), "+v"(my_ws)::"memory");
-    const int m_limit = g.M;
-    float as[2] = {0.0f, 0.0f}, ws[TN][16];
     if constexpr (EPI != RKH_EPI_I32) {
         float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
         const int t = threadIdx.x;
-        if (t < 128) sc[t] = as_valid ? my_as : 0.0f;
+        if (t < BM) sc[t] = as_valid ? my_as : 0.0f;
         if (t < 256) sc[128 + t] = ws_valid ? my_ws : 0.0f;
     }
     lds_barrier();
-    if constexpr (EPI != RKH_EPI_I32) {
-        const float* sc = reinterpret_cast<const float*>(lds_raw + WK_SCALES_OFF);
-#pragma unroll
-        for (int ii = 0; ii < 2; ++ii) as[ii] = sc[(wk * 2 + ii) * 32 + (lane & 31)];
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) ws[j][r] = sc[128 + (wn * TN + j) * 32 + tile_col(r, lane)];
-    }
 
-    // Sum the two k-halves: each wave hands the partner's two row blocks over
-    // (4 tiles, 16 KiB per wave, the whole ring) and adds what it receives.  The
-    // half index is a template tag so that accumulator registers are indexed
-    // with constants.
+    // The k-half index is a template tag so that accumulator registers are
+    // indexed with constants.  After the exchange a wave owns KEEP row blocks
+    // of its strip: TM = 4: blocks 2*wk, 2*wk+1; TM = 2: block wk; TM = 1: the
+    // wk = 0 wave owns the block and its partner only hands over.
     auto finish = [&](auto wk_tag) {
         constexpr int WK = decltype(wk_tag)::value;
+        constexpr int KEEP = TM == 1 ? (WK == 0 ? 1 : 0) : TM / 2;  // row blocks kept
+        constexpr int GIVE = TM == 1 ? (WK == 1 ? 1 : 0) : TM / 2;  // row blocks handed over
+        constexpr int KEEP0 = TM == 1 ? 0 : WK * (TM / 2);          // first kept row block
+        constexpr int GIVE0 = TM == 1 ? 0 : (WK ^ 1) * (TM / 2);    // first handed-over row block
+        constexpr int XT = (TM == 1 ? 1 : TM / 2) * TN;             // tiles per exchange slot of a wave
         int* xch = reinterpret_cast<int*>(lds_raw);
         const int partner = wave ^ 4;
-        static_assert(8 * 4 * 16 * 64 * 4 <= WK_SCALES_OFF, "exchange area");
+        static_assert(8 * XT * 16 * 64 * 4 <= WK_SCALES_OFF, "exchange area");
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const v16i& give = acc[(WK ^ 1) * 2 + (t >> 1)][t & 1];
+        for (int t = 0; t < GIVE * TN; ++t) {
+            const v16i& give = acc[GIVE0 + t / TN][t % TN];
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-                *reinterpret_cast<v4i*>(xch + (((wave * 4 + t) * 4 + q) * 64 + lane) * 4) =
+                *reinterpret_cast<v4i*>(xch + (((wave * XT + t) * 4 + q) * 64 + lane) * 4) =
                     v4i{give[q * 4], give[q * 4 + 1], give[q * 4 + 2], give[q * 4 + 3]};
         }
         lds_barrier();
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            v16i& keep = acc[WK * 2 + (t >> 1)][t & 1];
+        for (int t = 0; t < KEEP * TN; ++t) {
+            v16i& keep = acc[KEEP0 + t / TN][t % TN];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const v4i got = *reinterpret_cast<const v4i*>(xch + (((partner * 4 + t) * 4 + q) * 64 + lane) * 4);
+                const v4i got = *reinterpret_cast<const v4i*>(xch + (((partner * XT + t) * 4 + q) * 64 + lane) * 4);
                 keep[q * 4] += got.x;
                 keep[q * 4 + 1] += got.y;
                 keep[q * 4 + 2] += got.z;
@@ -1452,26 +1477,59 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             }
         }
         lds_barrier();
-        uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
+
+        if (ksplit > 1) {
+            // partial tile in accumulator order: [tile][part][owning wave][kept tile][q][lane] x 4 ints
+            constexpr int OWNERS = TM == 1 ? 4 : 8;
+            constexpr int PER_WAVE = (TM == 1 ? 1 : TM / 2) * TN * 1024;
+            const int owner = TM == 1 ? wn : wave;
+            int* dst0 = g.splitk_acc + ((size_t)tile * ksplit + kpart) * (OWNERS * PER_WAVE) + owner * PER_WAVE;
 #pragma unroll
-        for (int ii = 0; ii < 2; ++ii) {
-            constexpr int i0 = WK * 2;
-            const int m0 = mblk * BM + (i0 + ii) * 32;
-            if constexpr (W4) {
+            for (int t = 0; t < KEEP * TN; ++t) {
+                const v16i& mine = acc[KEEP0 + t / TN][t % TN];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<v4i*>(dst0 + t * 1024 + (q * 64 + lane) * 4) =
+                        v4i{mine[q * 4], mine[q * 4 + 1], mine[q * 4 + 2], mine[q * 4 + 3]};
+            }
+            return;
+        }
+
+        if constexpr (KEEP > 0) {
+            float as[KEEP], ws[TN][16];
+            if constexpr (EPI != RKH_EPI_I32) {
+                const float* sc = reinterpret_cast<const float*>(lds_raw + WK_SCALES_OFF);
+#pragma unroll
+                for (int ii = 0; ii < KEEP; ++ii) as[ii] = sc[(KEEP0 + ii) * 32 + (lane & 31)];
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[i0 + ii][j][r] >>= 4;
-            }
-            const int pb0 = nblk * 8 + wn * TN;
-            if constexpr (EPI == RKH_EPI_SWIGLU) {
-                epilogue_swiglu_scaled(g, acc[i0 + ii][0], acc[i0 + ii][1], m0, pb0, lane, as[ii], ws[0], ws[1],
-                                       m_limit, stage_lds);
+                    for (int r = 0; r < 16; ++r) ws[j][r] = sc[128 + (wn * TN + j) * 32 + tile_col(r, lane)];
             } else {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    epilogue_tile_scaled<EPI>(g, acc[i0 + ii][j], m0, pb0 + j, lane, as[ii], ws[j], m_limit,
-                                              stage_lds);
+                for (int ii = 0; ii < KEEP; ++ii) as[ii] = 0.0f;
+            }
+            uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
+#pragma unroll
+            for (int ii = 0; ii < KEEP; ++ii) {
+                constexpr int i0 = KEEP0;
+                const int m0 = mblk * BM + (i0 + ii) * 32;
+                if constexpr (W4) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i0 + ii][j][r] >>= 4;
+                }
+                const int pb0 = nblk * 8 + wn * TN;
+                if constexpr (EPI == RKH_EPI_SWIGLU) {
+                    epilogue_swiglu_scaled(g, acc[i0 + ii][0], acc[i0 + ii][1], m0, pb0, lane, as[ii], ws[0], ws[1],
+                                           m_limit, stage_lds);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        epilogue_tile_scaled<EPI>(g, acc[i0 + ii][j], m0, pb0 + j, lane, as[ii], ws[j], m_limit,
+                                                  stage_lds);
+                }
             }
         }
     };
@@ -1480,42 +1538,69 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 }
 #pragma clang diagnostic pop
 
-// Epilogue over the split-K scratch matrix; re-zeroes what it consumed so the
-// scratch is clean for the next call.
-__global__ __launch_bounds__(256) void splitk_epilogue_kernel(rkh_gemm_args g, int ld) {
-    const int m = blockIdx.y;
-    const int F = g.interleave_F;
-    if (g.epilogue == RKH_EPI_SWIGLU) {
-        const int n = blockIdx.x * 256 + threadIdx.x; // middle column
-        uint32_t bits = 0;
-        if (n < F) {
-            const int pg = (n >> 5) * 2;
-            const size_t ig = (size_t)m * ld + pg * 32 + (n & 31), iu = ig + 32;
-            const int ag = g.splitk_acc[ig], au = g.splitk_acc[iu];
-            g.splitk_acc[ig] = 0;
-            g.splitk_acc[iu] = 0;
-            const float as = g.a_scale[m];
-            const float y = __fmul_rn(silu_poly(dequant(ag, as, g.w_scale[n])),
-                                      dequant(au, as, g.w_scale[F + n]));
-            static_cast<float*>(g.C)[(size_t)m * g.ldc + n] = y;
-            bits = __float_as_uint(y) & 0x7fffffffu;
-        }
-        if (g.row_max_bits) {
+// Second half of a K-split launch: workgroup = output tile, same wave -> tile
+// ownership as gemm_wk_kernel after its k-half exchange; adds the ksplit
+// partial tiles and runs the epilogue.
+template <int TM, bool W4, int EPI>
+__global__ __launch_bounds__(512) void gemm_wk_reduce_kernel(rkh_gemm_args g, int mblocks, int nblocks, int ksplit) {
+    constexpr int TN = 2, BM = 32 * TM;
+    __shared__ __attribute__((aligned(16))) uint8_t stage_all[8 * 32 * (32 * 4 + 8)];
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int wn = wave & 3, wk = wave >> 2;
+    const int tile = blockIdx.x;
+    int mblk, nblk;
+    wk_tile_coords(tile, mblocks, nblocks, mblk, nblk);
+    auto body = [&](auto wk_tag) {
+        constexpr int WK = decltype(wk_tag)::value;
+        constexpr int KEEP = TM == 1 ? (WK == 0 ? 1 : 0) : TM / 2;
+        constexpr int KEEP0 = TM == 1 ? 0 : WK * (TM / 2);
+        constexpr int OWNERS = TM == 1 ? 4 : 8;
+        constexpr int PER_WAVE = (TM == 1 ? 1 : TM / 2) * TN * 1024;
+        if constexpr (KEEP > 0) {
+            const int owner = TM == 1 ? wn : wave;
+            const int* src0 = g.splitk_acc + (size_t)tile * ksplit * (OWNERS * PER_WAVE) + owner * PER_WAVE;
+            uint8_t* stage_lds = stage_all + wave * (32 * (32 * 4 + 8));
+            const int pb0 = nblk * 8 + wn * TN;
 #pragma unroll
-            for (int off = 16; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
-            if ((threadIdx.x & 31) == 0 && n < F) g.row_max_bits[(size_t)m * (F / 32) + (n >> 5)] = bits;
+            for (int ii = 0; ii < KEEP; ++ii) {
+                v16i sum[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sum[j][r] = 0;
+                for (int p = 0; p < ksplit; ++p) {
+                    const int* src = src0 + (size_t)p * (OWNERS * PER_WAVE) + ii * TN * 1024;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const v4i got = *reinterpret_cast<const v4i*>(src + j * 1024 + (q * 64 + lane) * 4);
+                            sum[j][q * 4] += got.x;
+                            sum[j][q * 4 + 1] += got.y;
+                            sum[j][q * 4 + 2] += got.z;
+                            sum[j][q * 4 + 3] += got.w;
+                        }
+                }
+                if constexpr (W4) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) sum[j][r] >>= 4;
+                }
+                const int m0 = mblk * BM + (KEEP0 + ii) * 32;
+                if constexpr (EPI == RKH_EPI_SWIGLU) {
+                    epilogue_swiglu(g, sum[0], sum[1], m0, pb0, lane, g.a_scale, g.w_scale, g.M, stage_lds);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        epilogue_tile<EPI>(g, sum[j], m0, pb0 + j, lane, g.a_scale, g.w_scale, g.M, stage_lds);
+                }
+            }
         }
-    } else {
-        const int pc = blockIdx.x * 256 + threadIdx.x; // physical column
-        const int n = block_first_col(pc >> 5, F) + (pc & 31);
-        if (pc < ld && n < g.N && (!F || (pc >> 5) < g.N / 32)) {
-            const size_t i = (size_t)m * ld + pc;
-            const int a = g.splitk_acc[i];
-            g.splitk_acc[i] = 0;
-            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, a, g.a_scale ? g.a_scale[m] : 1.0f,
-                      g.w_scale ? g.w_scale[n] : 1.0f);
-        }
-    }
+    };
+    if (wk == 0) body(std::integral_constant<int, 0>{});
+    else body(std::integral_constant<int, 1>{});
 }
 
 // ------------------------------------------------------------- MoE route
@@ -1660,64 +1745,61 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 }
 
 // ------------------------------------------------------------- launchers
-template <int WM, int WN, int TM, int TN, int KT>
-int launch_gemm_cfg(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    const bool grouped = g.blk_expert != nullptr;
-    const int mblocks = grouped ? (g.max_blocks + BM / 32 - 1) / (BM / 32) : (g.M + BM - 1) / BM;
-    const int cols = g.N;
-    const int nblocks = (cols + BN - 1) / BN;
-    const int ksteps_total = (int)((rkh_align_up(g.K, RKH_K_ALIGN) / 32 + KT - 1) / KT);
-    if (ksplit > ksteps_total) ksplit = ksteps_total;
-    if (ksplit < 1 || grouped) ksplit = 1;
-    const int per = (ksteps_total + ksplit - 1) / ksplit;
-    ksplit = (ksteps_total + per - 1) / per;
-    const dim3 grid(mblocks * nblocks * ksplit), block(WM * WN * 64);
-#define RK_LAUNCH(W4, EPI, GR)                                                              \
-    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, KT, W4, EPI, GR>), grid, block, 0, st, g,   \
-                       mblocks, nblocks, ksplit, per)
-#define RK_BY_EPI(W4, GR)                                                  \
-    switch (g.epilogue) {                                                  \
-    case RKH_EPI_I32: RK_LAUNCH(W4, RKH_EPI_I32, GR); break;               \
-    case RKH_EPI_F16: RK_LAUNCH(W4, RKH_EPI_F16, GR); break;               \
-    case RKH_EPI_F32: RK_LAUNCH(W4, RKH_EPI_F32, GR); break;               \
-    case RKH_EPI_SWIGLU:                                                   \
-        if (TN % 2 == 0) RK_LAUNCH(W4, (TN % 2 == 0 ? RKH_EPI_SWIGLU : RKH_EPI_F32), GR); \
-        else return RKH_ERR_RUNTIME;                                       \
-        break;                                                             \
-    default: return RKH_ERR_RUNTIME;                                       \
+// Grouped (MoE) launches: 32-row blocks of the sorted rows x 256 columns, four
+// waves, one workgroup per (block, column block); several workgroups share a
+// compute unit, which suits this weight-streaming shape (every expert's
+// weights are read once).
+int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
+    constexpr int WM = 1, WN = 4, TM = 1, TN = 2, KT = 2;
+    constexpr int BN = WN * TN * 32;
+    if (g.w_int4) return RKH_ERR_RUNTIME;
+    const int mblocks = g.max_blocks;
+    const int nblocks = (g.N + BN - 1) / BN;
+    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 32 / KT);
+    const dim3 grid(mblocks * nblocks), block(WM * WN * 64);
+#define RK_LAUNCH(EPI)                                                                          \
+    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, KT, false, EPI, true>), grid, block, 0, st, g, \
+                       mblocks, nblocks, 1, ksteps_total)
+    switch (g.epilogue) {
+    case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
+    case RKH_EPI_F16: RK_LAUNCH(RKH_EPI_F16); break;
+    case RKH_EPI_F32: RK_LAUNCH(RKH_EPI_F32); break;
+    case RKH_EPI_SWIGLU: RK_LAUNCH(RKH_EPI_SWIGLU); break;
+    default: return RKH_ERR_RUNTIME;
     }
-    if (grouped) {
-        if (g.w_int4) return RKH_ERR_RUNTIME;
-        RK_BY_EPI(false, true)
-    } else if (g.w_int4) {
-        RK_BY_EPI(true, false)
-    } else {
-        RK_BY_EPI(false, false)
-    }
-#undef RK_BY_EPI
 #undef RK_LAUNCH
     RKH_CHECK(hipGetLastError());
-    if (ksplit > 1) {
-        const int ld = nblocks * BN;
-        const int width = g.epilogue == RKH_EPI_SWIGLU ? g.interleave_F : ld;
-        const dim3 egrid((width + 255) / 256, g.M);
-        hipLaunchKernelGGL(splitk_epilogue_kernel, egrid, dim3(256), 0, st, g, ld);
-        RKH_CHECK(hipGetLastError());
-    }
     return RKH_OK;
 }
 
-int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g) {
-    const int mblocks = (g.M + 127) / 128, nblocks = (g.N + 255) / 256;
-    const dim3 grid(mblocks * nblocks), block(512);
+// Bytes of split-K scratch for `tiles` output tiles of bm rows split into
+// ksplit parts: the int32 partial tiles.
+static size_t wk_scratch_bytes(long tiles, int bm, int ksplit) {
+    return ksplit > 1 ? (size_t)tiles * ksplit * bm * 256 * 4 : 0;
+}
+
+template <int TM>
+int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
+    constexpr int BM = 32 * TM, KTS = 8 / TM;
+    const int mblocks = (g.M + BM - 1) / BM;
+    const int nblocks = (g.N + 255) / 256;
+    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 32 / KTS);
+    if (ksplit > ksteps_total) ksplit = ksteps_total;
+    if (ksplit < 1) ksplit = 1;
+    const int per = (ksteps_total + ksplit - 1) / ksplit;
+    ksplit = (ksteps_total + per - 1) / per; // no empty part
+    const dim3 grid(mblocks * nblocks * ksplit), block(512);
 #define RK_WK(W4, EPI)                                                                              \
     do {                                                                                            \
         static const hipError_t attr = hipFuncSetAttribute(                                         \
-            reinterpret_cast<const void*>(&gemm_wk_kernel<W4, EPI>),                                \
+            reinterpret_cast<const void*>(&gemm_wk_kernel<TM, W4, EPI>),                            \
             hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES);                              \
         RKH_CHECK(attr);                                                                            \
-        hipLaunchKernelGGL((gemm_wk_kernel<W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, nblocks); \
+        hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, \
+                           nblocks, ksplit, per);                                                   \
+        if (ksplit > 1)                                                                             \
+            hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>), dim3(mblocks * nblocks), block, 0, st, g, \
+                               mblocks, nblocks, ksplit);                                           \
     } while (0)
 #define RK_WK_EPI(W4)                                           \
     switch (g.epilogue) {                                       \
@@ -1933,33 +2015,47 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
 
 // Dense launch plan: rows per workgroup follow M, shrinking while the output
 // grid cannot fill the 256 compute units; what is still missing is made up by
-// splitting K (exact: integer partial sums are added atomically).
-// int4 operands ride as 16 * code, so one K part may span at most 2^17 k
-// before the int32 sum could wrap.
+// splitting K over workgroups (exact: integer partial tiles are added by the
+// last part to arrive).  int4 operands ride as 16 * code, so one K part may
+// span at most 2^17 k before the int32 sum could wrap.
 struct DensePlan { int bm, ksplit; };
 static int min_ksplit(int K, int w_int4) {
     return w_int4 ? (int)((rkh_align_up(K, RKH_K_ALIGN) + 131071) / 131072) : 1;
 }
+static long dense_tiles(int M, int N, int bm) { return (long)((M + bm - 1) / bm) * ((N + 255) / 256); }
 static DensePlan dense_plan(int M, int N, int K, int w_int4) {
-    const int ksteps = (int)(rkh_align_up(K, RKH_K_ALIGN) / 64);
+    const int kp = (int)rkh_align_up(K, RKH_K_ALIGN);
     int bm = M > 64 ? 128 : M > 32 ? 64 : 32;
-    auto tiles_of = [&](int rows) { return (long)((M + rows - 1) / rows) * ((N + 255) / 256); };
-    while (bm > 32 && tiles_of(bm) < 160) bm >>= 1;
-    const long tiles = tiles_of(bm);
+    while (bm > 32 && dense_tiles(M, N, bm) < 160) bm >>= 1;
+    const long tiles = dense_tiles(M, N, bm);
     int s = 1;
-    if (tiles < 192 && bm < 128) { // 128-row tiles are only chosen when they fill most of the chip
+    if (tiles < 160) {
         s = (int)((256 + tiles - 1) / tiles);
-        const int max_s = ksteps / 8 > 0 ? ksteps / 8 : 1; // at least 512 k per part
+        const int max_s = kp / 1024 > 0 ? kp / 1024 : 1; // at least 1024 k per part
         if (s > max_s) s = max_s;
     }
     const int need = min_ksplit(K, w_int4);
     return {bm, s > need ? s : need};
 }
+// RK_NPU_HIP_GEMM_PLAN="rows:ksplit" forces the workgroup tile rows (32 / 64 /
+// 128) and the K split of dense launches (tuning aid).
+static DensePlan effective_plan(int M, int N, int K, int w_int4) {
+    DensePlan plan = dense_plan(M, N, K, w_int4);
+    static const char* forced = getenv("RK_NPU_HIP_GEMM_PLAN");
+    if (forced) {
+        int rows = 0, split = 0;
+        if (sscanf(forced, "%d:%d", &rows, &split) == 2 && (rows == 32 || rows == 64 || rows == 128) && split >= 1) {
+            plan.bm = rows;
+            plan.ksplit = split > min_ksplit(K, w_int4) ? split : min_ksplit(K, w_int4);
+        }
+    }
+    return plan;
+}
 
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
     if (M <= 8) return 0;
-    if (dense_plan(M, N, K, w_int4).ksplit <= 1) return 0;
-    return (size_t)rkh_align_up(M, RKH_ROW_ALIGN) * (size_t)rkh_align_up(N, RKH_COL_ALIGN) * 4;
+    const DensePlan plan = effective_plan(M, N, K, w_int4);
+    return wk_scratch_bytes(dense_tiles(M, N, plan.bm), plan.bm, plan.ksplit);
 }
 
 int rkh_gemm(void* stream, const rkh_gemm_args* args) {
@@ -1967,28 +2063,16 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     hipStream_t st = (hipStream_t)stream;
     const bool grouped = g.blk_expert != nullptr;
     if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) return dispatch_gemv(st, g, nullptr);
-    if (grouped) return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, 1);
-    DensePlan plan = dense_plan(g.M, g.N, g.K, g.w_int4);
-    // Tuning aid: RK_NPU_HIP_GEMM_PLAN="rows:ksplit" forces the workgroup tile
-    // rows (32 / 64 / 128) and the K split of dense launches.
-    static const char* forced = getenv("RK_NPU_HIP_GEMM_PLAN");
-    if (forced) {
-        int rows = 0, split = 0;
-        if (sscanf(forced, "%d:%d", &rows, &split) == 2 && (rows == 32 || rows == 64 || rows == 128) && split >= 1) {
-            plan.bm = rows;
-            plan.ksplit = split > min_ksplit(g.K, g.w_int4) ? split : min_ksplit(g.K, g.w_int4);
-        }
-    }
+    if (grouped) return launch_gemm_grouped(st, g);
+    const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {
         if (min_ksplit(g.K, g.w_int4) > 1) return RKH_ERR_RUNTIME;
         ksplit = 1;
     }
-    const int bm = plan.bm;
-    if (bm == 128 && ksplit == 1) return launch_gemm_wk(st, g);
-    if (bm == 128) return launch_gemm_cfg<2, 4, 2, 2, 2>(st, g, ksplit);
-    if (bm == 64) return launch_gemm_cfg<1, 4, 2, 2, 2>(st, g, ksplit);
-    return launch_gemm_cfg<1, 4, 1, 2, 2>(st, g, ksplit);
+    if (plan.bm == 128) return launch_gemm_wk<4>(st, g, ksplit);
+    if (plan.bm == 64) return launch_gemm_wk<2>(st, g, ksplit);
+    return launch_gemm_wk<1>(st, g, ksplit);
 }
 
 int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_args* gargs) {
