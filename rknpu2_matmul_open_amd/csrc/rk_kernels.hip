@@ -507,7 +507,7 @@ __device__ __forceinline__ void store_out(void* C, int epi, size_t index, int ac
 // halves of a k-tile for column l%32, so the cross-lane reduction is one xor
 // shuffle, followed by a small LDS reduction across waves.
 constexpr int GEMV_WAVES = 8;
-constexpr int GEMV_UNROLL = 4;
+constexpr int GEMV_UNROLL = 8;
 constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
 
 constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
