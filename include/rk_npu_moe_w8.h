@@ -116,6 +116,47 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
                           const int32_t* expert_ids, const float* route_weights,
                           float* output, rk_npu_moe_w8_timings* timings);
 
+/* ---- other expert formats of the reference (reference :83-143) ---------------
+ * W4 experts, mixed routed-W4 + shared-W8 experts, mutable slot banks and the
+ * packed expert record import / export exist in the reference for the RK3588
+ * NPU's int4 mode and its expert paging.  They are outside this build's path:
+ * the entry points are exported so that callers link, and every one of them
+ * declines -- constructors return NULL, the record calls return
+ * RK_NPU_ERR_PARAM, the record size query returns 0 -- without touching the
+ * device or the caller's buffers. */
+#define RK_NPU_MOE_QUANT_BLOB_VERSION 3u
+typedef struct rk_npu_moe_import_timings {
+    double copy_us, validate_us, gate_sync_us, down_sync_us, total_us;
+} rk_npu_moe_import_timings;
+
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create(rk_npu_iommu_domain* domain,
+                                                       const rk_npu_moe_w8_weight_config* config,
+                                                       const rk_npu_moe_w8_expert* experts);
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create_full_k(rk_npu_iommu_domain* domain,
+                                                              const rk_npu_moe_w8_weight_config* config,
+                                                              const rk_npu_moe_w8_expert* experts);
+rk_npu_moe_w8_workspace* rk_npu_moe_quant_workspace_create(rk_npu_iommu_domain* domain,
+                                                           const rk_npu_moe_w8_config* config);
+rk_npu_moe_w8_weights* rk_npu_moe_w4_weights_create(rk_npu_iommu_domain* domain,
+                                                    const rk_npu_moe_w8_weight_config* config,
+                                                    const rk_npu_moe_w8_expert* experts);
+rk_npu_moe_w8_workspace* rk_npu_moe_w4_workspace_create(rk_npu_iommu_domain* domain,
+                                                        const rk_npu_moe_w8_config* config);
+rk_npu_moe_w8_weights* rk_npu_moe_w4_slots_create(rk_npu_iommu_domain* domain,
+                                                  const rk_npu_moe_w8_weight_config* config,
+                                                  const rk_npu_moe_w8_expert* shared);
+rk_npu_moe_w8_weights* rk_npu_moe_quant_slots_create(rk_npu_iommu_domain* domain,
+                                                     const rk_npu_moe_w8_weight_config* config);
+uint64_t rk_npu_moe_quant_expert_blob_bytes(const rk_npu_moe_w8_weights* weights);
+int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights* weights, int expert, void* data,
+                                   uint64_t bytes);
+int rk_npu_moe_quant_import_expert(rk_npu_moe_w8_weights* weights, int slot, const void* data,
+                                   uint64_t bytes);
+int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights* weights, int slot, const void* data,
+                                         uint64_t bytes, rk_npu_moe_import_timings* timings);
+int rk_npu_moe_quant_swap_slots(rk_npu_moe_w8_weights* first, int first_slot,
+                                rk_npu_moe_w8_weights* second, int second_slot);
+
 #ifdef __cplusplus
 }
 #endif

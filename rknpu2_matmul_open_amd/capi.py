@@ -195,6 +195,19 @@ _PROTOTYPES = {
     "rk_npu_moe_w8_workspace_device_bytes": (C.c_uint64, [P]),
     "rk_npu_moe_w8_run_quantized": (C.c_int, [P, P, C.c_int, P, P, P, P, P, C.POINTER(MoeTimings)]),
     "rk_npu_moe_w8_run_f32": (C.c_int, [P, P, C.c_int, P, P, P, P, C.POINTER(MoeTimings)]),
+    # other expert formats: exported, always declining
+    "rk_npu_moe_quant_weights_create": (P, [P, C.POINTER(MoeWeightConfig), C.POINTER(MoeExpert)]),
+    "rk_npu_moe_quant_weights_create_full_k": (P, [P, C.POINTER(MoeWeightConfig), C.POINTER(MoeExpert)]),
+    "rk_npu_moe_quant_workspace_create": (P, [P, C.POINTER(MoeConfig)]),
+    "rk_npu_moe_w4_weights_create": (P, [P, C.POINTER(MoeWeightConfig), C.POINTER(MoeExpert)]),
+    "rk_npu_moe_w4_workspace_create": (P, [P, C.POINTER(MoeConfig)]),
+    "rk_npu_moe_w4_slots_create": (P, [P, C.POINTER(MoeWeightConfig), C.POINTER(MoeExpert)]),
+    "rk_npu_moe_quant_slots_create": (P, [P, C.POINTER(MoeWeightConfig)]),
+    "rk_npu_moe_quant_expert_blob_bytes": (C.c_uint64, [P]),
+    "rk_npu_moe_quant_export_expert": (C.c_int, [P, C.c_int, P, C.c_uint64]),
+    "rk_npu_moe_quant_import_expert": (C.c_int, [P, C.c_int, P, C.c_uint64]),
+    "rk_npu_moe_quant_import_expert_timed": (C.c_int, [P, C.c_int, P, C.c_uint64, P]),
+    "rk_npu_moe_quant_swap_slots": (C.c_int, [P, C.c_int, P, C.c_int]),
     # rk_npu_hip.h
     "rk_npu_hip_stream": (P, [P]),
     "rk_npu_hip_device": (C.c_int, [P]),

@@ -11,6 +11,7 @@
 #include <algorithm>
 #include <new>
 
+#include <cerrno>
 #include "rk_host.h"
 #include "rk_npu_hip.h"
 #include "rk_npu_moe_w8.h"
@@ -392,6 +393,50 @@ rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* dom
 }
 
 void rk_npu_moe_w8_workspace_free(rk_npu_moe_w8_workspace* workspace) { delete workspace; }
+
+// ---- expert formats outside this build's path: exported, always declining ----
+// (reference src/rk_npu_moe_w8.cpp:885-999 implements them for the NPU's int4 mode)
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
+                                                       const rk_npu_moe_w8_expert*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create_full_k(rk_npu_iommu_domain*,
+                                                              const rk_npu_moe_w8_weight_config*,
+                                                              const rk_npu_moe_w8_expert*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_workspace* rk_npu_moe_quant_workspace_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_config*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_weights* rk_npu_moe_w4_weights_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
+                                                    const rk_npu_moe_w8_expert*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_workspace* rk_npu_moe_w4_workspace_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_config*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_weights* rk_npu_moe_w4_slots_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
+                                                  const rk_npu_moe_w8_expert*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+rk_npu_moe_w8_weights* rk_npu_moe_quant_slots_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*) {
+    errno = ENOTSUP;
+    return nullptr;
+}
+uint64_t rk_npu_moe_quant_expert_blob_bytes(const rk_npu_moe_w8_weights*) { return 0; }
+int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights*, int, void*, uint64_t) { return RK_NPU_ERR_PARAM; }
+int rk_npu_moe_quant_import_expert(rk_npu_moe_w8_weights*, int, const void*, uint64_t) { return RK_NPU_ERR_PARAM; }
+int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights*, int, const void*, uint64_t,
+                                         rk_npu_moe_import_timings*) {
+    return RK_NPU_ERR_PARAM;
+}
+int rk_npu_moe_quant_swap_slots(rk_npu_moe_w8_weights*, int, rk_npu_moe_w8_weights*, int) { return RK_NPU_ERR_PARAM; }
 
 uint64_t rk_npu_moe_w8_weights_device_bytes(const rk_npu_moe_w8_weights* w) {
     return w ? w->bytes() : 0;

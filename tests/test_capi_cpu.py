@@ -9,6 +9,7 @@ import re
 import subprocess
 import sys
 
+import numpy as np
 import pytest
 
 from rknpu2_matmul_open_amd import capi
@@ -227,6 +228,27 @@ def test_open_without_device_fails_cleanly(lib):
     assert lib.rk_npu_i8i8i32_run(None, None, None, None) == capi.RK_NPU_ERR_PARAM
     assert lib.rk_npu_w4a8_run_f32(None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
     assert lib.rk_npu_moe_w8_run_f32(None, None, 1, None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
+
+
+def test_other_moe_expert_formats_decline(lib):
+    """W4 / mixed / slot-bank / packed-record entry points of the reference
+    (include/rk_npu_moe_w8.h:83-143) link and decline without touching buffers."""
+    cfg = capi.MoeWeightConfig(64, 32, 3, 1)
+    full = capi.MoeConfig()
+    lib.rk_npu_moe_w8_config_init(C.byref(full), 64, 32, 3, 1, 2, 8)
+    for fn in (lib.rk_npu_moe_quant_weights_create, lib.rk_npu_moe_quant_weights_create_full_k,
+               lib.rk_npu_moe_w4_weights_create, lib.rk_npu_moe_w4_slots_create):
+        assert not fn(None, C.byref(cfg), None)
+    assert not lib.rk_npu_moe_quant_slots_create(None, C.byref(cfg))
+    assert not lib.rk_npu_moe_quant_workspace_create(None, C.byref(full))
+    assert not lib.rk_npu_moe_w4_workspace_create(None, C.byref(full))
+    assert lib.rk_npu_moe_quant_expert_blob_bytes(None) == 0
+    buf = np.full(64, 7, np.uint8)
+    assert lib.rk_npu_moe_quant_export_expert(None, 0, capi.ptr(buf), 64) == capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_moe_quant_import_expert(None, 0, capi.ptr(buf), 64) == capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_moe_quant_import_expert_timed(None, 0, capi.ptr(buf), 64, None) == capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_moe_quant_swap_slots(None, 0, None, 0) == capi.RK_NPU_ERR_PARAM
+    assert (buf == 7).all()
 
 
 def test_package_fails_loudly_without_the_library(monkeypatch, tmp_path):
