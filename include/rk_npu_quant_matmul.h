@@ -83,6 +83,23 @@ typedef struct rk_npu_matmul_weight_config {
     int k_tile; /* 1..K */
 } rk_npu_matmul_weight_config;
 
+/* reference :101-115.  One K partition is chosen for all m_values (distinct,
+ * > 0); frequencies (finite, > 0) weight the summary, NULL = equal weights. */
+typedef struct rk_npu_matmul_family_autotune_config {
+    int K;
+    int N;
+    int m_count;
+    const int* m_values;
+    const double* frequencies;
+    uint32_t allowed_npu_core_mask;
+    uint64_t allowed_cpu_core_mask;
+    int warmup;
+    int loops;
+    int repeats;
+    uint32_t timeout_ms;
+    int verbose;
+} rk_npu_matmul_family_autotune_config;
+
 /* reference :117-147 */
 typedef struct rk_npu_matmul_strategy {
     rk_npu_matmul_op_kind op_kind;
@@ -113,6 +130,13 @@ typedef struct rk_npu_f16i8f16_weights rk_npu_f16i8f16_weights;
 typedef struct rk_npu_f32i8f32_weights rk_npu_f32i8f32_weights;
 typedef struct rk_npu_matmul_workspace rk_npu_matmul_workspace;
 
+/* reference :154-158 */
+typedef struct rk_npu_matmul_family_summary {
+    rk_npu_matmul_weight_config weight_config;
+    double weighted_total_us;
+    double weighted_robust_us;
+} rk_npu_matmul_family_summary;
+
 /* reference :161-176.  The byte counts reproduce the reference's logical
  * payload formulas (they describe the RK3588 buffers a caller would have
  * budgeted for), not the HBM footprint of this build. */
@@ -138,9 +162,101 @@ typedef struct rk_npu_matmul_weight_requirements {
 void rk_npu_matmul_autotune_config_init(rk_npu_matmul_autotune_config* cfg,
                                         int M, int N, int K);
 
+/* Defaults {K, N, m_count, m_values, frequencies NULL, npu mask 7, cpu mask 0,
+ * warmup 2, loops 8, repeats 3, timeout 500 ms, verbose 0} (reference :182-184). */
+void rk_npu_matmul_family_autotune_config_init(rk_npu_matmul_family_autotune_config* cfg, int N,
+                                               int K, int m_count, const int* m_values);
+
 /* CPU-only policy query kept for callers that probe K partitions before
  * creating weights (reference :188). */
 int rk_npu_matmul_k_partition_query(int M, int K, int k_tile);
+
+/* Tuning (reference :190-215).  The reference searches NPU tile sizes and
+ * layouts; those knobs do not change what this build executes, so each call
+ * returns one canonical strategy -- core / CPU masks fixed from the allowed
+ * masks exactly as the reference fixes them, k_tile = required_k_tile or
+ * min(K, 2048), the widest safe n_tile, plain layouts -- whose total_us /
+ * robust_us are measured: the blocking host API is timed on seeded synthetic
+ * tensors with cfg's warmup / loops / repeats.  `fastest` and `stable` receive
+ * the same strategy; either may be NULL, not both. */
+int rk_npu_i8i8i32_autotune(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                            rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable);
+int rk_npu_f16i8f16_dynamic_autotune(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                                     rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable);
+int rk_npu_f16i8f16_static_autotune(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                                    rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable);
+int rk_npu_f32i8f32_dynamic_autotune(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                                     rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable);
+int rk_npu_f32i8f32_static_autotune(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                                    rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable);
+
+/* Result cache (reference :217-251).  One text file holds both strategies and
+ * the key (op kind, shape, normalised masks, measurement settings,
+ * required_k_tile, backend environment switches).  Load returns
+ * RK_NPU_ERR_CACHE_MISS when the file is absent, malformed or keyed
+ * differently; save writes a temporary file and renames it.  `cached` loads or
+ * tunes-and-saves; NULL cache_path = $XDG_CACHE_HOME/rk_npu_matmul or
+ * $HOME/.cache/rk_npu_matmul with a name derived from the key; refresh != 0
+ * skips the load; a failed save never hides a good result; cache_hit is
+ * optional.  The file format is this library's own (not readable by the
+ * reference and vice versa). */
+int rk_npu_matmul_autotune_cache_load(rk_npu_ctx* ctx, const char* cache_path,
+                                      rk_npu_matmul_op_kind kind,
+                                      const rk_npu_matmul_autotune_config* cfg,
+                                      rk_npu_matmul_strategy* fastest,
+                                      rk_npu_matmul_strategy* stable);
+int rk_npu_matmul_autotune_cache_save(rk_npu_ctx* ctx, const char* cache_path,
+                                      rk_npu_matmul_op_kind kind,
+                                      const rk_npu_matmul_autotune_config* cfg,
+                                      const rk_npu_matmul_strategy* fastest,
+                                      const rk_npu_matmul_strategy* stable);
+int rk_npu_matmul_autotune_cached(rk_npu_ctx* ctx, const rk_npu_matmul_autotune_config* cfg,
+                                  rk_npu_matmul_op_kind kind, const char* cache_path, int refresh,
+                                  rk_npu_matmul_strategy* fastest, rk_npu_matmul_strategy* stable,
+                                  int* cache_hit);
+
+/* Family tuning (reference :253-294): one K partition for all M values;
+ * strategy arrays have m_count entries in m_values order; a summary and its
+ * array are both NULL or both non-NULL, at least one pair is required.  The
+ * cached form keeps one single-M cache file per M in cache_directory (NULL =
+ * the per-user default) and counts hits / misses. */
+int rk_npu_i8i8i32_autotune_family(rk_npu_ctx* ctx, const rk_npu_matmul_family_autotune_config* cfg,
+                                   rk_npu_matmul_family_summary* fastest_summary,
+                                   rk_npu_matmul_strategy* fastest_strategies,
+                                   rk_npu_matmul_family_summary* stable_summary,
+                                   rk_npu_matmul_strategy* stable_strategies);
+int rk_npu_f16i8f16_dynamic_autotune_family(rk_npu_ctx* ctx,
+                                            const rk_npu_matmul_family_autotune_config* cfg,
+                                            rk_npu_matmul_family_summary* fastest_summary,
+                                            rk_npu_matmul_strategy* fastest_strategies,
+                                            rk_npu_matmul_family_summary* stable_summary,
+                                            rk_npu_matmul_strategy* stable_strategies);
+int rk_npu_f16i8f16_static_autotune_family(rk_npu_ctx* ctx,
+                                           const rk_npu_matmul_family_autotune_config* cfg,
+                                           rk_npu_matmul_family_summary* fastest_summary,
+                                           rk_npu_matmul_strategy* fastest_strategies,
+                                           rk_npu_matmul_family_summary* stable_summary,
+                                           rk_npu_matmul_strategy* stable_strategies);
+int rk_npu_f32i8f32_dynamic_autotune_family(rk_npu_ctx* ctx,
+                                            const rk_npu_matmul_family_autotune_config* cfg,
+                                            rk_npu_matmul_family_summary* fastest_summary,
+                                            rk_npu_matmul_strategy* fastest_strategies,
+                                            rk_npu_matmul_family_summary* stable_summary,
+                                            rk_npu_matmul_strategy* stable_strategies);
+int rk_npu_f32i8f32_static_autotune_family(rk_npu_ctx* ctx,
+                                           const rk_npu_matmul_family_autotune_config* cfg,
+                                           rk_npu_matmul_family_summary* fastest_summary,
+                                           rk_npu_matmul_strategy* fastest_strategies,
+                                           rk_npu_matmul_family_summary* stable_summary,
+                                           rk_npu_matmul_strategy* stable_strategies);
+int rk_npu_matmul_autotune_family_cached(rk_npu_ctx* ctx,
+                                         const rk_npu_matmul_family_autotune_config* cfg,
+                                         rk_npu_matmul_op_kind kind, const char* cache_directory,
+                                         int refresh, rk_npu_matmul_family_summary* fastest_summary,
+                                         rk_npu_matmul_strategy* fastest_strategies,
+                                         rk_npu_matmul_family_summary* stable_summary,
+                                         rk_npu_matmul_strategy* stable_strategies, int* cache_hits,
+                                         int* cache_misses);
 
 /* Logical byte accounting (reference :301-312). */
 int rk_npu_matmul_workspace_memory_query(const rk_npu_matmul_strategy* strategy,
@@ -203,6 +319,16 @@ rk_npu_f32i8f32_weights* rk_npu_f32i8f32_weights_create_compress(
 /* Always 0: no compressed layouts exist in this build (reference :398-399). */
 uint64_t rk_npu_f32i8f32_weights_compressed_layout_generation(
     const rk_npu_f32i8f32_weights* weights);
+
+/* fp32 weights quantized under a bits-per-weight budget for the NPU's lossless
+ * weight decompressor (reference :351-359,400-402).  That storage format does
+ * not exist here: both constructors report the budget search as unmet (NULL). */
+rk_npu_f16i8f16_weights* rk_npu_f16i8f16_weights_create_from_f32_compress(
+    rk_npu_iommu_domain* domain, const rk_npu_matmul_weight_config* config, const float* B_rowmajor,
+    float target_bpw);
+rk_npu_f32i8f32_weights* rk_npu_f32i8f32_weights_create_from_f32_compress(
+    rk_npu_iommu_domain* domain, const rk_npu_matmul_weight_config* config, const float* B_rowmajor,
+    float target_bpw);
 void rk_npu_f32i8f32_weights_free(rk_npu_f32i8f32_weights* weights);
 int rk_npu_f32i8f32_run_dynamic(rk_npu_matmul_workspace* workspace,
                                 const rk_npu_f32i8f32_weights* weights,

@@ -45,6 +45,18 @@ class MatmulWeightConfig(C.Structure):
     _fields_ = [("K", C.c_int), ("N", C.c_int), ("k_tile", C.c_int)]
 
 
+class MatmulFamilyAutotuneConfig(C.Structure):
+    _fields_ = [("K", C.c_int), ("N", C.c_int), ("m_count", C.c_int), ("m_values", C.POINTER(C.c_int)),
+                ("frequencies", C.POINTER(C.c_double)), ("allowed_npu_core_mask", C.c_uint32),
+                ("allowed_cpu_core_mask", C.c_uint64), ("warmup", C.c_int), ("loops", C.c_int),
+                ("repeats", C.c_int), ("timeout_ms", C.c_uint32), ("verbose", C.c_int)]
+
+
+class MatmulFamilySummary(C.Structure):
+    _fields_ = [("weight_config", MatmulWeightConfig), ("weighted_total_us", C.c_double),
+                ("weighted_robust_us", C.c_double)]
+
+
 class MatmulStrategy(C.Structure):
     _fields_ = [("op_kind", C.c_int), ("M", C.c_int), ("N", C.c_int), ("K", C.c_int),
                 ("k_tile", C.c_int), ("n_tile", C.c_int), ("a_layout", C.c_int),
@@ -149,6 +161,26 @@ _PROTOTYPES = {
     # rk_npu_quant_matmul.h
     "rk_npu_matmul_autotune_config_init": (None, [C.POINTER(MatmulAutotuneConfig), C.c_int, C.c_int, C.c_int]),
     "rk_npu_matmul_k_partition_query": (C.c_int, [C.c_int, C.c_int, C.c_int]),
+    "rk_npu_matmul_family_autotune_config_init": (None, [C.POINTER(MatmulFamilyAutotuneConfig), C.c_int, C.c_int,
+                                                         C.c_int, C.POINTER(C.c_int)]),
+    "rk_npu_i8i8i32_autotune": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_f16i8f16_dynamic_autotune": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_f16i8f16_static_autotune": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_f32i8f32_dynamic_autotune": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_f32i8f32_static_autotune": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_matmul_autotune_cache_load": (C.c_int, [P, C.c_char_p, C.c_int, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_matmul_autotune_cache_save": (C.c_int, [P, C.c_char_p, C.c_int, C.POINTER(MatmulAutotuneConfig), P, P]),
+    "rk_npu_matmul_autotune_cached": (C.c_int, [P, C.POINTER(MatmulAutotuneConfig), C.c_int, C.c_char_p, C.c_int, P, P,
+                                                C.POINTER(C.c_int)]),
+    "rk_npu_i8i8i32_autotune_family": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), P, P, P, P]),
+    "rk_npu_f16i8f16_dynamic_autotune_family": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), P, P, P, P]),
+    "rk_npu_f16i8f16_static_autotune_family": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), P, P, P, P]),
+    "rk_npu_f32i8f32_dynamic_autotune_family": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), P, P, P, P]),
+    "rk_npu_f32i8f32_static_autotune_family": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), P, P, P, P]),
+    "rk_npu_matmul_autotune_family_cached": (C.c_int, [P, C.POINTER(MatmulFamilyAutotuneConfig), C.c_int, C.c_char_p,
+                                                       C.c_int, P, P, P, P, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "rk_npu_f16i8f16_weights_create_from_f32_compress": (P, [P, C.POINTER(MatmulWeightConfig), P, C.c_float]),
+    "rk_npu_f32i8f32_weights_create_from_f32_compress": (P, [P, C.POINTER(MatmulWeightConfig), P, C.c_float]),
     "rk_npu_matmul_workspace_memory_query": (C.c_int, [C.POINTER(MatmulStrategy), C.POINTER(WorkspaceRequirements)]),
     "rk_npu_i8i8i32_weights_memory_query": (C.c_int, [C.POINTER(MatmulWeightConfig), C.POINTER(WeightRequirements)]),
     "rk_npu_f16i8f16_weights_memory_query": (C.c_int, [C.POINTER(MatmulWeightConfig), C.POINTER(WeightRequirements)]),

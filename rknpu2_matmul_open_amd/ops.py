@@ -129,12 +129,13 @@ class W8A8Linear:
                capi.F16I8F16_STATIC: "rk_npu_f16i8f16", capi.F32I8F32_DYNAMIC: "rk_npu_f32i8f32",
                capi.F32I8F32_STATIC: "rk_npu_f32i8f32"}
 
-    def __init__(self, sess, kind, M, B, w_scale=None, k_tile=None):
+    def __init__(self, sess, kind, M, B, w_scale=None, k_tile=None, strategy=None):
         self.s, self.kind, self.M = sess, kind, M
         self.K, self.N = B.shape
         lib = sess.lib
         self.prefix = self._CREATE[kind]
-        self.strategy = default_strategy(kind, M, self.N, self.K, k_tile)
+        # `strategy`: a rk_npu_matmul_strategy value, e.g. one returned by the tuning calls
+        self.strategy = strategy if strategy is not None else default_strategy(kind, M, self.N, self.K, k_tile)
         wc = capi.MatmulWeightConfig(self.K, self.N, self.strategy.k_tile)
         B = np.ascontiguousarray(B, np.int8)
         create = getattr(lib, self.prefix + "_weights_create")

@@ -57,6 +57,8 @@ def test_library_exports_every_declared_function(lib):
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     pairs = [("rk_npu_matmul_strategy", capi.MatmulStrategy), ("rk_npu_matmul_autotune_config", capi.MatmulAutotuneConfig),
              ("rk_npu_matmul_weight_config", capi.MatmulWeightConfig),
+             ("rk_npu_matmul_family_autotune_config", capi.MatmulFamilyAutotuneConfig),
+             ("rk_npu_matmul_family_summary", capi.MatmulFamilySummary),
              ("rk_npu_matmul_workspace_requirements", capi.WorkspaceRequirements),
              ("rk_npu_matmul_weight_requirements", capi.WeightRequirements),
              ("rk_npu_i4_weight_config", capi.I4WeightConfig), ("rk_npu_i4_memory_info", capi.I4MemoryInfo),
@@ -228,6 +230,37 @@ def test_open_without_device_fails_cleanly(lib):
     assert lib.rk_npu_i8i8i32_run(None, None, None, None) == capi.RK_NPU_ERR_PARAM
     assert lib.rk_npu_w4a8_run_f32(None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
     assert lib.rk_npu_moe_w8_run_f32(None, None, 1, None, None, None, None, None) == capi.RK_NPU_ERR_PARAM
+
+
+def test_autotune_entry_points_without_a_context(lib):
+    """reference src/rk_npu_quant_matmul.cpp:1536-1550 (family defaults) and the
+    argument checks every tuning / cache call makes before touching a device."""
+    ms = (C.c_int * 2)(1, 128)
+    fam = capi.MatmulFamilyAutotuneConfig()
+    lib.rk_npu_matmul_family_autotune_config_init(C.byref(fam), 96, 64, 2, ms)
+    assert (fam.K, fam.N, fam.m_count, fam.allowed_npu_core_mask, fam.allowed_cpu_core_mask) == (64, 96, 2, 7, 0)
+    assert (fam.warmup, fam.loops, fam.repeats, fam.timeout_ms, fam.verbose) == (2, 8, 3, 500, 0)
+    assert not fam.frequencies and fam.m_values[1] == 128
+    lib.rk_npu_matmul_family_autotune_config_init(None, 1, 1, 0, None)
+    cfg = capi.MatmulAutotuneConfig()
+    lib.rk_npu_matmul_autotune_config_init(C.byref(cfg), 4, 96, 64)
+    s1, s2 = capi.MatmulStrategy(), capi.MatmulStrategy()
+    P = capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_i8i8i32_autotune(None, C.byref(cfg), C.byref(s1), C.byref(s2)) == P
+    assert lib.rk_npu_matmul_autotune_cache_load(None, b"/tmp/x.tune", 0, C.byref(cfg), C.byref(s1), C.byref(s2)) == P
+    assert lib.rk_npu_matmul_autotune_cache_save(None, b"/tmp/x.tune", 0, C.byref(cfg), C.byref(s1), C.byref(s2)) == P
+    assert lib.rk_npu_matmul_autotune_cached(None, C.byref(cfg), 0, None, 0, C.byref(s1), C.byref(s2), None) == P
+    summ = capi.MatmulFamilySummary()
+    arr = (capi.MatmulStrategy * 2)()
+    assert lib.rk_npu_f16i8f16_dynamic_autotune_family(None, C.byref(fam), C.byref(summ), arr, None, None) == P
+    hits, misses = C.c_int(5), C.c_int(5)
+    assert lib.rk_npu_matmul_autotune_family_cached(None, C.byref(fam), 1, None, 0, C.byref(summ), arr, None, None,
+                                                    C.byref(hits), C.byref(misses)) == P
+    assert (hits.value, misses.value) == (0, 0)
+    wc = capi.MatmulWeightConfig(64, 96, 64)
+    w = np.zeros((64, 96), np.float32)
+    assert not lib.rk_npu_f16i8f16_weights_create_from_f32_compress(None, C.byref(wc), capi.ptr(w), 4.0)
+    assert not lib.rk_npu_f32i8f32_weights_create_from_f32_compress(None, C.byref(wc), capi.ptr(w), 4.0)
 
 
 def test_other_moe_expert_formats_decline(lib):
