@@ -1538,69 +1538,60 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 }
 #pragma clang diagnostic pop
 
-// Second half of a K-split launch: workgroup = output tile, same wave -> tile
-// ownership as gemm_wk_kernel after its k-half exchange; adds the ksplit
+// Second half of a K-split launch.  Workgroup = one wave = one owner of kept
+// tiles of an output tile (the wave -> tile ownership gemm_wk_kernel has after
+// its k-half exchange): blockIdx.x = tile * OWNERS + owner.  Adds the ksplit
 // partial tiles and runs the epilogue.
 template <int TM, bool W4, int EPI>
-__global__ __launch_bounds__(512) void gemm_wk_reduce_kernel(rkh_gemm_args g, int mblocks, int nblocks, int ksplit) {
+__global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int mblocks, int nblocks, int ksplit) {
     constexpr int TN = 2, BM = 32 * TM;
-    __shared__ __attribute__((aligned(16))) uint8_t stage_all[8 * 32 * (32 * 4 + 8)];
+    constexpr int OWNERS = TM == 1 ? 4 : 8;
+    constexpr int KEEP = TM == 1 ? 1 : TM / 2;             // row blocks per owner
+    constexpr int PER_WAVE = KEEP * TN * 1024;
+    __shared__ __attribute__((aligned(16))) uint8_t stage_lds[32 * (32 * 4 + 8)];
     const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
-    const int wn = wave & 3, wk = wave >> 2;
-    const int tile = blockIdx.x;
+    const int tile = blockIdx.x / OWNERS, owner = blockIdx.x % OWNERS;
+    const int wn = owner & 3, wk = owner >> 2;             // TM == 1: owners are the wk == 0 waves
     int mblk, nblk;
     wk_tile_coords(tile, mblocks, nblocks, mblk, nblk);
-    auto body = [&](auto wk_tag) {
-        constexpr int WK = decltype(wk_tag)::value;
-        constexpr int KEEP = TM == 1 ? (WK == 0 ? 1 : 0) : TM / 2;
-        constexpr int KEEP0 = TM == 1 ? 0 : WK * (TM / 2);
-        constexpr int OWNERS = TM == 1 ? 4 : 8;
-        constexpr int PER_WAVE = (TM == 1 ? 1 : TM / 2) * TN * 1024;
-        if constexpr (KEEP > 0) {
-            const int owner = TM == 1 ? wn : wave;
-            const int* src0 = g.splitk_acc + (size_t)tile * ksplit * (OWNERS * PER_WAVE) + owner * PER_WAVE;
-            uint8_t* stage_lds = stage_all + wave * (32 * (32 * 4 + 8));
-            const int pb0 = nblk * 8 + wn * TN;
+    const int keep0 = TM == 1 ? 0 : wk * (TM / 2);
+    const int* src0 = g.splitk_acc + (size_t)tile * ksplit * (OWNERS * PER_WAVE) + owner * PER_WAVE;
+    const int pb0 = nblk * 8 + wn * TN;
 #pragma unroll
-            for (int ii = 0; ii < KEEP; ++ii) {
-                v16i sum[TN];
+    for (int ii = 0; ii < KEEP; ++ii) {
+        v16i sum[TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) sum[j][r] = 0;
-                for (int p = 0; p < ksplit; ++p) {
-                    const int* src = src0 + (size_t)p * (OWNERS * PER_WAVE) + ii * TN * 1024;
+            for (int r = 0; r < 16; ++r) sum[j][r] = 0;
+        for (int p = 0; p < ksplit; ++p) {
+            const int* src = src0 + (size_t)p * (OWNERS * PER_WAVE) + ii * TN * 1024;
 #pragma unroll
-                    for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const v4i got = *reinterpret_cast<const v4i*>(src + j * 1024 + (q * 64 + lane) * 4);
-                            sum[j][q * 4] += got.x;
-                            sum[j][q * 4 + 1] += got.y;
-                            sum[j][q * 4 + 2] += got.z;
-                            sum[j][q * 4 + 3] += got.w;
-                        }
+                for (int q = 0; q < 4; ++q) {
+                    const v4i got = *reinterpret_cast<const v4i*>(src + j * 1024 + (q * 64 + lane) * 4);
+                    sum[j][q * 4] += got.x;
+                    sum[j][q * 4 + 1] += got.y;
+                    sum[j][q * 4 + 2] += got.z;
+                    sum[j][q * 4 + 3] += got.w;
                 }
-                if constexpr (W4) {
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) sum[j][r] >>= 4;
-                }
-                const int m0 = mblk * BM + (KEEP0 + ii) * 32;
-                if constexpr (EPI == RKH_EPI_SWIGLU) {
-                    epilogue_swiglu(g, sum[0], sum[1], m0, pb0, lane, g.a_scale, g.w_scale, g.M, stage_lds);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        epilogue_tile<EPI>(g, sum[j], m0, pb0 + j, lane, g.a_scale, g.w_scale, g.M, stage_lds);
-                }
-            }
         }
-    };
-    if (wk == 0) body(std::integral_constant<int, 0>{});
-    else body(std::integral_constant<int, 1>{});
+        if constexpr (W4) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum[j][r] >>= 4;
+        }
+        const int m0 = mblk * BM + (keep0 + ii) * 32;
+        if constexpr (EPI == RKH_EPI_SWIGLU) {
+            epilogue_swiglu(g, sum[0], sum[1], m0, pb0, lane, g.a_scale, g.w_scale, g.M, stage_lds);
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                epilogue_tile<EPI>(g, sum[j], m0, pb0 + j, lane, g.a_scale, g.w_scale, g.M, stage_lds);
+        }
+    }
 }
 
 // ------------------------------------------------------------- MoE route
@@ -1798,7 +1789,8 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, \
                            nblocks, ksplit, per);                                                   \
         if (ksplit > 1)                                                                             \
-            hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>), dim3(mblocks * nblocks), block, 0, st, g, \
+            hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>),                                \
+                               dim3(mblocks * nblocks * (TM == 1 ? 4 : 8)), dim3(64), 0, st, g,     \
                                mblocks, nblocks, ksplit);                                           \
     } while (0)
 #define RK_WK_EPI(W4)                                           \
