@@ -1604,17 +1604,28 @@ constexpr int ROUTE_WAVES = 4;
 __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_route_args a) {
     __shared__ int bins[ROUTE_WAVES][ROUTE_MAX_EXPERTS];
     __shared__ int start[ROUTE_MAX_EXPERTS + 1];
-    __shared__ int partial[ROUTE_WAVES * 64];
+    __shared__ int wave_total[ROUTE_WAVES];
+    __shared__ int live_total;
     const int t = threadIdx.x, lane = lane_id(), wave = wave_id();
     const int E = a.experts, Etot = E + a.shared;
     const int slots = a.top_k + a.shared;
     const int n = a.rows * a.top_k;
     for (int i = t; i < ROUTE_WAVES * Etot; i += ROUTE_WAVES * 64) bins[i / Etot][i % Etot] = 0;
-    __syncthreads();
+    if (t == 0) live_total = 0;
 
     const int chunks_total = (n + 63) / 64;
     const int chunks_per_wave = (chunks_total + ROUTE_WAVES - 1) / ROUTE_WAVES;
     const int first = wave * chunks_per_wave * 64;
+    // keys of this lane's assignments stay in registers between the counting and
+    // the placement pass (up to ROUTE_CACHE chunks per wave; re-read beyond)
+    constexpr int ROUTE_CACHE = 8;
+    int cached[ROUTE_CACHE];
+    auto key_of = [&](int c) {
+        const int i = first + c * 64 + lane;
+        return (i < n && a.routes[i] != 0.0f) ? a.ids[i] : -1;
+    };
+#pragma unroll
+    for (int c = 0; c < ROUTE_CACHE; ++c) cached[c] = c < chunks_per_wave ? key_of(c) : -1;
 
     auto same_key_mask = [&](int key) -> unsigned long long {
         unsigned long long mask = __ballot(key >= 0);
@@ -1624,19 +1635,27 @@ __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_rou
         }
         return key >= 0 ? mask : 0ull;
     };
+    __syncthreads();
 
+    int assigned = 0;
     for (int c = 0; c < chunks_per_wave; ++c) {
-        const int i = first + c * 64 + lane;
         int key = -1;
-        if (i < n && a.routes[i] != 0.0f) key = a.ids[i];
+        if (c < ROUTE_CACHE) {
+#pragma unroll
+            for (int u = 0; u < ROUTE_CACHE; ++u)
+                if (u == c) key = cached[u];
+        } else {
+            key = key_of(c);
+        }
         const unsigned long long mask = same_key_mask(key);
-        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull)
-            bins[wave][key] += __popcll(mask);
+        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull) bins[wave][key] += __popcll(mask);
+        assigned += key >= 0;
         __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
 
-    // bucket sizes -> padded exclusive scan (256 threads x 8 experts)
+    // bucket sizes -> padded exclusive scan: 8 experts per thread, a shuffle scan
+    // inside each wave, the four wave totals through LDS
     constexpr int PER = ROUTE_MAX_EXPERTS / (ROUTE_WAVES * 64);
     int sizes[PER];
     int local = 0;
@@ -1651,15 +1670,20 @@ __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_rou
         sizes[j] = (cnt + 31) & ~31;
         local += sizes[j];
     }
-    partial[t] = local;
-    __syncthreads();
-    for (int off = 1; off < ROUTE_WAVES * 64; off <<= 1) {
-        const int v = t >= off ? partial[t - off] : 0;
-        __syncthreads();
-        partial[t] += v;
-        __syncthreads();
+    int incl = local;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_up(incl, off);
+        if (lane >= off) incl += v;
     }
-    int run = partial[t] - local;
+    if (lane == 63) wave_total[wave] = incl;
+    // live assignments (for the all-routes-dropped check)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) assigned += __shfl_xor(assigned, off);
+    if (lane == 0) atomicAdd(&live_total, assigned);
+    __syncthreads();
+    int run = incl - local;
+    for (int w = 0; w < wave; ++w) run += wave_total[w];
     for (int j = 0; j < PER; ++j) {
         const int e = t * PER + j;
         if (e <= Etot) start[e] = run;
@@ -1672,7 +1696,8 @@ __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_rou
         run += sizes[j];
     }
     if (t == ROUTE_WAVES * 64 - 1) {
-        a.num_blocks[0] = min(partial[t] / 32, a.max_blocks);
+        a.num_blocks[0] = min(run / 32, a.max_blocks);
+        a.num_blocks[1] = live_total + (a.shared ? a.rows : 0);
     }
     __syncthreads();
     // per-wave running offsets
@@ -1685,18 +1710,19 @@ __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_rou
         }
     }
     __syncthreads();
-    int assigned = 0;
     for (int c = 0; c < chunks_per_wave; ++c) {
         const int i = first + c * 64 + lane;
         int key = -1;
-        if (i < n && a.routes[i] != 0.0f) key = a.ids[i];
+        if (c < ROUTE_CACHE) {
+#pragma unroll
+            for (int u = 0; u < ROUTE_CACHE; ++u)
+                if (u == c) key = cached[u];
+        } else {
+            key = key_of(c);
+        }
         const unsigned long long mask = same_key_mask(key);
         int dest = -1;
-        if (key >= 0) {
-            const int rank = __popcll(mask & ((1ull << lane) - 1ull));
-            dest = bins[wave][key] + rank;
-            ++assigned;
-        }
+        if (key >= 0) dest = bins[wave][key] + __popcll(mask & ((1ull << lane) - 1ull));
         __builtin_amdgcn_wave_barrier();
         if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull) bins[wave][key] += __popcll(mask);
         __builtin_amdgcn_wave_barrier();
@@ -1704,14 +1730,6 @@ __global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_rou
     }
     if (a.shared)
         for (int r = t; r < a.rows; r += ROUTE_WAVES * 64) a.dest_rows[(size_t)r * slots + a.top_k] = start[E] + r;
-    // total number of live assignments (for the all-routes-dropped check)
-    partial[t] = assigned;
-    __syncthreads();
-    if (t == 0) {
-        int total = a.shared ? a.rows : 0;
-        for (int i = 0; i < ROUTE_WAVES * 64; ++i) total += partial[i];
-        a.num_blocks[1] = total;
-    }
 }
 
 // out[t, n] = sum over slots, in slot order, of fma(Y[dest, n], w, out); the
