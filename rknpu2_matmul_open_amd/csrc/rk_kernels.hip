@@ -1800,10 +1800,16 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
     const dim3 grid(mblocks * nblocks * ksplit), block(512);
 #define RK_WK(W4, EPI)                                                                              \
     do {                                                                                            \
-        static const hipError_t attr = hipFuncSetAttribute(                                         \
-            reinterpret_cast<const void*>(&gemm_wk_kernel<TM, W4, EPI>),                            \
-            hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES);                              \
-        RKH_CHECK(attr);                                                                            \
+        /* the LDS opt-in is per function and per device: once for each device this process uses */ \
+        static bool opted_in[64] = {};                                                              \
+        int dev = 0;                                                                                \
+        RKH_CHECK(hipGetDevice(&dev));                                                              \
+        if (dev < 0 || dev >= 64) return RKH_ERR_RUNTIME;                                           \
+        if (!opted_in[dev]) {                                                                       \
+            RKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wk_kernel<TM, W4, EPI>), \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES)); \
+            opted_in[dev] = true;                                                                   \
+        }                                                                                           \
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, \
                            nblocks, ksplit, per);                                                   \
         if (ksplit > 1)                                                                             \

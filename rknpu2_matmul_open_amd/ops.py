@@ -83,6 +83,16 @@ class Session:
     def sync(self):
         return self.lib.rk_npu_hip_sync(self.ctx)
 
+    def spin_up(self, fn, seconds=0.05):
+        """Keep the device busy with fn() for `seconds` of wall time (untimed):
+        after an idle period the first milliseconds of work run at reduced clocks."""
+        import time
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            check(self.sync(), "sync")
+
     def time_us(self, fn, iters, warmup):
         """Average device time of fn() over `iters` calls, HIP events on the
         context's stream (the stream the kernels are launched on)."""
