@@ -774,10 +774,10 @@ __device__ __forceinline__ void store_tile(T* C, int ldc, int m0, int n0, int m_
             // rows are 8 bytes past a 16-byte boundary apart, so read as two 8-byte halves
             const uint2 lo = *reinterpret_cast<const uint2*>(stage_lds + row * ROW + part * 16);
             const uint2 hi = *reinterpret_cast<const uint2*>(stage_lds + row * ROW + part * 16 + 8);
-            if (m0 + row < m_limit)
-                *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(C) +
-                                          ((size_t)(m0 + row) * ldc + n0) * ES + part * 16) =
-                    make_uint4(lo.x, lo.y, hi.x, hi.y);
+            if (m0 + row < m_limit) // the output is not read again by this kernel: streaming store
+                __builtin_nontemporal_store(v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y},
+                                            reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(C) +
+                                                                   ((size_t)(m0 + row) * ldc + n0) * ES + part * 16));
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
