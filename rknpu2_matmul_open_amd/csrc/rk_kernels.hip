@@ -890,271 +890,6 @@ __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v1
     epilogue_swiglu_scaled(g, gate, up, m0, p, lane, as, wsg, wsu, m_limit, stage_lds);
 }
 
-// Workgroup tile BM x BN = (WM*TM*32) x (WN*TN*32), one wave per (wm, wn), each
-// wave owning TM x TN MFMA 32x32 accumulator tiles.  A K step is two 32-deep
-// k-tiles.
-//
-// Operand delivery.  Both matrices are stored as 1 KiB MFMA-ordered tiles, so a
-// fragment is one 16-byte-per-lane load.  With one wave per SIMD a wave can pull
-// only about 17 B/clk out of LDS, which makes LDS traffic, not MFMA, the limit
-// if both operands are staged there.  Therefore:
-//  - the weight fragments go global -> registers directly (each wave needs its
-//    own columns; the copy of the other wm-row of waves is served by the L1),
-//    through a ring of NS register stages that runs NS-1 K steps ahead;
-//  - only the activation tile, which every wave of the group needs, is staged
-//    through double-buffered LDS (global -> registers -> LDS, two steps ahead).
-// Software pipeline per step: the LDS writes of the next step are issued first,
-// the activation fragments of k-tile 1 are read and the int4 -> int8 unpack of
-// k-tile 1 is interleaved under the MFMAs of k-tile 0; the workgroup barrier
-// sits before k-tile 1 so that the first fragments of the next step are fetched
-// under k-tile 1's MFMAs.
-template <int WM, int WN, int TM, int TN, int KT, bool W4, int EPI, bool GROUPED>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(rkh_gemm_args g, int mblocks,
-                                                            int nblocks, int ksplit,
-                                                            int ksteps_per_part) {
-    static_assert(KT == 2, "the pipeline below is written for two k-tiles per step");
-    constexpr int NW = WM * WN;
-    constexpr int NS = 8;                             // register prefetch stages (even)
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int A_CH = BM / 32 * KT;                // 1 KiB activation chunks per K step
-    constexpr int LPW = (A_CH + NW - 1) / NW;         // activation chunk loads per wave per step
-    constexpr int WF = W4 ? TN : TN * KT;             // weight registers (v4i) per step
-    constexpr int STAGE_BYTES = NW * 32 * (32 * 4 + 8); // epilogue staging, one tile per wave
-    constexpr int LDS_BYTES = 2 * A_CH * 1024 > STAGE_BYTES ? 2 * A_CH * 1024 : STAGE_BYTES;
-    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
-    uint8_t(*lds)[A_CH * 1024] = reinterpret_cast<uint8_t(*)[A_CH * 1024]>(lds_raw);
-
-    const int lane = lane_id(), wave = wave_id();
-    const int wm = wave / WN, wn = wave % WN;
-    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
-    const int KB = Kp / 32;
-    const int ksteps_total = KB / KT;
-
-    // ---- tile assignment
-    const int total = mblocks * nblocks * ksplit;
-    const int logical = xcd_remap(blockIdx.x, total);
-    const int kpart = logical / (mblocks * nblocks);
-    const int tile = logical - kpart * (mblocks * nblocks);
-    int mblk, nblk;
-    if (GROUPED) {
-        mblk = tile % mblocks;
-        nblk = tile / mblocks;
-        if (mblk * (BM / 32) >= g.num_blocks[0]) return;
-    } else {
-        constexpr int GM = 4; // m-blocks per super-group (L2 reuse of the W columns)
-        const int per_group = GM * nblocks;
-        const int group = tile / per_group;
-        const int first_m = group * GM;
-        const int gm = min(mblocks - first_m, GM);
-        const int in_group = tile - group * per_group;
-        mblk = first_m + in_group % gm;
-        nblk = in_group / gm;
-    }
-    const int kstep0 = kpart * ksteps_per_part;
-    const int ksteps = min(ksteps_per_part, ksteps_total - kstep0);
-    if (ksteps <= 0) return;
-
-    const uint8_t* Wb = g.W;
-    const float* w_scale = g.w_scale;
-    if (GROUPED) {
-        const int e = g.blk_expert[mblk * (BM / 32)];
-        Wb += (size_t)e * g.w_expert_stride;
-        if (w_scale) w_scale += (size_t)e * g.ws_expert_stride;
-    }
-
-    // ---- sources.  Activation chunk c of a step = [row block c / KT][k-tile c % KT].
-    const uint8_t* asrc[LPW];
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-        const int c = min(wave + i * NW, A_CH - 1); // surplus slots alias the last chunk, unused
-        const int rb = mblk * (BM / 32) + c / KT;
-        asrc[i] = g.A + ((size_t)rb * KB + (size_t)kstep0 * KT + c % KT) * 1024 + lane * 16;
-    }
-    // Weight column block j of this wave: int4 = one chunk per step (both
-    // k-tiles), int8 = two consecutive chunks per step.
-    const uint8_t* wsrc[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int pb = nblk * (BN / 32) + wn * TN + j;
-        wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0) * 1024 + lane * 16
-                     : Wb + ((size_t)pb * KB + (size_t)kstep0 * KT) * 1024 + lane * 16;
-    }
-    constexpr int A_STEP = KT * 1024, W_STEP = W4 ? 1024 : KT * 1024;
-
-    v16i acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    v4i stage[NS][LPW]; // activation prefetch ring (same depth as the weight ring)
-    v4i afr[2][TM];     // activation fragments of k-tile 0 / 1
-    v4i wring[NS][WF];  // weights: raw int4 words of a step, or int8 fragments [j * KT + kt]
-    v4i wop[2][TN];     // int4 only: unpacked int8 operands of k-tile 0 / 1
-
-    auto load_a = [&](v4i* regs) {
-#pragma unroll
-        for (int i = 0; i < LPW; ++i) {
-            if (A_CH % NW == 0 || wave + i * NW < A_CH) regs[i] = *reinterpret_cast<const v4i*>(asrc[i]);
-            asrc[i] += A_STEP;
-        }
-    };
-    auto store_a = [&](const v4i* regs, int buf) {
-#pragma unroll
-        for (int i = 0; i < LPW; ++i)
-            if (A_CH % NW == 0 || wave + i * NW < A_CH)
-                *reinterpret_cast<v4i*>(&lds[buf][(wave + i * NW) * 1024 + lane * 16]) = regs[i];
-    };
-    auto load_w = [&](v4i* regs) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if constexpr (W4) {
-                regs[j] = *reinterpret_cast<const v4i*>(wsrc[j]);
-            } else {
-                regs[j * KT] = *reinterpret_cast<const v4i*>(wsrc[j]);
-                regs[j * KT + 1] = *reinterpret_cast<const v4i*>(wsrc[j] + 1024);
-            }
-            wsrc[j] += W_STEP;
-        }
-    };
-    auto read_a = [&](v4i* dst, int buf, int kt) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-            dst[i] = *reinterpret_cast<const v4i*>(&lds[buf][((wm * TM + i) * KT + kt) * 1024 + lane * 16]);
-    };
-    auto unpack = [&](v4i* dst, const v4i* raw, int kt) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int w0 = kt ? raw[j].z : raw[j].x;
-            const int w1 = kt ? raw[j].w : raw[j].y;
-            dst[j].x = (w0 << 4) & 0xF0F0F0F0;
-            dst[j].y = w0 & 0xF0F0F0F0;
-            dst[j].z = (w1 << 4) & 0xF0F0F0F0;
-            dst[j].w = w1 & 0xF0F0F0F0;
-        }
-    };
-    // MFMAs of one k-tile; weights are the first operand (see tile_col()).
-    auto mfma_all = [&](const v4i* a, const v4i* w, int wstride, int woff) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[j * wstride + woff], a[i], acc[i][j], 0, 0, 0);
-    };
-
-    // One K step.  SLOT = s % NS selects the register stage, SLOT % 2 the LDS
-    // buffer.  n1 / n3: step s+1 / s+(NS-1) exists (compile-time true in the
-    // steady state, run-time flags in the tail).
-    auto k_step = [&](auto slot_tag, auto n1, auto n3) {
-        constexpr int SLOT = decltype(slot_tag)::value;
-        constexpr int P = SLOT & 1;
-        // ---- k-tile 0
-        // Loads complete in issue order: the activations go first so that waiting
-        // for them (for the LDS write two steps later) leaves the weight loads of
-        // the same and later steps in flight.
-        if (n3) load_a(stage[(SLOT + NS - 1) % NS]);
-        if (n3) load_w(wring[(SLOT + NS - 1) % NS]);
-        read_a(afr[1], P, 1);
-        if (n1) store_a(stage[(SLOT + 1) % NS], P ^ 1);
-        if constexpr (W4) {
-            unpack(wop[1], wring[SLOT], 1);
-            mfma_all(afr[0], wop[0], 1, 0);
-#pragma unroll
-            for (int q = 0; q < TM * TN; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // 1 MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0);
-                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);      // 1 LDS op
-                if (q < TN + LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // 1 global load
-            }
-        } else {
-            mfma_all(afr[0], wring[SLOT], KT, 0);
-#pragma unroll
-            for (int q = 0; q < TM * TN; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (q < TM + LPW) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
-                if (q < TN * KT + LPW) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        lds_barrier();
-        // ---- k-tile 1: fetch the first fragments of the next step under its MFMAs
-        if (n1) read_a(afr[0], P ^ 1, 0);
-        if constexpr (W4) {
-            mfma_all(afr[1], wop[1], 1, 0);
-            if (n1) unpack(wop[0], wring[(SLOT + 1) % NS], 0);
-#pragma unroll
-            for (int q = 0; q < TM * TN; ++q) {
-                if (q < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // LDS reads first
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, (TN * 6 + TM * TN - 1) / (TM * TN), 0);
-            }
-        } else {
-            mfma_all(afr[1], wring[SLOT], KT, 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    using T_ = std::true_type;
-
-    // prologue: weights of steps 0..NS-2 and activations of steps 0, 1 in flight;
-    // step 0 in LDS, its first fragments in registers
-#pragma unroll
-    for (int i = 0; i < NS - 1; ++i) {
-        if (i < ksteps) {
-            load_a(stage[i]);
-            load_w(wring[i]);
-        }
-    }
-    store_a(stage[0], 0);
-    lds_barrier();
-    read_a(afr[0], 0, 0);
-    if constexpr (W4) unpack(wop[0], wring[0], 0);
-
-    int s = 0;
-    // steady state: NS steps per trip, every look-ahead exists
-    for (; s + 2 * NS - 2 < ksteps; s += NS)
-        static_for<NS>([&](auto slot) { k_step(slot, T_{}, T_{}); });
-    // tail: run-time look-ahead flags
-    for (; s < ksteps; s += NS)
-        static_for<NS>([&](auto slot) {
-            constexpr int SL = decltype(slot)::value;
-            if (s + SL < ksteps) k_step(slot, s + SL + 1 < ksteps, s + SL + NS - 1 < ksteps);
-        });
-
-    if (W4) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] >>= 4;
-    }
-
-    // ---- epilogue
-    const int m_limit = GROUPED ? g.num_blocks[0] * 32 : g.M;
-    // all waves are past their last LDS fragment read (the barrier of the last
-    // step precedes only register work), so the buffers can be reused as
-    // wave-private staging for the stores
-    lds_barrier();
-    uint8_t* stage_lds = lds_raw + wave * (32 * (32 * 4 + 8));
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m0 = mblk * BM + (wm * TM + i) * 32;
-        if constexpr (EPI == RKH_EPI_SWIGLU) {
-#pragma unroll
-            for (int j = 0; j < TN; j += 2)
-                epilogue_swiglu(g, acc[i][j], acc[i][j + 1], m0, nblk * (BN / 32) + wn * TN + j, lane,
-                                g.a_scale, w_scale, m_limit, stage_lds);
-        } else {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                epilogue_tile<EPI>(g, acc[i][j], m0, nblk * (BN / 32) + wn * TN + j, lane,
-                                   g.a_scale, w_scale, m_limit, stage_lds);
-        }
-    }
-}
-
 // ---- tiles of (32 * TM) rows x 256 columns, waves split K --------------------
 // Eight waves = 4 column groups (wn) x 2 k-halves (wk): wave (wn, wk)
 // accumulates the whole (32*TM) x 64 strip of column group wn, but only over
@@ -1433,6 +1168,14 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     // ---- epilogue.  Drain the look-ahead copies (they write LDS) and the scale
     // loads; then every wave is past its last fragment read and LDS is reused.
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(my_as), "+v"(my_ws)::"memory");
+    // The weight loads issued for sub-steps beyond K were in flight until this
+    // wait, while the compiler regards their destination registers as dead: the
+    // uses below keep it from giving one of them to an epilogue value ahead of
+    // the wait (the load would then land on top of that value).
+#pragma unroll
+    for (int t = 0; t < NSW; ++t)
+#pragma unroll
+        for (int e = 0; e < NWREG; ++e) asm volatile("" : "+v"(wring[t][e]));
     if constexpr (EPI != RKH_EPI_I32) {
         float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
         const int t = threadIdx.x;
@@ -1591,6 +1334,108 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
             for (int j = 0; j < TN; ++j)
                 epilogue_tile<EPI>(g, sum[j], m0, pb0 + j, lane, g.a_scale, g.w_scale, g.M, stage_lds);
         }
+    }
+}
+
+// ---- grouped (MoE) GEMM: 32 sorted rows x 256 columns, weights streamed -----
+// With a few dozen rows per expert this GEMM is a weight stream: there are two
+// MFMAs per KiB of expert weights.  So there is no LDS staging and no workgroup
+// barrier: each of the four waves owns two 32-column blocks of the tile over
+// the whole K and runs its own ring of RING k-tiles of loads -- the activation
+// tile (1 KiB, shared with the other waves through the L1) and its two weight
+// tiles, 16 bytes per lane each -- waiting with an explicit counter (loads
+// complete in issue order; every step issues exactly three of them, also
+// beyond the end of K, where the sources stop advancing).  Several workgroups
+// share a compute unit.  An expert with more than 32 rows has one workgroup per
+// row block and column tile; they run side by side and the second one finds
+// the weights in L2 (taking all row blocks of an expert into one workgroup was
+// measured slower: fewer workgroups than compute units remain).
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
+    constexpr int TN = 2, WAVES = 4;
+    constexpr int RING = 8;
+    constexpr int LPS = 1 + TN;
+    static_assert((RING - 1) * LPS <= 63, "vmcnt field");
+    __shared__ __attribute__((aligned(16))) uint8_t stage_raw[WAVES * 32 * (32 * 4 + 8)];
+
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+    const int KB = (int)rkh_align_up(g.K, RKH_K_ALIGN) / 32; // k-tiles: a multiple of 8 = RING
+
+    const int logical = xcd_remap(blockIdx.x, mblocks * nblocks);
+    const int mblk = logical % mblocks, nblk = logical / mblocks;
+    if (mblk >= g.num_blocks[0]) return;
+    const int e = g.blk_expert[mblk];
+    const uint8_t* Wb = g.W + (size_t)e * g.w_expert_stride;
+    const float* w_scale = g.w_scale ? g.w_scale + (size_t)e * g.ws_expert_stride : nullptr;
+
+    const int pb0 = (nblk * WAVES + wave) * TN;
+    const uint8_t* asrc = g.A + (size_t)mblk * KB * 1024;
+    const uint8_t* wsrc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) wsrc[j] = Wb + (size_t)(pb0 + j) * KB * 1024;
+    const unsigned lane_off = lane * 16;
+    int left = KB - 1; // how often the sources may still advance
+
+    v16i acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+    v4i ring[RING][LPS]; // [0] = activations, [1 + j] = weights of column block j
+
+    auto issue = [&](v4i* regs) {
+        static_for<LPS>([&](auto l_tag) {
+            constexpr int L = decltype(l_tag)::value;
+            const unsigned off = lane_off; // (locals: asm operands cannot name captures of an enclosing lambda)
+            const uint8_t* base = L == 0 ? asrc : wsrc[L == 0 ? 0 : L - 1];
+            v4i r;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
+            regs[L] = r;
+        });
+        const int step = left > 0 ? 1024 : 0;
+        asrc += step;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) wsrc[j] += step;
+        --left;
+    };
+    auto wait = [&](v4i* regs) { // all but the latest (RING-1) steps' loads have landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RING - 1) * LPS) : "memory");
+#pragma unroll
+        for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(regs[l]));
+    };
+
+#pragma unroll
+    for (int t = 0; t < RING - 1; ++t) issue(ring[t]);
+    for (int s = 0; s < KB; s += RING)
+        static_for<RING>([&](auto slot_tag) {
+            constexpr int SLOT = decltype(slot_tag)::value;
+            issue(ring[(SLOT + RING - 1) % RING]);
+            wait(ring[SLOT]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][1 + j], ring[SLOT][0], acc[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    // The look-ahead loads beyond K are still in flight here and the compiler
+    // regards their destination registers as dead: without the uses below it may
+    // give one of them to an epilogue value ahead of the wait, and the load then
+    // lands on top of that value.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < RING; ++t)
+#pragma unroll
+        for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(ring[t][l]));
+
+    const int m_limit = g.num_blocks[0] * 32;
+    uint8_t* stage_lds = stage_raw + wave * (32 * (32 * 4 + 8));
+    const int m0 = mblk * 32;
+    if constexpr (EPI == RKH_EPI_SWIGLU) {
+        epilogue_swiglu(g, acc[0], acc[1], m0, pb0, lane, g.a_scale, w_scale, m_limit, stage_lds);
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            epilogue_tile<EPI>(g, acc[j], m0, pb0 + j, lane, g.a_scale, w_scale, m_limit, stage_lds);
     }
 }
 
@@ -1754,21 +1599,14 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 }
 
 // ------------------------------------------------------------- launchers
-// Grouped (MoE) launches: 32-row blocks of the sorted rows x 256 columns, four
-// waves, one workgroup per (block, column block); several workgroups share a
-// compute unit, which suits this weight-streaming shape (every expert's
-// weights are read once).
+// Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
+// 256-column tile); blocks beyond the live count exit at once.
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
-    constexpr int WM = 1, WN = 4, TM = 1, TN = 2, KT = 2;
-    constexpr int BN = WN * TN * 32;
     if (g.w_int4) return RKH_ERR_RUNTIME;
     const int mblocks = g.max_blocks;
-    const int nblocks = (g.N + BN - 1) / BN;
-    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 32 / KT);
-    const dim3 grid(mblocks * nblocks), block(WM * WN * 64);
-#define RK_LAUNCH(EPI)                                                                          \
-    hipLaunchKernelGGL((gemm_kernel<WM, WN, TM, TN, KT, false, EPI, true>), grid, block, 0, st, g, \
-                       mblocks, nblocks, 1, ksteps_total)
+    const int nblocks = (g.N + 255) / 256;
+    const dim3 grid(mblocks * nblocks), block(256);
+#define RK_LAUNCH(EPI) hipLaunchKernelGGL((gemm_stream_kernel<EPI>), grid, block, 0, st, g, mblocks, nblocks)
     switch (g.epilogue) {
     case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
     case RKH_EPI_F16: RK_LAUNCH(RKH_EPI_F16); break;
