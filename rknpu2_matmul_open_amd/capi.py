@@ -123,6 +123,39 @@ class W4A8FfnTimings(C.Structure):
     _fields_ = [("gate_up", W4A8Timings), ("down", W4A8Timings), ("total_us", C.c_double)]
 
 
+# rk_npu_w4a8_tune.h
+W4A8_F32, W4A8_F16 = 0, 1
+
+
+class W4A8AutotuneConfig(C.Structure):
+    _fields_ = [("M", C.c_int), ("N", C.c_int), ("K", C.c_int), ("activation_type", C.c_int),
+                ("allowed_npu_core_mask", C.c_uint32), ("allowed_cpu_core_mask", C.c_uint64),
+                ("warmup", C.c_int), ("loops", C.c_int), ("repeats", C.c_int), ("timeout_ms", C.c_uint32),
+                ("verbose", C.c_int), ("required_k_tile", C.c_int), ("k_tile_multiplier", C.c_double)]
+
+
+class W4A8Strategy(C.Structure):
+    _fields_ = [("config", W4A8Config), ("activation_type", C.c_int), ("cpu_core_mask", C.c_uint64),
+                ("weights", W4A8WeightInfo), ("weight_fingerprint", C.c_uint64),
+                ("tuning_revision", C.c_uint32), ("input_us", C.c_double), ("npu_us", C.c_double),
+                ("sync_us", C.c_double), ("output_us", C.c_double), ("total_us", C.c_double),
+                ("jitter_pct", C.c_double), ("robust_us", C.c_double)]
+
+
+class W4A8StrategyEx(C.Structure):
+    _fields_ = [("base", W4A8Strategy), ("execution", W4A8Options)]
+
+
+class W4A8FamilyConfig(C.Structure):
+    _fields_ = [("base", W4A8AutotuneConfig), ("m_count", C.c_int), ("m_values", C.POINTER(C.c_int)),
+                ("frequencies", C.POINTER(C.c_double))]
+
+
+class W4A8FamilySummary(C.Structure):
+    _fields_ = [("weights", W4A8WeightInfo), ("weight_fingerprint", C.c_uint64),
+                ("weighted_total_us", C.c_double), ("weighted_robust_us", C.c_double)]
+
+
 class MoeWeightConfig(C.Structure):
     _fields_ = [("hidden", C.c_int), ("intermediate", C.c_int), ("routed_experts", C.c_int),
                 ("shared_expert", C.c_int)]
@@ -217,6 +250,50 @@ _PROTOTYPES = {
     "rk_npu_w4a8_run_f16": (C.c_int, [P, P, P, P, C.POINTER(W4A8Timings)]),
     "rk_npu_w4a8_run_swiglu_f32": (C.c_int, [P, P, P, P, C.POINTER(W4A8Timings)]),
     "rk_npu_w4a8_run_ffn_f32": (C.c_int, [P, P, P, P, P, P, P, C.POINTER(W4A8FfnTimings)]),
+    # rk_npu_w4a8_tune.h
+    "rk_npu_w4a8_autotune_config_init": (None, [C.POINTER(W4A8AutotuneConfig), C.c_int, C.c_int, C.c_int]),
+    "rk_npu_w4a8_family_config_init": (None, [C.POINTER(W4A8FamilyConfig), C.c_int, C.c_int, C.c_int,
+                                              C.POINTER(C.c_int)]),
+    "rk_npu_w4a8_tuning_profile_from_weights": (P, [P]),
+    "rk_npu_w4a8_tuning_profile_free": (None, [P]),
+    "rk_npu_w4a8_tuning_profile_fingerprint": (C.c_uint64, [P]),
+    "rk_npu_w4a8_autotune_cache_load_profile_ex": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, C.c_char_p,
+                                                             C.POINTER(W4A8StrategyEx), C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_autotune": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.POINTER(W4A8Strategy),
+                                       C.POINTER(W4A8Strategy)]),
+    "rk_npu_w4a8_autotune_cached": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p, C.c_int,
+                                              C.POINTER(W4A8Strategy), C.POINTER(W4A8Strategy),
+                                              C.POINTER(C.c_int)]),
+    "rk_npu_w4a8_autotune_cache_load": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p,
+                                                  C.POINTER(W4A8Strategy), C.POINTER(W4A8Strategy)]),
+    "rk_npu_w4a8_autotune_cache_save": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p,
+                                                  C.POINTER(W4A8Strategy), C.POINTER(W4A8Strategy)]),
+    "rk_npu_w4a8_weights_create_tuned": (P, [P, C.POINTER(W4A8Strategy), P, P]),
+    "rk_npu_w4a8_autotune_family": (C.c_int, [P, C.POINTER(W4A8FamilyConfig), P, P,
+                                              C.POINTER(W4A8FamilySummary), C.POINTER(W4A8Strategy),
+                                              C.POINTER(W4A8FamilySummary), C.POINTER(W4A8Strategy)]),
+    "rk_npu_w4a8_autotune_family_cached": (C.c_int, [P, C.POINTER(W4A8FamilyConfig), P, P, C.c_char_p, C.c_int,
+                                                     C.POINTER(W4A8FamilySummary), C.POINTER(W4A8Strategy),
+                                                     C.POINTER(W4A8FamilySummary), C.POINTER(W4A8Strategy),
+                                                     C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "rk_npu_w4a8_autotune_ex": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.POINTER(W4A8StrategyEx),
+                                          C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_autotune_cached_ex": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p, C.c_int,
+                                                 C.POINTER(W4A8StrategyEx), C.POINTER(W4A8StrategyEx),
+                                                 C.POINTER(C.c_int)]),
+    "rk_npu_w4a8_autotune_cache_load_ex": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p,
+                                                     C.POINTER(W4A8StrategyEx), C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_autotune_cache_save_ex": (C.c_int, [P, C.POINTER(W4A8AutotuneConfig), P, P, C.c_char_p,
+                                                     C.POINTER(W4A8StrategyEx), C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_weights_create_tuned_ex": (P, [P, C.POINTER(W4A8StrategyEx), P, P]),
+    "rk_npu_w4a8_workspace_create_tuned_ex": (P, [P, C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_autotune_family_ex": (C.c_int, [P, C.POINTER(W4A8FamilyConfig), P, P,
+                                                 C.POINTER(W4A8FamilySummary), C.POINTER(W4A8StrategyEx),
+                                                 C.POINTER(W4A8FamilySummary), C.POINTER(W4A8StrategyEx)]),
+    "rk_npu_w4a8_autotune_family_cached_ex": (C.c_int, [P, C.POINTER(W4A8FamilyConfig), P, P, C.c_char_p, C.c_int,
+                                                        C.POINTER(W4A8FamilySummary), C.POINTER(W4A8StrategyEx),
+                                                        C.POINTER(W4A8FamilySummary), C.POINTER(W4A8StrategyEx),
+                                                        C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     # rk_npu_moe_w8.h
     "rk_npu_moe_w8_config_init": (None, [C.POINTER(MoeConfig)] + [C.c_int] * 6),
     "rk_npu_moe_w8_weights_create": (P, [P, C.POINTER(MoeWeightConfig), C.POINTER(MoeExpert)]),

@@ -12,10 +12,12 @@
 #include <climits>
 #include <cstdlib>
 #include <new>
+#include <thread>
 
 #include "rk_host.h"
 #include "rk_npu_hip.h"
 #include "rk_npu_w4a8.h"
+#include "rk_w4a8_internal.h"
 
 using namespace rkhost;
 
@@ -120,27 +122,94 @@ struct BoundScan {
 
 // K is bounded by INT32_MAX/1024, so 8*K*... prefix sums fit int32: max per
 // element contribution is 64, 64 * 2^21 = 2^27.
-int largest_certified_tile(const int8_t* B, int K, int N, int requested /*0 = search*/) {
-    BoundScan s{K, N, (K + 31) / 32, {}, {}};
-    // Column slabs keep the prefix tables small for wide matrices.
+//
+// Largest certified tile (or -1: an out-of-range code, or nothing certified).
+// `requested` = 0 searches all tile sizes up to 2048, else only that one is
+// tested.  `mask` (optional) receives one bit per certified size, bit t-1 for
+// 32*t.  Column slabs keep the prefix tables small and are independent, so
+// they are spread over a few host threads.
+int largest_certified_tile(const int8_t* B, int K, int N, int requested /*0 = search*/, uint64_t* mask = nullptr) {
+    const int blocks = (K + 31) / 32;
     constexpr int kSlab = 256;
-    const int limit = requested ? requested / 32 : std::min(kKTileMax / 32, s.blocks);
-    std::vector<char> safe((size_t)limit + 1, 0);
-    for (int t = 1; t <= limit; ++t) safe[t] = !requested || t == limit;
-    std::vector<int8_t> slab;
-    for (int n0 = 0; n0 < N; n0 += kSlab) {
-        const int width = std::min(kSlab, N - n0);
-        slab.resize((size_t)K * width);
-        for (int k = 0; k < K; ++k)
-            std::memcpy(slab.data() + (size_t)k * width, B + (size_t)k * N + n0, (size_t)width);
-        BoundScan part{K, width, s.blocks, {}, {}};
-        if (!part.scan(slab.data())) return -1;
-        for (int t = 1; t <= limit; ++t)
-            if (safe[t] && !part.certifies(t)) safe[t] = 0;
+    const int limit = requested ? requested / 32 : std::min(kKTileMax / 32, blocks);
+    const int slabs = (N + kSlab - 1) / kSlab;
+    const int workers = std::max(1, std::min({slabs, 8, (int)std::thread::hardware_concurrency()}));
+    std::vector<std::vector<char>> safe_of((size_t)workers, std::vector<char>((size_t)limit + 1, 1));
+    std::vector<char> failed((size_t)workers, 0);
+    auto work = [&](int id) {
+        std::vector<int8_t> slab;
+        std::vector<char>& safe = safe_of[(size_t)id];
+        for (int t = 1; t <= limit; ++t) safe[(size_t)t] = !requested || t == limit;
+        for (int si = id; si < slabs; si += workers) {
+            const int n0 = si * kSlab, width = std::min(kSlab, N - n0);
+            slab.resize((size_t)K * width);
+            for (int k = 0; k < K; ++k)
+                std::memcpy(slab.data() + (size_t)k * width, B + (size_t)k * N + n0, (size_t)width);
+            BoundScan part{K, width, blocks, {}, {}};
+            if (!part.scan(slab.data())) {
+                failed[(size_t)id] = 1;
+                return;
+            }
+            for (int t = 1; t <= limit; ++t)
+                if (safe[(size_t)t] && !part.certifies(t)) safe[(size_t)t] = 0;
+        }
+    };
+    if (workers == 1) {
+        work(0);
+    } else {
+        std::vector<std::thread> pool;
+        for (int id = 0; id < workers; ++id) pool.emplace_back(work, id);
+        for (auto& t : pool) t.join();
     }
-    for (int t = limit; t >= 1; --t)
-        if (safe[t]) return t * 32;
-    return -1;
+    for (char f : failed)
+        if (f) return -1;
+    uint64_t bits = 0;
+    int best = -1;
+    for (int t = 1; t <= limit; ++t) {
+        bool ok = true;
+        for (int id = 0; id < workers; ++id) ok = ok && safe_of[(size_t)id][(size_t)t];
+        if (ok) {
+            bits |= uint64_t(1) << (t - 1);
+            best = t * 32;
+        }
+    }
+    if (mask) *mask = bits;
+    return best;
+}
+
+// Identity of a weight matrix (codes and scales), not a security hash: FNV-1a
+// per 1 MiB piece, the piece digests folded in order, so that the pieces can be
+// hashed side by side.
+uint64_t fingerprint_of(int K, int N, const int8_t* B, const float* w_scale) {
+    auto fnv = [](uint64_t h, const void* data, size_t bytes) {
+        const uint8_t* p = static_cast<const uint8_t*>(data);
+        for (size_t i = 0; i < bytes; ++i) {
+            h ^= p[i];
+            h *= 0x100000001b3ull;
+        }
+        return h;
+    };
+    constexpr uint64_t kBasis = 0xcbf29ce484222325ull;
+    constexpr size_t kPiece = 1u << 20;
+    const size_t total = (size_t)K * N, pieces = (total + kPiece - 1) / kPiece;
+    std::vector<uint64_t> digest(pieces);
+    const int workers = std::max(1, std::min({(int)pieces, 8, (int)std::thread::hardware_concurrency()}));
+    auto work = [&](int id) {
+        for (size_t i = (size_t)id; i < pieces; i += (size_t)workers)
+            digest[i] = fnv(kBasis, B + i * kPiece, std::min(kPiece, total - i * kPiece));
+    };
+    if (workers == 1) {
+        work(0);
+    } else {
+        std::vector<std::thread> pool;
+        for (int id = 0; id < workers; ++id) pool.emplace_back(work, id);
+        for (auto& t : pool) t.join();
+    }
+    uint64_t h = kBasis;
+    const int64_t shape[2] = {K, N};
+    h = fnv(h, shape, sizeof(shape));
+    h = fnv(h, digest.data(), digest.size() * sizeof(uint64_t));
+    return fnv(h, w_scale, (size_t)N * sizeof(float));
 }
 
 } // namespace
@@ -148,6 +217,7 @@ int largest_certified_tile(const int8_t* B, int K, int N, int requested /*0 = se
 struct rk_npu_w4a8_weights {
     Owner owner;
     rk_npu_w4a8_weight_info info{};
+    rkhost::W4Profile profile;
     int interleave_F = 0;  // N/2 when N % 64 == 0 (gate/up column blocks interleaved)
     DeviceBuffer tiled;    // tiled int4
     DeviceBuffer w_scale;  // [N]
@@ -347,6 +417,77 @@ int validate_ffn(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights* guw,
 
 } // namespace
 
+namespace rkhost {
+
+double w4a8_env_multiplier() {
+    const char* text = std::getenv("RK_NPU_W4A8_K_TILE_MULTIPLIER");
+    if (!text) return 1.0;
+    errno = 0;
+    char* end = nullptr;
+    const double factor = std::strtod(text, &end);
+    if (errno || end == text || *end || !std::isfinite(factor) || factor < 1) return -1.0;
+    return factor;
+}
+
+// reference src/rk_npu_w4a8_tune_policy.cpp:46-70 (the weight-dependent part)
+int w4a8_make_profile(int K, int N, double multiplier, const int8_t* B, const float* w_scale, W4Profile* out) {
+    if (!out || !B || !w_scale || !valid_shape(K, N) || N > INT_MAX - 63 || !std::isfinite(multiplier) ||
+        multiplier < 1)
+        return RK_NPU_ERR_PARAM;
+    if (!finite_positive(w_scale, (size_t)N)) return RK_NPU_ERR_PARAM;
+    W4Profile p;
+    p.K = K;
+    p.N = N;
+    p.multiplier = multiplier;
+    p.safe = largest_certified_tile(B, K, N, 0, &p.safe_tiles);
+    if (p.safe < 32) return RK_NPU_ERR_PARAM;
+    const int cap = std::min(kKTileMax, (int)align_up64(K, 32));
+    p.limit = (int)(std::min((double)cap, p.safe * multiplier) / 32) * 32;
+    p.fingerprint = fingerprint_of(K, N, B, w_scale);
+    *out = p;
+    return RK_NPU_OK;
+}
+
+// reference src/rk_npu_w4a8.cpp:208-247
+rk_npu_w4a8_weights* w4a8_create_weights(rk_npu_iommu_domain* domain, const rk_npu_w4a8_weight_info& info,
+                                         const int8_t* B, const float* w_scale, const W4Profile* profile) {
+    const rk_npu_i4_weight_config& cfg = info.config;
+    if (!domain || !domain->ctx || !B || !w_scale || !valid_shape(cfg.K, cfg.N) ||
+        !weight_key_valid(cfg.K, cfg.N, cfg.k_tile))
+        return nullptr;
+    if (!finite_positive(w_scale, (size_t)cfg.N)) return nullptr;
+    std::unique_ptr<rk_npu_w4a8_weights> w(new (std::nothrow) rk_npu_w4a8_weights());
+    if (!w) return nullptr;
+    if (profile) {
+        w->profile = *profile;
+    } else if (w4a8_make_profile(cfg.K, cfg.N, info.multiplier, B, w_scale, &w->profile)) {
+        // the full proof is captured independently of the requested partition
+        // (an explicit k_tile may be wider than K)
+        return nullptr;
+    }
+    w->owner.bind(domain);
+    w->info = info;
+    w->interleave_F = cfg.N % 64 == 0 ? cfg.N / 2 : 0;
+    rk_npu_ctx* ctx = domain->ctx;
+    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
+    DeviceBuffer raw, bad;
+    if (upload(w->owner, raw, B, (size_t)cfg.K * cfg.N)) return nullptr;
+    if (bad.alloc(w->owner, sizeof(int), true)) return nullptr;
+    if (w->tiled.alloc(w->owner, rkh_tiled_i4_bytes(cfg.N, cfg.K, RKH_COL_ALIGN), false)) return nullptr;
+    if (rkh_pack_w4(ctx->stream, raw.as<int8_t>(), cfg.K, cfg.N, w->interleave_F, w->tiled.as<>(),
+                    bad.as<int>()))
+        return nullptr;
+    if (upload(w->owner, w->w_scale, w_scale, (size_t)cfg.N * sizeof(float))) return nullptr;
+    int bad_host = 0;
+    if (rkh_d2h(ctx->stream, &bad_host, bad.as<>(), sizeof(int)) || rkh_sync(ctx->stream)) return nullptr;
+    if (bad_host) return nullptr; // a code outside [-8, 7]
+    return w.release();
+}
+
+const W4Profile& w4a8_profile_of(const rk_npu_w4a8_weights* weights) { return weights->profile; }
+
+} // namespace rkhost
+
 extern "C" {
 
 void rk_npu_w4a8_config_init(rk_npu_w4a8_config* cfg, int M, int N, int K) {
@@ -429,47 +570,17 @@ rk_npu_w4a8_weights* rk_npu_w4a8_weights_create(rk_npu_iommu_domain* domain,
     info.safe_k_tile = cfg->k_tile;
     info.multiplier = 1.0;
     if (cfg->k_tile == 0) {
-        const int safe = largest_certified_tile(B, cfg->K, cfg->N, 0);
-        if (safe < 32) return nullptr;
-        double factor = 1.0;
-        if (const char* text = std::getenv("RK_NPU_W4A8_K_TILE_MULTIPLIER")) {
-            errno = 0;
-            char* end = nullptr;
-            factor = std::strtod(text, &end);
-            if (errno || end == text || *end || !std::isfinite(factor) || factor < 1) return nullptr;
-        }
-        const int cap = std::min(kKTileMax, (int)align_up64(cfg->K, 32));
-        info.config.k_tile = (int)(std::min((double)cap, safe * factor) / 32) * 32;
-        info.safe_k_tile = safe;
-        info.multiplier = factor;
-        info.bound_relaxed = info.config.k_tile > safe;
-    } else {
-        if (!weight_key_valid(cfg->K, cfg->N, cfg->k_tile)) return nullptr;
-        if (cfg->k_tile > kKTileUniversal &&
-            largest_certified_tile(B, cfg->K, cfg->N, cfg->k_tile) != cfg->k_tile)
-            return nullptr;
+        const double factor = rkhost::w4a8_env_multiplier();
+        if (factor < 1) return nullptr;
+        rkhost::W4Profile profile;
+        if (rkhost::w4a8_make_profile(cfg->K, cfg->N, factor, B, w_scale, &profile)) return nullptr;
+        return rkhost::w4a8_create_weights(domain, profile.info(profile.limit), B, w_scale, &profile);
     }
-    if (!finite_positive(w_scale, (size_t)cfg->N)) return nullptr;
-
-    std::unique_ptr<rk_npu_w4a8_weights> w(new (std::nothrow) rk_npu_w4a8_weights());
-    if (!w) return nullptr;
-    w->owner.bind(domain);
-    w->info = info;
-    w->interleave_F = cfg->N % 64 == 0 ? cfg->N / 2 : 0;
-    rk_npu_ctx* ctx = domain->ctx;
-    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
-    DeviceBuffer raw, bad;
-    if (upload(w->owner, raw, B, (size_t)cfg->K * cfg->N)) return nullptr;
-    if (bad.alloc(w->owner, sizeof(int), true)) return nullptr;
-    if (w->tiled.alloc(w->owner, rkh_tiled_i4_bytes(cfg->N, cfg->K, RKH_COL_ALIGN), false)) return nullptr;
-    if (rkh_pack_w4(ctx->stream, raw.as<int8_t>(), cfg->K, cfg->N, w->interleave_F, w->tiled.as<>(),
-                    bad.as<int>()))
+    if (!weight_key_valid(cfg->K, cfg->N, cfg->k_tile)) return nullptr;
+    if (cfg->k_tile > kKTileUniversal &&
+        largest_certified_tile(B, cfg->K, cfg->N, cfg->k_tile) != cfg->k_tile)
         return nullptr;
-    if (upload(w->owner, w->w_scale, w_scale, (size_t)cfg->N * sizeof(float))) return nullptr;
-    int bad_host = 0;
-    if (rkh_d2h(ctx->stream, &bad_host, bad.as<>(), sizeof(int)) || rkh_sync(ctx->stream)) return nullptr;
-    if (bad_host) return nullptr; // a code outside [-8, 7]
-    return w.release();
+    return rkhost::w4a8_create_weights(domain, info, B, w_scale, nullptr);
 }
 
 void rk_npu_w4a8_weights_free(rk_npu_w4a8_weights* weights) { delete weights; }

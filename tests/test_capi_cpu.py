@@ -17,7 +17,7 @@ from rknpu2_matmul_open_amd import capi
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 INC = os.path.join(ROOT, "include")
 HEADERS = ["rk_npu_common.h", "rk_npu_quant_matmul.h", "rk_npu_matmul_i4.h", "rk_npu_w4a8.h",
-           "rk_npu_moe_w8.h", "rk_npu_hip.h"]
+           "rk_npu_w4a8_tune.h", "rk_npu_moe_w8.h", "rk_npu_hip.h"]
 
 
 @pytest.fixture(scope="module")
@@ -66,10 +66,14 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
              ("rk_npu_w4a8_options", capi.W4A8Options), ("rk_npu_w4a8_memory_info_ex", capi.W4A8MemoryInfoEx),
              ("rk_npu_w4a8_timings", capi.W4A8Timings), ("rk_npu_w4a8_weight_info", capi.W4A8WeightInfo),
              ("rk_npu_w4a8_ffn_timings", capi.W4A8FfnTimings),
+             ("rk_npu_w4a8_autotune_config", capi.W4A8AutotuneConfig), ("rk_npu_w4a8_strategy", capi.W4A8Strategy),
+             ("rk_npu_w4a8_strategy_ex", capi.W4A8StrategyEx), ("rk_npu_w4a8_family_config", capi.W4A8FamilyConfig),
+             ("rk_npu_w4a8_family_summary", capi.W4A8FamilySummary),
              ("rk_npu_moe_w8_weight_config", capi.MoeWeightConfig), ("rk_npu_moe_w8_config", capi.MoeConfig),
              ("rk_npu_moe_w8_expert", capi.MoeExpert), ("rk_npu_moe_w8_timings", capi.MoeTimings),
              ("rk_npu_domain_memory_stats", capi.DomainMemoryStats)]
-    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rk_npu_hip.h"', "int main(void) {"]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rk_npu_hip.h"', '#include "rk_npu_w4a8_tune.h"',
+             "int main(void) {"]
     for cname, ct in pairs:
         lines.append('printf("%s %%zu", sizeof(%s));' % (cname, cname))
         for fname, _ in ct._fields_:
@@ -289,3 +293,55 @@ def test_package_fails_loudly_without_the_library(monkeypatch, tmp_path):
     monkeypatch.setattr(capi, "_LIB", None)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         capi.load_library()
+
+
+def test_w4a8_tune_entry_points_without_a_context(lib):
+    """reference src/rk_npu_w4a8_tune_policy.cpp:178-185 (defaults) and the NULL / argument checks of
+    src/rk_npu_w4a8_tune.cpp:124-127, src/rk_npu_w4a8_tune_cache.cpp:71,88,111,
+    src/rk_npu_w4a8_tune_family.cpp:14-15: every entry point refuses before touching a device."""
+    c = capi.W4A8AutotuneConfig()
+    lib.rk_npu_w4a8_autotune_config_init(C.byref(c), 3, 193, 257)
+    assert (c.M, c.N, c.K, c.activation_type, c.allowed_npu_core_mask, c.allowed_cpu_core_mask, c.warmup, c.loops,
+            c.repeats, c.timeout_ms, c.verbose, c.required_k_tile, c.k_tile_multiplier) == (
+                3, 193, 257, capi.W4A8_F32, 7, 0, 2, 8, 3, 500, 0, 0, 0.0)
+    ms = (C.c_int * 2)(1, 4)
+    f = capi.W4A8FamilyConfig()
+    lib.rk_npu_w4a8_family_config_init(C.byref(f), 193, 257, 2, ms)
+    assert (f.base.M, f.base.N, f.base.K, f.m_count, f.m_values[1], bool(f.frequencies)) == (1, 193, 257, 2, 4, False)
+    B = np.zeros((257, 193), np.int8)
+    sc = np.full(193, 0.01, np.float32)
+    s, sx = capi.W4A8Strategy(), capi.W4A8StrategyEx()
+    hit = C.c_int(7)
+    P = capi.RK_NPU_ERR_PARAM
+    assert lib.rk_npu_w4a8_autotune(None, C.byref(c), capi.ptr(B), capi.ptr(sc), C.byref(s), None) == P
+    assert lib.rk_npu_w4a8_autotune_ex(None, C.byref(c), capi.ptr(B), capi.ptr(sc), C.byref(sx), None) == P
+    assert lib.rk_npu_w4a8_autotune_cached(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, 0, C.byref(s), None,
+                                           C.byref(hit)) == P and hit.value == 0
+    assert lib.rk_npu_w4a8_autotune_cached_ex(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, 0, C.byref(sx), None,
+                                              None) == P
+    assert lib.rk_npu_w4a8_autotune_cache_load(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, C.byref(s),
+                                               C.byref(s)) == P
+    assert lib.rk_npu_w4a8_autotune_cache_save(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, C.byref(s),
+                                               C.byref(s)) == P
+    assert lib.rk_npu_w4a8_autotune_cache_load_ex(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, C.byref(sx),
+                                                  C.byref(sx)) == P
+    assert lib.rk_npu_w4a8_autotune_cache_save_ex(None, C.byref(c), capi.ptr(B), capi.ptr(sc), None, C.byref(sx),
+                                                  C.byref(sx)) == P
+    assert lib.rk_npu_w4a8_autotune_cache_load_profile_ex(None, C.byref(c), None, None, C.byref(sx), C.byref(sx)) == P
+    fam, fs = capi.W4A8FamilySummary(), (capi.W4A8Strategy * 2)()
+    fsx = (capi.W4A8StrategyEx * 2)()
+    assert lib.rk_npu_w4a8_autotune_family(None, C.byref(f), capi.ptr(B), capi.ptr(sc), C.byref(fam), fs, None, None) == P
+    assert lib.rk_npu_w4a8_autotune_family_ex(None, C.byref(f), capi.ptr(B), capi.ptr(sc), C.byref(fam), fsx, None,
+                                              None) == P
+    hits, misses = C.c_int(5), C.c_int(5)
+    assert lib.rk_npu_w4a8_autotune_family_cached(None, C.byref(f), capi.ptr(B), capi.ptr(sc), None, 0, C.byref(fam), fs,
+                                                  None, None, C.byref(hits), C.byref(misses)) == P
+    assert (hits.value, misses.value) == (0, 0)
+    assert lib.rk_npu_w4a8_autotune_family_cached_ex(None, C.byref(f), capi.ptr(B), capi.ptr(sc), None, 0, C.byref(fam),
+                                                     fsx, None, None, None, None) == P
+    assert not lib.rk_npu_w4a8_weights_create_tuned(None, C.byref(s), capi.ptr(B), capi.ptr(sc))
+    assert not lib.rk_npu_w4a8_weights_create_tuned_ex(None, C.byref(sx), capi.ptr(B), capi.ptr(sc))
+    assert not lib.rk_npu_w4a8_workspace_create_tuned_ex(None, C.byref(sx))  # revision 0 is not a tuned strategy
+    assert not lib.rk_npu_w4a8_tuning_profile_from_weights(None)
+    assert lib.rk_npu_w4a8_tuning_profile_fingerprint(None) == 0
+    lib.rk_npu_w4a8_tuning_profile_free(None)
