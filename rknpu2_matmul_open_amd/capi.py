@@ -87,6 +87,25 @@ class I4MemoryInfo(C.Structure):
                 ("wave_count", C.c_uint32), ("tasks_per_wave", C.c_uint32)]
 
 
+class I4Config(C.Structure):
+    _fields_ = [("M", C.c_int), ("N", C.c_int), ("K", C.c_int), ("m_tile", C.c_int), ("k_tile", C.c_int),
+                ("n_tile", C.c_int), ("npu_core_mask", C.c_uint32), ("timeout_ms", C.c_uint32),
+                ("pipeline", C.c_int), ("cpu_threads", C.c_int)]
+
+
+class I4Timings(C.Structure):
+    _fields_ = [("pack_us", C.c_double), ("sync_us", C.c_double), ("submit_us", C.c_double),
+                ("reduce_us", C.c_double), ("total_us", C.c_double)]
+
+
+class I4InputTile(C.Structure):
+    _fields_ = [("m0", C.c_int), ("rows", C.c_int), ("k0", C.c_int), ("k", C.c_int), ("padded_k", C.c_int),
+                ("dst", C.POINTER(C.c_uint8)), ("bytes", C.c_uint64)]
+
+
+I4_INPUT_PRODUCER = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(I4InputTile))
+
+
 class W4A8Config(C.Structure):
     _fields_ = [("M", C.c_int), ("N", C.c_int), ("K", C.c_int), ("m_tile", C.c_int),
                 ("k_tile", C.c_int), ("n_tile", C.c_int), ("npu_core_mask", C.c_uint32),
@@ -250,6 +269,17 @@ _PROTOTYPES = {
     "rk_npu_w4a8_run_f16": (C.c_int, [P, P, P, P, C.POINTER(W4A8Timings)]),
     "rk_npu_w4a8_run_swiglu_f32": (C.c_int, [P, P, P, P, C.POINTER(W4A8Timings)]),
     "rk_npu_w4a8_run_ffn_f32": (C.c_int, [P, P, P, P, P, P, P, C.POINTER(W4A8FfnTimings)]),
+    # rk_npu_matmul_i4.h
+    "rk_npu_i4_config_init": (None, [C.POINTER(I4Config), C.c_int, C.c_int, C.c_int]),
+    "rk_npu_i4_memory_query": (C.c_int, [C.POINTER(I4Config), C.POINTER(I4MemoryInfo)]),
+    "rk_npu_i4_weights_memory_query": (C.c_int, [C.POINTER(I4WeightConfig), C.POINTER(C.c_uint64)]),
+    "rk_npu_i4i4i32_weights_create": (P, [P, C.POINTER(I4WeightConfig), P]),
+    "rk_npu_i4i4i32_weights_free": (None, [P]),
+    "rk_npu_i4_workspace_create": (P, [P, C.POINTER(I4Config)]),
+    "rk_npu_i4_workspace_free": (None, [P]),
+    "rk_npu_i4i4i32_run": (C.c_int, [P, P, P, P, C.POINTER(I4Timings)]),
+    "rk_npu_i4i4i32_run_with_producer": (C.c_int, [P, P, I4_INPUT_PRODUCER, C.c_void_p, P, C.POINTER(I4Timings)]),
+    "rk_npu_i4_pack_a_tile": (C.c_int, [C.POINTER(I4InputTile), P, C.c_int]),
     # rk_npu_w4a8_tune.h
     "rk_npu_w4a8_autotune_config_init": (None, [C.POINTER(W4A8AutotuneConfig), C.c_int, C.c_int, C.c_int]),
     "rk_npu_w4a8_family_config_init": (None, [C.POINTER(W4A8FamilyConfig), C.c_int, C.c_int, C.c_int,

@@ -486,6 +486,10 @@ rk_npu_w4a8_weights* w4a8_create_weights(rk_npu_iommu_domain* domain, const rk_n
 
 const W4Profile& w4a8_profile_of(const rk_npu_w4a8_weights* weights) { return weights->profile; }
 
+bool i4_tile_certified(const int8_t* B, int K, int N, int k_tile) {
+    return largest_certified_tile(B, K, N, k_tile) == k_tile;
+}
+
 } // namespace rkhost
 
 extern "C" {

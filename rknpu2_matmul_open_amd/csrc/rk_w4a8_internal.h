@@ -46,6 +46,10 @@ const W4Profile& w4a8_profile_of(const rk_npu_w4a8_weights* weights);
 // RK_NPU_W4A8_K_TILE_MULTIPLIER: 1 when unset, < 0 when set but invalid.
 double w4a8_env_multiplier();
 
+// True when the INT16-partial certificate holds for exactly this K tile
+// (multiple of 32) on B[K, N]; false also for a code outside [-8, 7].
+bool i4_tile_certified(const int8_t* B, int K, int N, int k_tile);
+
 } // namespace rkhost
 
 #endif

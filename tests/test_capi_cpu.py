@@ -62,6 +62,8 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
              ("rk_npu_matmul_workspace_requirements", capi.WorkspaceRequirements),
              ("rk_npu_matmul_weight_requirements", capi.WeightRequirements),
              ("rk_npu_i4_weight_config", capi.I4WeightConfig), ("rk_npu_i4_memory_info", capi.I4MemoryInfo),
+             ("rk_npu_i4_config", capi.I4Config), ("rk_npu_i4_timings", capi.I4Timings),
+             ("rk_npu_i4_input_tile", capi.I4InputTile),
              ("rk_npu_w4a8_config", capi.W4A8Config), ("rk_npu_w4a8_memory_info", capi.W4A8MemoryInfo),
              ("rk_npu_w4a8_options", capi.W4A8Options), ("rk_npu_w4a8_memory_info_ex", capi.W4A8MemoryInfoEx),
              ("rk_npu_w4a8_timings", capi.W4A8Timings), ("rk_npu_w4a8_weight_info", capi.W4A8WeightInfo),
@@ -345,3 +347,73 @@ def test_w4a8_tune_entry_points_without_a_context(lib):
     assert not lib.rk_npu_w4a8_tuning_profile_from_weights(None)
     assert lib.rk_npu_w4a8_tuning_profile_fingerprint(None) == 0
     lib.rk_npu_w4a8_tuning_profile_free(None)
+
+
+def _i4_code(packed, index):
+    q = (int(packed[index // 2]) >> (0 if index & 1 else 4)) & 15
+    return q - 16 if q >= 8 else q
+
+
+def test_i4_host_side(lib):
+    """reference tests/test_i4_cpu.cpp:16-31 (native K32 activation panel: signed codes, padding, guard bytes,
+    rejected code) and :49-59,81-89 (memory accounting and range checks)."""
+    for k in (1, 31, 32, 33, 127, 479, 480, 991, 992, 1472, 1984, 2048):
+        rows, pk, lda = 3, (k + 31) // 32 * 32, k + 7
+        a = ((np.arange(5 * lda) * 7 % 16) - 8).astype(np.int8)
+        packed = np.full(rows * pk // 2 + 16, 0x5A, np.uint8)
+        t = capi.I4InputTile(1, rows, 2, k, pk, packed.ctypes.data_as(C.POINTER(C.c_uint8)), rows * pk // 2)
+        assert lib.rk_npu_i4_pack_a_tile(C.byref(t), capi.ptr(a), lda) == 0
+        for m in range(rows):
+            for j in range(pk):
+                want = int(a[(m + 1) * lda + j + 2]) if j < k else 0
+                assert _i4_code(packed, (j // 32 * rows + m) * 32 + j % 32) == want
+        assert (packed[-16:] == 0x5A).all()
+        a[lda + 2] = 8
+        assert lib.rk_npu_i4_pack_a_tile(C.byref(t), capi.ptr(a), lda) == capi.RK_NPU_ERR_PARAM
+        t.bytes -= 1
+        a[lda + 2] = 0
+        assert lib.rk_npu_i4_pack_a_tile(C.byref(t), capi.ptr(a), lda) == capi.RK_NPU_ERR_PARAM
+    cfg = capi.I4Config()
+    lib.rk_npu_i4_config_init(C.byref(cfg), 129, 65, 513)
+    assert (cfg.M, cfg.N, cfg.K, cfg.m_tile, cfg.k_tile, cfg.n_tile, cfg.npu_core_mask, cfg.timeout_ms,
+            cfg.pipeline, cfg.cpu_threads) == (129, 65, 513, 128, 480, 1024, 1, 500, 1, 1)
+    cfg.m_tile, cfg.n_tile = 64, 64
+    info = capi.I4MemoryInfo()
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == 0
+    assert (info.wave_count, info.tasks_per_wave, info.packed_weight_bytes) == (2, 6, 34816)
+    assert info.input_bytes == 2 * 129 * 480 // 2 and info.partial_bytes == 2 * 129 * 128 * 2
+    cfg.k_tile = 512
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == 0
+    P = capi.RK_NPU_ERR_PARAM
+    cfg.k_tile = 2080
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == P
+    cfg.k_tile, cfg.npu_core_mask = 480, 5
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == P
+    cfg.npu_core_mask, cfg.K = 1, 2 ** 31 - 1
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == P
+    for n in (4160, 8128):
+        lib.rk_npu_i4_config_init(C.byref(cfg), 2, n, 64)
+        cfg.n_tile = n
+        assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == 0 and info.tasks_per_wave == 1
+    cfg.n_tile = 8192
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == P
+    lib.rk_npu_i4_config_init(C.byref(cfg), 2, 8192, 64)  # only the tile is capped: 8192 = 8128 + 64
+    cfg.n_tile = 8128
+    assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == 0 and info.tasks_per_wave == 2
+    for field, value in (("m_tile", 0), ("m_tile", 129), ("n_tile", 96), ("pipeline", 2), ("cpu_threads", 5),
+                         ("timeout_ms", 0), ("M", 0), ("npu_core_mask", 7)):
+        lib.rk_npu_i4_config_init(C.byref(cfg), 4, 128, 64)
+        setattr(cfg, field, value)
+        assert lib.rk_npu_i4_memory_query(C.byref(cfg), C.byref(info)) == P, field
+    wc = capi.I4WeightConfig(513, 65, 480)
+    nbytes = C.c_uint64(0)
+    assert lib.rk_npu_i4_weights_memory_query(C.byref(wc), C.byref(nbytes)) == 0 and nbytes.value == 544 * 128 // 2
+    wc.k_tile = 0
+    assert lib.rk_npu_i4_weights_memory_query(C.byref(wc), C.byref(nbytes)) == P
+    # no device needed to be refused
+    B = np.zeros((513, 65), np.int8)
+    assert not lib.rk_npu_i4i4i32_weights_create(None, C.byref(wc), capi.ptr(B))
+    assert not lib.rk_npu_i4_workspace_create(None, C.byref(cfg))
+    assert lib.rk_npu_i4i4i32_run(None, None, capi.ptr(B), capi.ptr(B), None) == P
+    lib.rk_npu_i4i4i32_weights_free(None)
+    lib.rk_npu_i4_workspace_free(None)
