@@ -967,8 +967,17 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     constexpr int NSW = (TM == 4 || (TM == 2 && W4)) ? 8 : 4;
     constexpr int NBUF = WK_NBUF, G = WK_G, D = WK_D, BM = 32 * TM, BUF = WK_BUF;
     constexpr int UNR = 16;            // sub-steps per unrolled trip: multiple of NSW, NBUF, G and 2
-    constexpr int LPS = 1 + KTW * TN;  // loads per sub-step and wave
-    constexpr int NWREG = KTW * TN;    // weight registers (and unpack items) per sub-step
+    // int4 weights come in 1 KiB super-tiles of two k-tiles (16 bytes per lane).  When a
+    // wave has two or more k-tiles per sub-step it takes WHOLE super-tiles (k-tiles
+    // 4v + 2*wk, 4v + 2*wk + 1), one 16-byte load each; taking every second k-tile
+    // instead would make both k-halves fetch every cache line for half of its bytes,
+    // which doubles the weight traffic through the L1 and makes that the limit of the
+    // 64- and 32-row tiles.  (With one k-tile per wave and sub-step, TM = 4, the two
+    // halves of a super-tile necessarily go to the two waves, 8 bytes per lane each.)
+    constexpr bool PAIRED = W4 && KTW >= 2;
+    constexpr int NWOP = KTW * TN;                              // weight operands (k-tile x column block) per sub-step
+    constexpr int NWREG = PAIRED ? (KTW / 2) * TN : KTW * TN;   // weight loads (registers of the ring) per sub-step
+    constexpr int LPS = 1 + NWREG;                              // loads per sub-step and wave
     static_assert(UNR % NSW == 0 && UNR % NBUF == 0 && UNR % G == 0, "slot arithmetic must be compile-time");
     static_assert(D >= NSW + G - 1 && NBUF >= D + G, "see the ordering rules above");
     static_assert((NSW - 2) * LPS <= 63, "vmcnt field");
@@ -1005,16 +1014,16 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int pb = nblk * 8 + wn * TN + j;
-        wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0 * KTW) * 1024 + wk * 8
+        wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0 * KTW) * 1024 + (PAIRED ? wk * 1024 : wk * 8)
                      : Wb + ((size_t)pb * KB + (size_t)kstep0 * KTS + wk) * 1024 + W_BIAS;
     }
     const unsigned lane_off = lane * 16;
     constexpr int A_STEP = KTS * 1024, W_STEP = W4 ? KTW * 1024 : KTS * 1024;
-    using wraw_t = typename std::conditional<W4, v2i, v4i>::type;
+    using wraw_t = typename std::conditional<W4 && !PAIRED, v2i, v4i>::type;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds_raw;
     const uint32_t copy_dst = lds_base + wave * 1024; // this wave's chunk inside buffer 0
     // LDS byte addresses of this lane's fragment (row block 0, this wave's first k-tile) in buffers 0 and 8
-    uint32_t frag_lo = lds_base + wk * 1024 + lane * 16;
+    uint32_t frag_lo = lds_base + wk * (PAIRED ? 2048 : 1024) + lane * 16;
     uint32_t frag_hi = frag_lo + 8 * BUF;
     int a_left = ksteps - 1, w_left = ksteps - 1; // how often the sources may still advance
 
@@ -1028,7 +1037,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
 
     wraw_t wring[NSW][NWREG]; // weight prefetch ring, index u * TN + j
     v4i afr[2][4];            // activation fragments (index u * TM + i), this sub-step / next
-    v4i wop[2][NWREG];        // int4 only: unpacked operands, this sub-step / next
+    v4i wop[2][NWOP];         // int4 only: unpacked operands (index u * TN + j), this sub-step / next
 
     auto copy_a = [&](int buf) { // global -> LDS, 16 bytes per lane, lane-contiguous
         asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(asrc),
@@ -1043,7 +1052,9 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             const unsigned off = lane_off; // (locals: asm operands cannot name captures of an enclosing lambda)
             const uint8_t* base = wsrc[J];
             wraw_t r;
-            if constexpr (W4)
+            if constexpr (PAIRED) // U counts this wave's super-tiles: every second one of the sub-step
+                asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(r) : "v"(off), "s"(base), "n"(U * 2048));
+            else if constexpr (W4)
                 asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(r) : "v"(off), "s"(base), "n"(U * 1024));
             else
                 asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(r) : "v"(off), "s"(base), "n"(U * 2048 - W_BIAS));
@@ -1063,7 +1074,8 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     auto read_frag = [&](v4i& dst, auto buf_tag, auto f_tag) {
         constexpr int BUFI = decltype(buf_tag)::value, FI = decltype(f_tag)::value;
         constexpr int U = FI / TM, I = FI % TM;
-        constexpr int OFF = (BUFI % 8) * BUF + (I * KTS + 2 * U) * 1024;
+        constexpr int KT = PAIRED ? (U / 2) * 4 + U % 2 : 2 * U; // this wave's u-th k-tile, relative to its first
+        constexpr int OFF = (BUFI % 8) * BUF + (I * KTS + KT) * 1024;
         static_assert(OFF < 65536, "ds_read offset field");
         const uint32_t addr = BUFI < 8 ? frag_lo : frag_hi;
         asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
@@ -1071,12 +1083,20 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     auto frags_wait = [&](v4i* f) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3])::"memory");
     };
-    auto unpack_one = [&](v4i& dst, const wraw_t& raw) {
-        if constexpr (W4) {
-            dst.x = (raw.x << 4) & 0xF0F0F0F0;
-            dst.y = raw.x & 0xF0F0F0F0;
-            dst.z = (raw.y << 4) & 0xF0F0F0F0;
-            dst.w = raw.y & 0xF0F0F0F0;
+    // ring register e of a sub-step -> its operand(s) in dst[NWOP]
+    auto unpack_item = [&](v4i* dst, const wraw_t* ring_regs, auto e_tag) {
+        constexpr int E = decltype(e_tag)::value;
+        if constexpr (PAIRED) {
+            constexpr int V = E / TN, J = E % TN; // super-tile V of this wave = its k-tiles 2V, 2V + 1
+            const wraw_t raw = ring_regs[E];
+            dst[(2 * V) * TN + J] = v4i{(raw.x << 4) & (int)0xF0F0F0F0, raw.x & (int)0xF0F0F0F0,
+                                        (raw.y << 4) & (int)0xF0F0F0F0, raw.y & (int)0xF0F0F0F0};
+            dst[(2 * V + 1) * TN + J] = v4i{(raw.z << 4) & (int)0xF0F0F0F0, raw.z & (int)0xF0F0F0F0,
+                                            (raw.w << 4) & (int)0xF0F0F0F0, raw.w & (int)0xF0F0F0F0};
+        } else if constexpr (W4) {
+            const wraw_t raw = ring_regs[E];
+            dst[E] = v4i{(raw.x << 4) & (int)0xF0F0F0F0, raw.x & (int)0xF0F0F0F0, (raw.y << 4) & (int)0xF0F0F0F0,
+                         raw.y & (int)0xF0F0F0F0};
         }
     };
 
@@ -1105,9 +1125,11 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
             if constexpr (Q < 4) read_frag(afr[F ^ 1][Q], NextBuf{}, std::integral_constant<int, Q>{});
             if constexpr (Q == 1) w_wait(wring[(SLOT + 1) % NSW]);
             if constexpr (W4 && Q >= 2 && Q < 6) {
-#pragma unroll
-                for (int e = (Q - 2) * UPS; e < (Q - 1) * UPS; ++e)
-                    if (e < NWREG) unpack_one(wop[F ^ 1][e], wring[(SLOT + 1) % NSW][e]);
+                static_for<UPS>([&](auto t_tag) {
+                    constexpr int E = (Q - 2) * UPS + decltype(t_tag)::value;
+                    if constexpr (E < NWREG)
+                        unpack_item(wop[F ^ 1], wring[(SLOT + 1) % NSW], std::integral_constant<int, E>{});
+                });
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -1153,8 +1175,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mbloc
     w_wait(wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
     asm volatile("s_barrier" ::: "memory");
     static_for<4>([&](auto f_tag) { read_frag(afr[0][decltype(f_tag)::value], std::integral_constant<int, 0>{}, f_tag); });
-#pragma unroll
-    for (int e = 0; e < NWREG; ++e) unpack_one(wop[0][e], wring[0][e]);
+    static_for<NWREG>([&](auto e_tag) { unpack_item(wop[0], wring[0], e_tag); });
     frags_wait(afr[0]);
 
     int s = 0;
