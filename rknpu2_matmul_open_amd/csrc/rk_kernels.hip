@@ -506,8 +506,14 @@ __device__ __forceinline__ void store_out(void* C, int epi, size_t index, int ac
 // memory); activations sit in LDS; lanes l and l+32 hold the two 16-byte
 // halves of a k-tile for column l%32, so the cross-lane reduction is one xor
 // shuffle, followed by a small LDS reduction across waves.
-constexpr int GEMV_WAVES = 8;
-constexpr int GEMV_UNROLL = 8;
+#ifndef RK_GEMV_WAVES
+#define RK_GEMV_WAVES 8
+#endif
+#ifndef RK_GEMV_UNROLL
+#define RK_GEMV_UNROLL 8
+#endif
+constexpr int GEMV_WAVES = RK_GEMV_WAVES;
+constexpr int GEMV_UNROLL = RK_GEMV_UNROLL;
 constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
 
 constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
