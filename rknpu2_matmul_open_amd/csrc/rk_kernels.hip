@@ -197,17 +197,24 @@ __device__ __forceinline__ uint4 quantize16(const float* v, float inv) {
 
 constexpr int QR_CACHE = 4; // 16-element chunks kept in registers per thread
 
+// `split` workgroups share a row (blockIdx.x = row * split + part), each taking a
+// contiguous range of its 16-element chunks.  Only the modes that do not scan the
+// row for its maximum are launched with split > 1: re-quantization finds the
+// maximum in the partial maxima the GEMM left behind, which every part reads.
 template <typename T>
-__global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
+__global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int split) {
     __shared__ float wave_max[4];
     __shared__ int wave_bad[4];
-    const int m = blockIdx.x, t = threadIdx.x;
+    const int m = blockIdx.x / split, part = blockIdx.x - m * split, t = threadIdx.x;
     if (a.active_blocks && m >= a.active_blocks[0] * 32) return;
     const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
-    const int nchunks = (K + 15) >> 4;
+    const int row_chunks = (K + 15) >> 4;
+    const int per_part = (row_chunks + split - 1) / split;
+    const int chunk0 = part * per_part;                         // this workgroup's chunks: chunk0 .. nchunks - 1
+    const int nchunks = min(row_chunks, chunk0 + per_part);
     const T* row = static_cast<const T*>(a.src) + (size_t)m * K;
     const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
-    const bool cached = nchunks <= 256 * QR_CACHE;
+    const bool cached = nchunks - chunk0 <= 256 * QR_CACHE;
     const int mode = a.mode;
     if constexpr (sizeof(T) == 1) {
         // int8 input is re-tiled byte for byte (the full range -128..127 is legal
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
             }
         }
         const int8_t* brow = reinterpret_cast<const int8_t*>(row);
-        for (int c = t; c < nchunks; c += 256) {
+        for (int c = chunk0 + t; c < nchunks; c += 256) {
             uint32_t w[4] = {0, 0, 0, 0};
             if (vec && c * 16 + 16 <= K) {
                 const uint4 v4 = *reinterpret_cast<const uint4*>(brow + c * 16);
@@ -252,7 +259,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     if (cached) {
 #pragma unroll
         for (int i = 0; i < QR_CACHE; ++i) {
-            const int c = t + i * 256;
+            const int c = chunk0 + t + i * 256;
             if (c < nchunks) {
                 RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
                 if (need_max) {
@@ -265,7 +272,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
             }
         }
     } else if (need_max) {
-        for (int c = t; c < nchunks; c += 256) {
+        for (int c = chunk0 + t; c < nchunks; c += 256) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
 #pragma unroll
@@ -322,7 +329,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
 
     int ndest = 1;
     if (a.dest_rows) ndest = a.dest_stride;
-    if (t == 0) {
+    if (t == 0 && part == 0) {
         if (!a.dest_rows) {
             if (a.scale && mode != RKH_Q_W8_STATIC && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
         } else {
@@ -350,11 +357,11 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a) {
     if (cached) {
 #pragma unroll
         for (int i = 0; i < QR_CACHE; ++i) {
-            const int c = t + i * 256;
+            const int c = chunk0 + t + i * 256;
             if (c < nchunks) emit(c, v[i]);
         }
     } else {
-        for (int c = t; c < nchunks; c += 256) {
+        for (int c = chunk0 + t; c < nchunks; c += 256) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
             emit(c, tmp);
@@ -1883,11 +1890,18 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
-    const dim3 grid(args->M);
+    // Re-quantization of a few long rows: several workgroups per row, about 256 chunks
+    // each, until the grid has a few hundred workgroups.
+    int split = 1;
+    if ((mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) && !args->dest_rows) {
+        const int row_chunks = (args->K + 15) / 16;
+        while (split < 8 && args->M * split < 512 && row_chunks / (split * 2) >= 128) split *= 2;
+    }
+    const dim3 grid(args->M * split);
     switch (args->in_dtype) {
-    case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args); break;
-    case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args); break;
-    case RKH_I8: hipLaunchKernelGGL(quant_rows_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args); break;
+    case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args, split); break;
+    case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args, split); break;
+    case RKH_I8: hipLaunchKernelGGL(quant_rows_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args, split); break;
     default: return RKH_ERR_RUNTIME;
     }
     RKH_CHECK(hipGetLastError());
