@@ -18,8 +18,9 @@
  * Differences from the RK3588 limits: intermediate may be up to 8192 (the
  * reference stops at 512 because of a fixed CPU scratch row); npu_cores,
  * cpu_threads, native_input and timeout_ms are range-checked and unused.
- * The W4 / mixed / slot-bank / blob import-export entry points of the
- * reference header (:88-143) are not part of this library.
+ * INT4 experts, mixed banks, slot banks and packed expert records (reference
+ * :83-143) are the same arithmetic with weight codes restricted to [-8, 7];
+ * see the second half of this header.
  */
 #ifndef RK_NPU_MOE_W8_H
 #define RK_NPU_MOE_W8_H
@@ -116,15 +117,48 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
                           const int32_t* expert_ids, const float* route_weights,
                           float* output, rk_npu_moe_w8_timings* timings);
 
-/* ---- other expert formats of the reference (reference :83-143) ---------------
- * W4 experts, mixed routed-W4 + shared-W8 experts, mutable slot banks and the
- * packed expert record import / export exist in the reference for the RK3588
- * NPU's int4 mode and its expert paging.  They are outside this build's path:
- * the entry points are exported so that callers link, and every one of them
- * declines -- constructors return NULL, the record calls return
- * RK_NPU_ERR_PARAM, the record size query returns 0 -- without touching the
- * device or the caller's buffers. */
-#define RK_NPU_MOE_QUANT_BLOB_VERSION 3u
+/* ---- INT4 experts, mixed banks, slot banks, packed records (reference :83-143) ----
+ *
+ * Expert tensors are passed exactly as for the W8 factories (one int8_t per
+ * weight, the same scale vectors); an INT4 expert's codes must lie in [-8, 7].
+ * On the RK3588 these formats select the NPU's int4 mode, K-sliced INT16
+ * partials and their certificates; here an INT4 code is an int8 value, the
+ * int8 MFMA path accumulates it in int32 without any intermediate narrowing,
+ * and results are bit-identical to the W8 path given the same codes.  What is
+ * kept from the reference is the contract: geometry (hidden and intermediate
+ * multiples of 64, hidden <= 8128), code range validation, native_input = 0,
+ * and that weights only bind to a workspace made by the factory of the same
+ * format (RK_NPU_ERR_PARAM otherwise).  All handles use the run / free / byte
+ * query functions above.
+ *
+ *   quant_*      every expert INT4, the shared one included (reference :83-94).
+ *                _full_k is the same here: there is no K slicing to certify.
+ *   w4_*         routed experts INT4, the shared expert full-range int8
+ *                (reference :96-106).
+ *   *_slots_create  a bank whose routed slots start empty (zero weights, zero
+ *                scales) and are filled by import; quant_slots needs
+ *                shared_expert = 0, w4_slots needs shared_expert = 1 and packs
+ *                `shared` at creation (reference :101-119).  The caller owns
+ *                the logical expert -> slot map and passes slot numbers as
+ *                expert_ids.
+ *
+ * Packed record of one INT4 expert, rk_npu_moe_quant_expert_blob_bytes() bytes
+ * (0 for W8 handles): {u32 magic "RKHM", u32 RK_NPU_MOE_QUANT_BLOB_VERSION,
+ * u32 hidden, u32 intermediate}, the gate/up image and the down image in this
+ * library's execution layout, 2*intermediate gate/up scales, hidden down
+ * scales.  Records are native to this library (not interchangeable with the
+ * RK3588 build's) and identical between the all-INT4 and the mixed bank of one
+ * geometry.  export / import accept a larger buffer than the record, reject a
+ * shorter one, a W8 handle, the shared int8 expert, an out-of-range slot, a
+ * foreign header and non-finite or non-positive scales with RK_NPU_ERR_PARAM;
+ * a rejected import leaves the slot unchanged.  Import only between blocking
+ * runs that use the bank.  The timed import reports validate_us (header and
+ * scale checks), copy_us (scales), gate_sync_us / down_sync_us (the two weight
+ * images) and total_us.
+ *
+ * swap_slots exchanges the contents of two slots of all-INT4 banks of equal
+ * geometry in the same context and domain (device-side copy; the reference
+ * exchanges buffer ownership, the observable result is the same). */
 typedef struct rk_npu_moe_import_timings {
     double copy_us, validate_us, gate_sync_us, down_sync_us, total_us;
 } rk_npu_moe_import_timings;

@@ -200,6 +200,11 @@ class MoeTimings(C.Structure):
                 ("middle_tasks", C.c_uint32), ("gemm_tasks", C.c_uint32)]
 
 
+class MoeImportTimings(C.Structure):
+    _fields_ = [("copy_us", C.c_double), ("validate_us", C.c_double), ("gate_sync_us", C.c_double),
+                ("down_sync_us", C.c_double), ("total_us", C.c_double)]
+
+
 P = C.c_void_p
 _PROTOTYPES = {
     # rk_npu_common.h

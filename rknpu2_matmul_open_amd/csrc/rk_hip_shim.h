@@ -76,6 +76,7 @@ int rkh_h2d(void* stream, void* dst, const void* src, size_t bytes);   /* async 
 int rkh_d2h(void* stream, void* dst, const void* src, size_t bytes);   /* async */
 int rkh_d2d(void* stream, void* dst, const void* src, size_t bytes);   /* async */
 int rkh_fill32(void* stream, void* dst, uint32_t value, size_t words); /* fill kernel */
+int rkh_exchange32(void* stream, void* x, void* y, size_t words);      /* swaps two disjoint arrays, async */
 int rkh_sync(void* stream);
 /* Test hook: make the n-th next rkh_malloc fail (n = 1 fails the next one,
  * 0 disables).  Lets allocation-failure paths be exercised from the host. */

@@ -56,6 +56,17 @@ __global__ void fill32_kernel(uint32_t* dst, uint32_t value, size_t words) {
     for (; i < words; i += stride) dst[i] = value;
 }
 
+// Exchanges two disjoint arrays of 32-bit words in place.
+__global__ void exchange32_kernel(uint32_t* x, uint32_t* y, size_t words) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < words; i += stride) {
+        const uint32_t a = x[i], b = y[i];
+        x[i] = b;
+        y[i] = a;
+    }
+}
+
 // ------------------------------------------------------------ weight pack
 // One thread produces one lane's 16 bytes of one tile.
 __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__ src, int K, int N,
@@ -1826,6 +1837,14 @@ int rkh_fill32(void* stream, void* dst, uint32_t value, size_t words) {
     const int blocks = (int)((words + 255) / 256 < 4096 ? (words + 255) / 256 : 4096);
     hipLaunchKernelGGL(fill32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                        static_cast<uint32_t*>(dst), value, words);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+int rkh_exchange32(void* stream, void* x, void* y, size_t words) {
+    if (!words) return RKH_OK;
+    const int blocks = (int)((words + 255) / 256 < 4096 ? (words + 255) / 256 : 4096);
+    hipLaunchKernelGGL(exchange32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<uint32_t*>(x), static_cast<uint32_t*>(y), words);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }

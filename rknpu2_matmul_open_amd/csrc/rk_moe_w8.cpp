@@ -40,6 +40,24 @@ bool valid(const rk_npu_moe_w8_config& c) {
            (c.native_input == 0 || c.native_input == 1) && c.timeout_ms >= 1 &&
            c.timeout_ms <= 60000 && c.middle == RK_NPU_MOE_MIDDLE_CPU;
 }
+// Expert formats (reference src/rk_npu_moe_w8.cpp:366-387).  W4 experts hold
+// signed INT4 codes in the same int8 arrays; the arithmetic is that of the W8
+// path with codes restricted to [-8, 7] (the reference's own test runs one body
+// against both), so they execute on the same kernels and are kept as int8 on
+// the device.
+enum Mode { kW8 = 0, kW4 = 1, kRoutedW4SharedW8 = 2 };
+bool expert_is_w4(int mode, int expert, int routed) {
+    return mode == kW4 || (mode == kRoutedW4SharedW8 && expert < routed);
+}
+// reference :384-387 (8128 = widest INT4 task of the NPU)
+bool valid_w4(const rk_npu_moe_w8_weight_config& c) {
+    return valid(c) && c.hidden % 64 == 0 && c.intermediate % 64 == 0 && c.hidden <= 8128;
+}
+bool int4_codes(const int8_t* p, size_t n) {
+    unsigned bad = 0;
+    for (size_t i = 0; i < n; ++i) bad |= (unsigned)(uint8_t)(p[i] + 8) & 0xf0u;
+    return bad == 0;
+}
 bool overlap(const void* a, size_t na, const void* b, size_t nb) {
     const auto x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
     return x <= y ? y - x < na : x - y < nb;
@@ -50,6 +68,7 @@ bool overlap(const void* a, size_t na, const void* b, size_t nb) {
 struct rk_npu_moe_w8_weights {
     Owner owner;
     rk_npu_moe_w8_weight_config config{};
+    int mode = kW8;
     int count = 0;              // routed + shared
     size_t gate_stride = 0;     // bytes between experts in gate_up
     size_t down_stride = 0;
@@ -65,6 +84,7 @@ struct rk_npu_moe_w8_weights {
 struct rk_npu_moe_w8_workspace {
     Owner owner;
     rk_npu_moe_w8_config config{};
+    int mode = kW8;
     int slots = 0, max_blocks = 0, sorted_rows = 0;
     DeviceBuffer input;        // [max_rows, H] fp32 (or int8) as uploaded
     DeviceBuffer token_scale;  // [max_rows]
@@ -212,7 +232,7 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
 }
 
 int check_handles(const rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w) {
-    if (!same(ws->config.weights, w->config)) return RK_NPU_ERR_PARAM;
+    if (ws->mode != w->mode || !same(ws->config.weights, w->config)) return RK_NPU_ERR_PARAM;
     if (!w->owner.same(ws->owner)) return RK_NPU_ERR_DOMAIN;
     return RK_NPU_OK;
 }
@@ -315,58 +335,111 @@ void rk_npu_moe_w8_config_init(rk_npu_moe_w8_config* c, int hidden, int intermed
     c->timeout_ms = 1000;
 }
 
-rk_npu_moe_w8_weights* rk_npu_moe_w8_weights_create(rk_npu_iommu_domain* domain,
-                                                    const rk_npu_moe_w8_weight_config* config,
-                                                    const rk_npu_moe_w8_expert* experts) {
-    if (!domain || !domain->ctx || !config || !experts || !valid(*config)) return nullptr;
+} // extern "C"
+
+namespace {
+
+// Packs one expert into slot e of the bank (the context's submit mutex is held).
+int pack_expert(rk_npu_moe_w8_weights* w, DeviceBuffer& raw, int e, const rk_npu_moe_w8_expert& x) {
+    const int H = w->config.hidden, I = w->config.intermediate;
+    void* stream = w->owner.ctx->stream;
+    int rc = rkh_h2d(stream, raw.as<>(), x.gate_up, (size_t)H * 2 * I);
+    if (!rc) rc = rkh_pack_w8(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e);
+    if (!rc) rc = rkh_h2d(stream, raw.as<>(), x.down, (size_t)I * H);
+    if (!rc) rc = rkh_pack_w8(stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e);
+    if (!rc) rc = rkh_h2d(stream, w->gate_scales.as<float>() + (size_t)e * 2 * I, x.gate_up_scales, (size_t)2 * I * sizeof(float));
+    if (!rc) rc = rkh_h2d(stream, w->down_scales.as<float>() + (size_t)e * H, x.down_scales, (size_t)H * sizeof(float));
+    // the staging buffer is reused: finish this expert before the next copy lands
+    if (!rc) rc = rkh_sync(stream);
+    return rc;
+}
+
+bool expert_ok(const rk_npu_moe_w8_expert& x, int H, int I, bool w4) {
+    if (!x.gate_up || !x.down || !finite_positive(x.gate_up_scales, (size_t)2 * I) ||
+        !finite_positive(x.down_scales, (size_t)H))
+        return false;
+    return !w4 || (int4_codes(x.gate_up, (size_t)H * 2 * I) && int4_codes(x.down, (size_t)I * H));
+}
+
+// experts: all routed + shared experts, or NULL for a bank of empty slots (then
+// `shared`, if given, fills the shared expert's slot).  Empty slots hold zero
+// weights and zero scales until a record is imported.
+rk_npu_moe_w8_weights* create_weights(rk_npu_iommu_domain* domain, const rk_npu_moe_w8_weight_config* config,
+                                      const rk_npu_moe_w8_expert* experts, int mode,
+                                      const rk_npu_moe_w8_expert* shared) {
+    if (!domain || !domain->ctx || !config || !(mode == kW8 ? valid(*config) : valid_w4(*config))) return nullptr;
     const int H = config->hidden, I = config->intermediate;
     const int count = config->routed_experts + config->shared_expert;
-    for (int e = 0; e < count; ++e) {
-        const auto& x = experts[e];
-        if (!x.gate_up || !x.down || !finite_positive(x.gate_up_scales, (size_t)2 * I) ||
-            !finite_positive(x.down_scales, (size_t)H))
-            return nullptr;
-    }
+    if (experts)
+        for (int e = 0; e < count; ++e)
+            if (!expert_ok(experts[e], H, I, expert_is_w4(mode, e, config->routed_experts))) return nullptr;
+    if (shared && !expert_ok(*shared, H, I, expert_is_w4(mode, config->routed_experts, config->routed_experts)))
+        return nullptr;
     std::unique_ptr<rk_npu_moe_w8_weights> w(new (std::nothrow) rk_npu_moe_w8_weights());
     if (!w) return nullptr;
     w->owner.bind(domain);
     w->config = *config;
+    w->mode = mode;
     w->count = count;
     w->gate_stride = rkh_tiled_i8_bytes(2 * I, H, RKH_COL_ALIGN);
     w->down_stride = rkh_tiled_i8_bytes(H, I, RKH_COL_ALIGN);
     rk_npu_ctx* ctx = domain->ctx;
     std::lock_guard<std::mutex> lock(ctx->submit_mutex);
     DeviceBuffer raw;
-    if (w->gate_up.alloc(w->owner, w->gate_stride * count, false) ||
-        w->down.alloc(w->owner, w->down_stride * count, false) ||
-        w->gate_scales.alloc(w->owner, (size_t)count * 2 * I * sizeof(float), false) ||
-        w->down_scales.alloc(w->owner, (size_t)count * H * sizeof(float), false) ||
+    const bool zero = experts == nullptr;
+    if (w->gate_up.alloc(w->owner, w->gate_stride * count, zero) ||
+        w->down.alloc(w->owner, w->down_stride * count, zero) ||
+        w->gate_scales.alloc(w->owner, (size_t)count * 2 * I * sizeof(float), zero) ||
+        w->down_scales.alloc(w->owner, (size_t)count * H * sizeof(float), zero) ||
         raw.alloc(w->owner, (size_t)H * 2 * I, false))
         return nullptr;
-    for (int e = 0; e < count; ++e) {
-        const auto& x = experts[e];
-        int rc = rkh_h2d(ctx->stream, raw.as<>(), x.gate_up, (size_t)H * 2 * I);
-        if (!rc) rc = rkh_pack_w8(ctx->stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e);
-        if (!rc) rc = rkh_h2d(ctx->stream, raw.as<>(), x.down, (size_t)I * H);
-        if (!rc) rc = rkh_pack_w8(ctx->stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e);
-        if (!rc) rc = rkh_h2d(ctx->stream, w->gate_scales.as<float>() + (size_t)e * 2 * I, x.gate_up_scales, (size_t)2 * I * sizeof(float));
-        if (!rc) rc = rkh_h2d(ctx->stream, w->down_scales.as<float>() + (size_t)e * H, x.down_scales, (size_t)H * sizeof(float));
-        // the staging buffer is reused: finish this expert before the next copy lands
-        if (!rc) rc = rkh_sync(ctx->stream);
-        if (rc) return nullptr;
-    }
+    if (experts)
+        for (int e = 0; e < count; ++e)
+            if (pack_expert(w.get(), raw, e, experts[e])) return nullptr;
+    if (shared && pack_expert(w.get(), raw, config->routed_experts, *shared)) return nullptr;
+    if (rkh_sync(ctx->stream)) return nullptr;
     return w.release();
+}
+
+} // namespace
+
+extern "C" {
+
+rk_npu_moe_w8_weights* rk_npu_moe_w8_weights_create(rk_npu_iommu_domain* domain,
+                                                    const rk_npu_moe_w8_weight_config* config,
+                                                    const rk_npu_moe_w8_expert* experts) {
+    return experts ? create_weights(domain, config, experts, kW8, nullptr) : nullptr;
 }
 
 void rk_npu_moe_w8_weights_free(rk_npu_moe_w8_weights* weights) { delete weights; }
 
+} // extern "C"
+
+namespace {
+rk_npu_moe_w8_workspace* create_workspace(rk_npu_iommu_domain* domain, const rk_npu_moe_w8_config* config, int mode);
+}
+
+extern "C" {
+
 rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* domain,
                                                         const rk_npu_moe_w8_config* config) {
+    return create_workspace(domain, config, kW8);
+}
+
+} // extern "C"
+
+namespace {
+
+// reference src/rk_npu_moe_w8.cpp:892-896,910-914: the INT4 modes take fp32 or
+// pre-quantized rows in the normal (not NPU-native) layout only
+rk_npu_moe_w8_workspace* create_workspace(rk_npu_iommu_domain* domain, const rk_npu_moe_w8_config* config, int mode) {
     if (!domain || !domain->ctx || !config || !valid(*config)) return nullptr;
+    if (mode != kW8 && (!valid_w4(config->weights) || config->native_input)) return nullptr;
     std::unique_ptr<rk_npu_moe_w8_workspace> ws(new (std::nothrow) rk_npu_moe_w8_workspace());
     if (!ws) return nullptr;
     ws->owner.bind(domain);
     ws->config = *config;
+    ws->mode = mode;
     const auto& wc = config->weights;
     const int R = config->max_rows, H = wc.hidden, I = wc.intermediate, top = config->top_k;
     ws->slots = top + wc.shared_expert;
@@ -392,51 +465,177 @@ rk_npu_moe_w8_workspace* rk_npu_moe_w8_workspace_create(rk_npu_iommu_domain* dom
     return ws.release();
 }
 
+} // namespace
+
+extern "C" {
+
 void rk_npu_moe_w8_workspace_free(rk_npu_moe_w8_workspace* workspace) { delete workspace; }
 
-// ---- expert formats outside this build's path: exported, always declining ----
-// (reference src/rk_npu_moe_w8.cpp:885-999 implements them for the NPU's int4 mode)
-rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
-                                                       const rk_npu_moe_w8_expert*) {
-    errno = ENOTSUP;
-    return nullptr;
+// ---- INT4 experts, mixed banks, slot banks and packed expert records ----------
+// reference src/rk_npu_moe_w8.cpp:885-926
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create(rk_npu_iommu_domain* domain,
+                                                       const rk_npu_moe_w8_weight_config* config,
+                                                       const rk_npu_moe_w8_expert* experts) {
+    return experts ? create_weights(domain, config, experts, kW4, nullptr) : nullptr;
 }
-rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create_full_k(rk_npu_iommu_domain*,
-                                                              const rk_npu_moe_w8_weight_config*,
-                                                              const rk_npu_moe_w8_expert*) {
-    errno = ENOTSUP;
-    return nullptr;
+// The reference certifies a full-K gate/up tile here; accumulation is int32 in
+// this build, so both factories produce the same weights.
+rk_npu_moe_w8_weights* rk_npu_moe_quant_weights_create_full_k(rk_npu_iommu_domain* domain,
+                                                              const rk_npu_moe_w8_weight_config* config,
+                                                              const rk_npu_moe_w8_expert* experts) {
+    return rk_npu_moe_quant_weights_create(domain, config, experts);
 }
-rk_npu_moe_w8_workspace* rk_npu_moe_quant_workspace_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_config*) {
-    errno = ENOTSUP;
-    return nullptr;
+rk_npu_moe_w8_workspace* rk_npu_moe_quant_workspace_create(rk_npu_iommu_domain* domain,
+                                                           const rk_npu_moe_w8_config* config) {
+    return create_workspace(domain, config, kW4);
 }
-rk_npu_moe_w8_weights* rk_npu_moe_w4_weights_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
-                                                    const rk_npu_moe_w8_expert*) {
-    errno = ENOTSUP;
-    return nullptr;
+rk_npu_moe_w8_weights* rk_npu_moe_w4_weights_create(rk_npu_iommu_domain* domain,
+                                                    const rk_npu_moe_w8_weight_config* config,
+                                                    const rk_npu_moe_w8_expert* experts) {
+    return experts ? create_weights(domain, config, experts, kRoutedW4SharedW8, nullptr) : nullptr;
 }
-rk_npu_moe_w8_workspace* rk_npu_moe_w4_workspace_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_config*) {
-    errno = ENOTSUP;
-    return nullptr;
+rk_npu_moe_w8_workspace* rk_npu_moe_w4_workspace_create(rk_npu_iommu_domain* domain,
+                                                        const rk_npu_moe_w8_config* config) {
+    return create_workspace(domain, config, kRoutedW4SharedW8);
 }
-rk_npu_moe_w8_weights* rk_npu_moe_w4_slots_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*,
-                                                  const rk_npu_moe_w8_expert*) {
-    errno = ENOTSUP;
-    return nullptr;
+rk_npu_moe_w8_weights* rk_npu_moe_w4_slots_create(rk_npu_iommu_domain* domain,
+                                                  const rk_npu_moe_w8_weight_config* config,
+                                                  const rk_npu_moe_w8_expert* shared) {
+    if (!config || !shared || config->shared_expert != 1) return nullptr;
+    return create_weights(domain, config, nullptr, kRoutedW4SharedW8, shared);
 }
-rk_npu_moe_w8_weights* rk_npu_moe_quant_slots_create(rk_npu_iommu_domain*, const rk_npu_moe_w8_weight_config*) {
-    errno = ENOTSUP;
-    return nullptr;
+rk_npu_moe_w8_weights* rk_npu_moe_quant_slots_create(rk_npu_iommu_domain* domain,
+                                                     const rk_npu_moe_w8_weight_config* config) {
+    if (!config || config->shared_expert) return nullptr;
+    return create_weights(domain, config, nullptr, kW4, nullptr);
 }
-uint64_t rk_npu_moe_quant_expert_blob_bytes(const rk_npu_moe_w8_weights*) { return 0; }
-int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights*, int, void*, uint64_t) { return RK_NPU_ERR_PARAM; }
-int rk_npu_moe_quant_import_expert(rk_npu_moe_w8_weights*, int, const void*, uint64_t) { return RK_NPU_ERR_PARAM; }
-int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights*, int, const void*, uint64_t,
-                                         rk_npu_moe_import_timings*) {
-    return RK_NPU_ERR_PARAM;
+
+} // extern "C"
+
+namespace {
+
+// A packed expert record: header, then the expert's device images exactly as the
+// kernels read them (gate/up and down tiles, gate/up and down scales).  Records
+// are produced by rk_npu_moe_quant_export_expert of this library and are not
+// interchangeable with the reference's (its records hold NPU tile images).
+struct RecordHeader {
+    uint32_t magic, version, hidden, intermediate;
+};
+constexpr uint32_t kRecordMagic = 0x4d484b52u; // "RKHM"
+
+uint64_t record_bytes(const rk_npu_moe_w8_weights* w) {
+    return sizeof(RecordHeader) + w->gate_stride + w->down_stride +
+           ((uint64_t)2 * w->config.intermediate + w->config.hidden) * sizeof(float);
 }
-int rk_npu_moe_quant_swap_slots(rk_npu_moe_w8_weights*, int, rk_npu_moe_w8_weights*, int) { return RK_NPU_ERR_PARAM; }
+
+} // namespace
+
+extern "C" {
+
+// reference :927-929: 0 for handles without INT4 experts
+uint64_t rk_npu_moe_quant_expert_blob_bytes(const rk_npu_moe_w8_weights* w) {
+    return w && w->mode != kW8 ? record_bytes(w) : 0;
+}
+
+// reference :931-947
+int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights* w, int e, void* data, uint64_t bytes) {
+    const uint64_t need = rk_npu_moe_quant_expert_blob_bytes(w);
+    if (!need || !data || bytes < need || e < 0 || e >= w->count ||
+        !expert_is_w4(w->mode, e, w->config.routed_experts))
+        return RK_NPU_ERR_PARAM;
+    const int H = w->config.hidden, I = w->config.intermediate;
+    rk_npu_ctx* ctx = w->owner.ctx;
+    uint8_t* p = static_cast<uint8_t*>(data);
+    const RecordHeader header{kRecordMagic, RK_NPU_MOE_QUANT_BLOB_VERSION, (uint32_t)H, (uint32_t)I};
+    std::memcpy(p, &header, sizeof(header));
+    p += sizeof(header);
+    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
+    int rc = rkh_d2h(ctx->stream, p, w->gate_up.as<>() + w->gate_stride * e, w->gate_stride);
+    p += w->gate_stride;
+    if (!rc) rc = rkh_d2h(ctx->stream, p, w->down.as<>() + w->down_stride * e, w->down_stride);
+    p += w->down_stride;
+    if (!rc) rc = rkh_d2h(ctx->stream, p, w->gate_scales.as<float>() + (size_t)e * 2 * I, (size_t)2 * I * sizeof(float));
+    p += (size_t)2 * I * sizeof(float);
+    if (!rc) rc = rkh_d2h(ctx->stream, p, w->down_scales.as<float>() + (size_t)e * H, (size_t)H * sizeof(float));
+    const int wait = rkh_sync(ctx->stream);
+    return map_error(rc ? rc : wait);
+}
+
+int rk_npu_moe_quant_import_expert(rk_npu_moe_w8_weights* w, int slot, const void* data, uint64_t bytes) {
+    return rk_npu_moe_quant_import_expert_timed(w, slot, data, bytes, nullptr);
+}
+
+// reference :952-985.  The record is checked (header, scales) before anything is
+// written, so a rejected record leaves the slot as it was.
+int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights* w, int slot, const void* data, uint64_t bytes,
+                                         rk_npu_moe_import_timings* timings) {
+    const uint64_t need = rk_npu_moe_quant_expert_blob_bytes(w);
+    if (!need || !data || bytes < need || slot < 0 || slot >= w->count ||
+        !expert_is_w4(w->mode, slot, w->config.routed_experts))
+        return RK_NPU_ERR_PARAM;
+    if (timings) *timings = rk_npu_moe_import_timings{};
+    const auto begin = Clock::now();
+    const int H = w->config.hidden, I = w->config.intermediate;
+    const uint8_t* p = static_cast<const uint8_t*>(data);
+    RecordHeader header;
+    std::memcpy(&header, p, sizeof(header));
+    const uint8_t* gate = p + sizeof(header);
+    const uint8_t* down = gate + w->gate_stride;
+    const uint8_t* gate_scales = down + w->down_stride;
+    const uint8_t* down_scales = gate_scales + (size_t)2 * I * sizeof(float);
+    auto at = Clock::now();
+    bool ok = header.magic == kRecordMagic && header.version == RK_NPU_MOE_QUANT_BLOB_VERSION &&
+              header.hidden == (uint32_t)H && header.intermediate == (uint32_t)I;
+    if (ok) {
+        std::vector<float> scales((size_t)2 * I + H); // the record need not be aligned for float access
+        std::memcpy(scales.data(), gate_scales, scales.size() * sizeof(float));
+        ok = finite_positive(scales.data(), scales.size());
+    }
+    if (timings) timings->validate_us = elapsed_us(at);
+    if (!ok) return RK_NPU_ERR_PARAM;
+    rk_npu_ctx* ctx = w->owner.ctx;
+    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
+    at = Clock::now();
+    int rc = rkh_h2d(ctx->stream, w->gate_scales.as<float>() + (size_t)slot * 2 * I, gate_scales, (size_t)2 * I * sizeof(float));
+    if (!rc) rc = rkh_h2d(ctx->stream, w->down_scales.as<float>() + (size_t)slot * H, down_scales, (size_t)H * sizeof(float));
+    if (!rc) rc = rkh_sync(ctx->stream);
+    if (timings) timings->copy_us = elapsed_us(at);
+    at = Clock::now();
+    if (!rc) rc = rkh_h2d(ctx->stream, w->gate_up.as<>() + w->gate_stride * slot, gate, w->gate_stride);
+    if (!rc) rc = rkh_sync(ctx->stream);
+    if (timings) timings->gate_sync_us = elapsed_us(at);
+    at = Clock::now();
+    if (!rc) rc = rkh_h2d(ctx->stream, w->down.as<>() + w->down_stride * slot, down, w->down_stride);
+    if (!rc) rc = rkh_sync(ctx->stream);
+    if (timings) {
+        timings->down_sync_us = elapsed_us(at);
+        timings->total_us = elapsed_us(begin);
+    }
+    return map_error(rc);
+}
+
+// reference :987-998.  The reference exchanges buffer ownership; a bank here is
+// one allocation that the kernels index by slot, so the two slots' images are
+// exchanged in place by a kernel enqueued on the context's stream.  Nothing
+// waits on the host: runs, imports and exports of the same context are ordered
+// behind it on that stream.
+int rk_npu_moe_quant_swap_slots(rk_npu_moe_w8_weights* a, int ai, rk_npu_moe_w8_weights* b, int bi) {
+    if (!a || !b || a->mode != kW4 || b->mode != kW4 || a->config.hidden != b->config.hidden ||
+        a->config.intermediate != b->config.intermediate || !a->owner.same(b->owner) || ai < 0 || bi < 0 ||
+        ai >= a->count || bi >= b->count)
+        return RK_NPU_ERR_PARAM;
+    if (a == b && ai == bi) return RK_NPU_OK;
+    const size_t H = a->config.hidden, I = a->config.intermediate;
+    rk_npu_ctx* ctx = a->owner.ctx;
+    std::lock_guard<std::mutex> lock(ctx->submit_mutex);
+    int rc = rkh_exchange32(ctx->stream, a->gate_up.as<>() + a->gate_stride * ai, b->gate_up.as<>() + b->gate_stride * bi,
+                            a->gate_stride / 4);
+    if (!rc) rc = rkh_exchange32(ctx->stream, a->down.as<>() + a->down_stride * ai, b->down.as<>() + b->down_stride * bi,
+                                 a->down_stride / 4);
+    if (!rc) rc = rkh_exchange32(ctx->stream, a->gate_scales.as<float>() + ai * 2 * I, b->gate_scales.as<float>() + bi * 2 * I, 2 * I);
+    if (!rc) rc = rkh_exchange32(ctx->stream, a->down_scales.as<float>() + ai * H, b->down_scales.as<float>() + bi * H, H);
+    return map_error(rc);
+}
 
 uint64_t rk_npu_moe_w8_weights_device_bytes(const rk_npu_moe_w8_weights* w) {
     return w ? w->bytes() : 0;

@@ -286,16 +286,22 @@ def w4a8_ffn(sess, gu_ws, gu_w, dn_ws, dn_w, A, timings=None):
 
 
 class MoeW8:
-    def __init__(self, sess, H, I, E, shared, top_k, max_rows, experts):
+    """flavour: "w8" (int8 experts), "quant" (every expert INT4 codes) or "w4" (routed INT4, shared int8)."""
+    _CREATE = {"w8": ("rk_npu_moe_w8_weights_create", "rk_npu_moe_w8_workspace_create"),
+               "quant": ("rk_npu_moe_quant_weights_create", "rk_npu_moe_quant_workspace_create"),
+               "w4": ("rk_npu_moe_w4_weights_create", "rk_npu_moe_w4_workspace_create")}
+
+    def __init__(self, sess, H, I, E, shared, top_k, max_rows, experts, flavour="w8"):
         self.s, self.H, self.I, self.E, self.shared, self.top_k = sess, H, I, E, shared, top_k
+        self.flavour = flavour
         lib = sess.lib
         cfg = capi.MoeConfig()
         lib.rk_npu_moe_w8_config_init(C.byref(cfg), H, I, E, shared, top_k, max_rows)
         self.cfg = cfg
-        self.w = self.create_weights(experts)
-        self.ws = lib.rk_npu_moe_w8_workspace_create(sess.domain, C.byref(cfg))
+        self.w = self.create_weights(experts) if experts is not None else None
+        self.ws = getattr(lib, self._CREATE[flavour][1])(sess.domain, C.byref(cfg))
         if not self.ws:
-            raise RuntimeError("rk_npu_moe_w8_workspace_create failed")
+            raise RuntimeError("%s failed" % self._CREATE[flavour][1])
 
     def create_weights(self, experts, domain=None):
         keep = []
@@ -307,9 +313,10 @@ class MoeW8:
             ds = np.ascontiguousarray(ds, np.float32)
             keep += [g, gs, d, ds]
             arr[i] = capi.MoeExpert(g.ctypes.data, gs.ctypes.data, d.ctypes.data, ds.ctypes.data)
-        h = self.s.lib.rk_npu_moe_w8_weights_create(domain or self.s.domain, C.byref(self.cfg.weights), arr)
+        name = self._CREATE[self.flavour][0]
+        h = getattr(self.s.lib, name)(domain or self.s.domain, C.byref(self.cfg.weights), arr)
         if not h:
-            raise RuntimeError("rk_npu_moe_w8_weights_create failed")
+            raise RuntimeError("%s failed" % name)
         return h
 
     def run_f32(self, x, ids, routes, weights=None, timings=None, out=None):

@@ -73,6 +73,7 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
              ("rk_npu_w4a8_family_summary", capi.W4A8FamilySummary),
              ("rk_npu_moe_w8_weight_config", capi.MoeWeightConfig), ("rk_npu_moe_w8_config", capi.MoeConfig),
              ("rk_npu_moe_w8_expert", capi.MoeExpert), ("rk_npu_moe_w8_timings", capi.MoeTimings),
+             ("rk_npu_moe_import_timings", capi.MoeImportTimings),
              ("rk_npu_domain_memory_stats", capi.DomainMemoryStats)]
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rk_npu_hip.h"', '#include "rk_npu_w4a8_tune.h"',
              "int main(void) {"]
@@ -269,12 +270,12 @@ def test_autotune_entry_points_without_a_context(lib):
     assert not lib.rk_npu_f32i8f32_weights_create_from_f32_compress(None, C.byref(wc), capi.ptr(w), 4.0)
 
 
-def test_other_moe_expert_formats_decline(lib):
+def test_int4_moe_entry_points_without_a_device(lib):
     """W4 / mixed / slot-bank / packed-record entry points of the reference
-    (include/rk_npu_moe_w8.h:83-143) link and decline without touching buffers."""
-    cfg = capi.MoeWeightConfig(64, 32, 3, 1)
+    (include/rk_npu_moe_w8.h:83-143): refused without a domain or handle, buffers untouched."""
+    cfg = capi.MoeWeightConfig(64, 64, 3, 1)
     full = capi.MoeConfig()
-    lib.rk_npu_moe_w8_config_init(C.byref(full), 64, 32, 3, 1, 2, 8)
+    lib.rk_npu_moe_w8_config_init(C.byref(full), 64, 64, 3, 1, 2, 8)
     for fn in (lib.rk_npu_moe_quant_weights_create, lib.rk_npu_moe_quant_weights_create_full_k,
                lib.rk_npu_moe_w4_weights_create, lib.rk_npu_moe_w4_slots_create):
         assert not fn(None, C.byref(cfg), None)
