@@ -380,24 +380,31 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
     }
 }
 
-// Dense quantization of many rows: one workgroup per 8 consecutive rows, so
-// that every store instruction writes whole 128-byte lines of the tiled int8
-// matrix (for a fixed 16-element chunk, 8 consecutive rows are 8 consecutive
-// 16-byte slots of a tile).  Lane = (row r = lane % 8, chunk column lane / 8 +
-// 8 * wave): a row's loads are 8 consecutive chunks per wave instruction.  Rows
-// of up to 32 * Q8_CACHE chunks are held in registers between the maximum and
-// the quantization (all loads of a thread in flight at once); longer rows are
-// read twice, the second time from L2.
+// Dense quantization of many rows: one workgroup per ROWS (8 or 4) consecutive
+// rows.  For a fixed 16-element chunk, consecutive rows are consecutive 16-byte
+// slots of a tile of the int8 matrix, so with 8 rows every store instruction
+// writes whole 128-byte lines (64-byte halves with 4).  Lane = (row r = lane %
+// ROWS, chunk column lane / ROWS + (64 / ROWS) * wave): a row's loads are 64 /
+// ROWS consecutive chunks per wave instruction.  Rows of up to (256 / ROWS) *
+// Q8_CACHE chunks are held in registers between the maximum and the
+// quantization (all loads of a thread in flight at once); longer rows are read
+// twice, the second time from L2.  The kernel is one load phase, one reduction
+// and one store phase, so a compute unit only overlaps loads with stores when
+// it holds several workgroups: 4 rows are used while 8 would leave fewer than
+// two workgroups per compute unit.
 // Modes: dynamic W8 / W4A8 maxima or a given static scale; rows written in place.
 constexpr int Q8_CACHE = 8;
 
-template <typename T>
+template <typename T, int ROWS>
 __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
-    __shared__ float part_max[4][8];
+    static_assert(ROWS == 8 || ROWS == 4, "rows per workgroup");
+    constexpr int CPW = 64 / ROWS;    // chunk columns per wave instruction
+    constexpr int CSTEP = 4 * CPW;    // chunk columns per workgroup pass
+    __shared__ float part_max[4][ROWS];
     __shared__ int part_bad[4];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int r = lane & 7, cl = (lane >> 3) + 8 * wave;
-    const int m = blockIdx.x * 8 + r;
+    const int r = lane % ROWS, cl = lane / ROWS + CPW * wave;
+    const int m = blockIdx.x * ROWS + r;
     const bool live = m < a.M;
     const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
     const int nchunks = (K + 15) >> 4;
@@ -406,7 +413,7 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
     const int mode = a.mode;
     const bool need_max = mode != RKH_Q_W8_STATIC;
     const bool check = mode == RKH_Q_W4A8;
-    const bool cached = nchunks <= 32 * Q8_CACHE;
+    const bool cached = nchunks <= CSTEP * Q8_CACHE;
 
     float v[Q8_CACHE][16];
     float mx = 0.0f;
@@ -414,13 +421,13 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
     if (cached) {
 #pragma unroll
         for (int i = 0; i < Q8_CACHE; ++i) {
-            const int c = cl + 32 * i;
+            const int c = cl + CSTEP * i;
             if (c < nchunks) RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
         }
         if (need_max) {
 #pragma unroll
             for (int i = 0; i < Q8_CACHE; ++i) {
-                if (cl + 32 * i < nchunks) {
+                if (cl + CSTEP * i < nchunks) {
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
                         mx = fmaxf(mx, fabsf(v[i][j]));
@@ -430,7 +437,7 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
             }
         }
     } else if (need_max) {
-        for (int c = cl; c < nchunks; c += 32) {
+        for (int c = cl; c < nchunks; c += CSTEP) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
 #pragma unroll
@@ -443,16 +450,16 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
     float scale = 1.0f;
     if (need_max) {
 #pragma unroll
-        for (int off = 8; off < 64; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        for (int off = ROWS; off < 64; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
         const unsigned long long bad_mask = __ballot(bad && check && live);
-        if (lane < 8) part_max[wave][lane] = mx;
+        if (lane < ROWS) part_max[wave][lane] = mx;
         if (lane == 0) part_bad[wave] = bad_mask != 0ull;
         __syncthreads();
         mx = fmaxf(fmaxf(part_max[0][r], part_max[1][r]), fmaxf(part_max[2][r], part_max[3][r]));
         if (t == 0 && a.bad_flag && (part_bad[0] | part_bad[1] | part_bad[2] | part_bad[3])) atomicOr(a.bad_flag, 1);
         if (mode == RKH_Q_W4A8) scale = mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN);
         else scale = mx > 0.0f ? mx / 127.0f : 1.0f;
-        if (t < 8 && live && a.scale) a.scale[m] = scale;
+        if (t < ROWS && live && a.scale) a.scale[m] = scale;
     } else {
         scale = a.scale[live ? m : a.M - 1];
     }
@@ -461,12 +468,12 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
     if (cached) {
 #pragma unroll
         for (int i = 0; i < Q8_CACHE; ++i) {
-            const int c = cl + 32 * i;
+            const int c = cl + CSTEP * i;
             if (c < nchunks)
                 *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(v[i], inv);
         }
     } else {
-        for (int c = cl; c < nchunks; c += 32) {
+        for (int c = cl; c < nchunks; c += CSTEP) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
             *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(tmp, inv);
@@ -1901,11 +1908,16 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     const int mode = args->mode;
     if (args->M >= 256 && !args->dest_rows && !args->active_blocks && args->in_dtype != RKH_I8 &&
         (mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_W8_STATIC)) {
-        const dim3 grid8((args->M + 7) / 8);
-        if (args->in_dtype == RKH_F16)
-            hipLaunchKernelGGL(quant_rows8_kernel<uint16_t>, grid8, block, 0, (hipStream_t)stream, *args);
-        else
-            hipLaunchKernelGGL(quant_rows8_kernel<float>, grid8, block, 0, (hipStream_t)stream, *args);
+        const bool rows4 = args->M < 8 * 2 * 256; // 8 rows would give fewer than two workgroups per compute unit
+        const dim3 grid(rows4 ? (args->M + 3) / 4 : (args->M + 7) / 8);
+        const hipStream_t st = (hipStream_t)stream;
+        if (args->in_dtype == RKH_F16) {
+            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 4>), grid, block, 0, st, *args);
+            else hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 8>), grid, block, 0, st, *args);
+        } else {
+            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<float, 4>), grid, block, 0, st, *args);
+            else hipLaunchKernelGGL((quant_rows8_kernel<float, 8>), grid, block, 0, st, *args);
+        }
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
