@@ -105,7 +105,6 @@ enum rkh_quant_mode {
     RKH_Q_W8_DYNAMIC = 0, /* s = max>0 ? max/127 : 1 ; ties away ; no finite check     */
     RKH_Q_W8_STATIC = 1,  /* s given in scale[] ; ties away                             */
     RKH_Q_W4A8 = 2,       /* s = max==0 ? 1 : max(max/127, FLT_MIN) ; ties away ; check */
-    RKH_Q_MOE = 3,        /* s = max ? max/127 : 1 ; ties even ; check                  */
     RKH_Q_COPY_I8 = 4,    /* input already int8: re-tile only (scale[] passes through)  */
     RKH_Q_REUSE_BITS = 5, /* s from row_max_bits[] (W4A8 rule) ; ties away              */
     RKH_Q_REUSE_BITS_MOE = 6 /* s from row_max_bits[] (MoE rule) ; ties even            */
@@ -122,12 +121,6 @@ typedef struct rkh_quant_args {
     int* bad_flag;       /* OR 1: non-finite input (modes with a check), may be NULL */
     const uint32_t* row_max_bits; /* REUSE modes: [M][row_max_parts] partial maxima of |x| bits */
     int row_max_parts;
-    /* MoE scatter: when dest_rows != NULL, source row m is written to every
-     * tiled row dest_rows[m * dest_stride + j] >= 0, j < dest_stride, and
-     * scale_rows[dest row] receives the row's scale. */
-    const int* dest_rows;
-    int dest_stride;
-    float* scale_rows;
     /* If non-NULL, rows at or beyond active_blocks[0] * 32 are skipped. */
     const int* active_blocks;
 } rkh_quant_args;
@@ -174,7 +167,12 @@ int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_arg
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4);
 
 /* ---- MoE routing and combine ---- */
-typedef struct rkh_moe_route_args {
+/* Routing + token scatter in one launch: assignments with a non-zero
+ * coefficient are bucketed by expert, stably, each bucket padded to 32 sorted
+ * rows (the shared expert, id == experts, takes every token); each token is
+ * quantized per row (s = max ? max/127 : 1, ties even, non-finite -> bad_flag)
+ * or, for int8 input, copied, into the sorted rows of its assignments. */
+typedef struct rkh_moe_scatter_args {
     const int32_t* ids;    /* [rows, top_k] device                                 */
     const float* routes;   /* [rows, top_k] device                                 */
     int rows, top_k, experts, shared; /* experts = routed count                    */
@@ -182,8 +180,15 @@ typedef struct rkh_moe_route_args {
     int* blk_expert;       /* [max_blocks] out                                     */
     int* num_blocks;       /* [2] out: {row blocks, assignments}                   */
     int max_blocks;
-} rkh_moe_route_args;
-int rkh_moe_route(void* stream, const rkh_moe_route_args* args);
+    const void* src;       /* [rows, K] tokens: RKH_F32, or RKH_I8 codes           */
+    int in_dtype;
+    int K;
+    float* token_scale;    /* [rows]: out for fp32 tokens, in for int8 codes       */
+    uint8_t* dst;          /* tiled int8 sorted rows                               */
+    float* scale_rows;     /* [sorted rows] out: scale of the token in that row    */
+    int* bad_flag;         /* OR 1 on a non-finite fp32 token, may be NULL         */
+} rkh_moe_scatter_args;
+int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args);
 
 typedef struct rkh_moe_combine_args {
     const float* Y;        /* [sorted rows, H] fp32 expert outputs                 */

@@ -229,16 +229,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
     const int mode = a.mode;
     if constexpr (sizeof(T) == 1) {
         // int8 input is re-tiled byte for byte (the full range -128..127 is legal
-        // for the raw integer operator); scale[] passes through for the MoE path.
-        const int nd = a.dest_rows ? a.dest_stride : 1;
-        if (t == 0 && a.dest_rows) {
-            for (int j = 0; j < nd; ++j) {
-                const int d = a.dest_rows[(size_t)m * nd + j];
-                if (d >= 0) {
-                    if (a.scale_rows && a.scale) a.scale_rows[d] = a.scale[m];
-                }
-            }
-        }
+        // for the raw integer operator)
         const int8_t* brow = reinterpret_cast<const int8_t*>(row);
         for (int c = chunk0 + t; c < nchunks; c += 256) {
             uint32_t w[4] = {0, 0, 0, 0};
@@ -249,20 +240,12 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
                 for (int j = 0; j < 16; ++j)
                     if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
             }
-            const uint4 packed = make_uint4(w[0], w[1], w[2], w[3]);
-            if (!a.dest_rows) {
-                *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
-            } else {
-                for (int j = 0; j < nd; ++j) {
-                    const int d = a.dest_rows[(size_t)m * nd + j];
-                    if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
-                }
-            }
+            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = make_uint4(w[0], w[1], w[2], w[3]);
         }
         return;
     }
-    const bool need_max = mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
-    const bool check = mode == RKH_Q_W4A8 || mode == RKH_Q_MOE;
+    const bool need_max = mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8;
+    const bool check = mode == RKH_Q_W4A8;
 
     float v[QR_CACHE][16];
     float mx = 0.0f;
@@ -336,34 +319,13 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
         }
     }
     const float inv = mode == RKH_Q_COPY_I8 ? 1.0f : 1.0f / scale;
-    const bool even = mode == RKH_Q_MOE || mode == RKH_Q_REUSE_BITS_MOE;
+    const bool even = mode == RKH_Q_REUSE_BITS_MOE;
 
-    int ndest = 1;
-    if (a.dest_rows) ndest = a.dest_stride;
-    if (t == 0 && part == 0) {
-        if (!a.dest_rows) {
-            if (a.scale && mode != RKH_Q_W8_STATIC && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
-        } else {
-            if (a.scale && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
-            for (int j = 0; j < ndest; ++j) {
-                const int d = a.dest_rows[(size_t)m * ndest + j];
-                if (d >= 0) {
-                    a.scale_rows[d] = scale;
-                }
-            }
-        }
-    }
+    if (t == 0 && part == 0 && a.scale && mode != RKH_Q_W8_STATIC && mode != RKH_Q_COPY_I8) a.scale[m] = scale;
 
     auto emit = [&](int c, const float* vals) {
         const uint4 packed = even ? quantize16<true>(vals, inv) : quantize16<false>(vals, inv);
-        if (!a.dest_rows) {
-            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
-        } else {
-            for (int j = 0; j < ndest; ++j) {
-                const int d = a.dest_rows[(size_t)m * ndest + j];
-                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
-            }
-        }
+        *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
     };
     if (cached) {
 #pragma unroll
@@ -1491,142 +1453,238 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     }
 }
 
-// ------------------------------------------------------------- MoE route
-// Single workgroup.  Assignments (row-major over [rows, top_k]) with a non-zero
-// coefficient are bucketed by expert id, stably, each bucket padded to a
-// multiple of 32 rows; the shared expert (id == experts) gets every row.
+// ---------------------------------------------------- MoE route + scatter
+// One workgroup per token.  Live assignments (row-major over [rows, top_k], non-
+// zero coefficient) are bucketed by expert id, stably, each bucket padded to a
+// multiple of 32 sorted rows; the shared expert (id == experts) gets every row.
+// Instead of a routing pass of its own, every workgroup derives the sorted rows
+// of its token's assignments from the whole table (a few KiB, served by L2)
+// while its token row is on its way from memory:
+//   sorted row of assignment i with expert e  =  start[e] + #{live i' < i with expert e},
+//   start[e] = sum over e' < e of pad32(count[e']),
+// then quantizes the token (or copies pre-quantized codes) into each of those
+// rows.  Workgroup 0 also writes the row-block -> expert table and the totals.
+// Counting uses wave ballots: each wave owns a contiguous range of assignments;
+// lanes with equal keys find each other bit by bit of the key, one lane per
+// distinct key adds the group's size to its wave's bins, and the lane that
+// holds one of the token's own assignments notes how many equal keys came
+// before it.  (LDS atomics on a few dozen hot counters serialize and took three
+// times as long.)  The loop is kept rolled: each workgroup runs it once, from a
+// cold instruction cache, so straight-line code costs more than it saves.
 constexpr int ROUTE_MAX_EXPERTS = 2048;
-constexpr int ROUTE_WAVES = 4;
+constexpr int ROUTE_MAX_TOPK = 8;
+constexpr int ROUTE_MAX_ASSIGNMENTS = 2048; // rows * top_k
 
-__global__ __launch_bounds__(ROUTE_WAVES * 64) void moe_route_kernel(rkh_moe_route_args a) {
-    __shared__ int bins[ROUTE_WAVES][ROUTE_MAX_EXPERTS];
-    __shared__ int start[ROUTE_MAX_EXPERTS + 1];
-    __shared__ int wave_total[ROUTE_WAVES];
-    __shared__ int live_total;
-    const int t = threadIdx.x, lane = lane_id(), wave = wave_id();
-    const int E = a.experts, Etot = E + a.shared;
-    const int slots = a.top_k + a.shared;
-    const int n = a.rows * a.top_k;
-    for (int i = t; i < ROUTE_WAVES * Etot; i += ROUTE_WAVES * 64) bins[i / Etot][i % Etot] = 0;
-    if (t == 0) live_total = 0;
+template <typename T>
+__global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a) {
+    __shared__ int bins[4][ROUTE_MAX_EXPERTS];   // live assignments per expert, per wave
+    __shared__ int start[ROUTE_MAX_EXPERTS + 1]; // first sorted row of each bucket
+    __shared__ int own_key[ROUTE_MAX_TOPK], own_rank[ROUTE_MAX_TOPK], own_wave[ROUTE_MAX_TOPK];
+    __shared__ int dest[ROUTE_MAX_TOPK + 1];
+    __shared__ int wave_total[4];
+    __shared__ int wave_live[4];
+    __shared__ float wave_max[4];
+    __shared__ int wave_bad[4];
+    const int m = blockIdx.x, t = threadIdx.x, lane = lane_id(), wave = wave_id();
+    const int E = a.experts, top_k = a.top_k, slots = top_k + a.shared, n = a.rows * top_k;
+    const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
+    const int nchunks = (K + 15) >> 4;
+    const T* row = static_cast<const T*>(a.src) + (size_t)m * K;
+    const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    const bool cached = nchunks <= 256 * QR_CACHE;
 
-    const int chunks_total = (n + 63) / 64;
-    const int chunks_per_wave = (chunks_total + ROUTE_WAVES - 1) / ROUTE_WAVES;
-    const int first = wave * chunks_per_wave * 64;
-    // keys of this lane's assignments stay in registers between the counting and
-    // the placement pass (up to ROUTE_CACHE chunks per wave; re-read beyond)
-    constexpr int ROUTE_CACHE = 8;
-    int cached[ROUTE_CACHE];
-    auto key_of = [&](int c) {
-        const int i = first + c * 64 + lane;
-        return (i < n && a.routes[i] != 0.0f) ? a.ids[i] : -1;
-    };
+    // Loads: this wave's share of the routing table first, then the token's row
+    // -- loads return in issue order, so the routing can start while the row is
+    // still on its way.  Wave w owns assignments [w, w + 1) * per_wave * 64.
+    constexpr int PER_WAVE = ROUTE_MAX_ASSIGNMENTS / 256; // 64-assignment groups per wave
+    const int per_wave = ((n + 63) / 64 + 3) / 4;
+    const int wave_first = wave * per_wave * 64;
+    int keys[PER_WAVE]; // expert of a live assignment, -1 if dropped or beyond the table
 #pragma unroll
-    for (int c = 0; c < ROUTE_CACHE; ++c) cached[c] = c < chunks_per_wave ? key_of(c) : -1;
-
-    auto same_key_mask = [&](int key) -> unsigned long long {
-        unsigned long long mask = __ballot(key >= 0);
-        for (int b = 0; b < 11; ++b) {
-            const unsigned long long set = __ballot((key >> b) & 1);
-            mask &= ((key >> b) & 1) ? set : ~set;
+    for (int c = 0; c < PER_WAVE; ++c) {
+        const int i = wave_first + c * 64 + lane;
+        keys[c] = -1;
+        if (c < per_wave && i < n) {
+            const int id = a.ids[i];
+            keys[c] = (a.routes[i] != 0.0f && (unsigned)id < (unsigned)E) ? id : -1;
         }
-        return key >= 0 ? mask : 0ull;
-    };
-    __syncthreads();
-
-    int assigned = 0;
-    for (int c = 0; c < chunks_per_wave; ++c) {
-        int key = -1;
-        if (c < ROUTE_CACHE) {
-#pragma unroll
-            for (int u = 0; u < ROUTE_CACHE; ++u)
-                if (u == c) key = cached[u];
-        } else {
-            key = key_of(c);
-        }
-        const unsigned long long mask = same_key_mask(key);
-        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull) bins[wave][key] += __popcll(mask);
-        assigned += key >= 0;
-        __builtin_amdgcn_wave_barrier();
     }
-    __syncthreads();
+    float v[QR_CACHE][16];
+    if constexpr (sizeof(T) == 4) {
+        if (cached) {
+#pragma unroll
+            for (int i = 0; i < QR_CACHE; ++i) {
+                const int c = t + i * 256;
+                if (c < nchunks) RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
+            }
+        }
+    }
 
+    // ---- routing
+    for (int e = lane; e < E; e += 64) bins[wave][e] = 0;
+    __builtin_amdgcn_wave_barrier(); // a wave only touches its own bins until the workgroup barrier below
+    int key_bits = 1;
+    while ((1 << key_bits) < E) ++key_bits;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int own0 = m * top_k;
+    int live = 0;
+#pragma unroll 1
+    for (int c = 0; c < per_wave; ++c) {
+        const int key = keys[0];
+#pragma unroll
+        for (int u = 0; u + 1 < PER_WAVE; ++u) keys[u] = keys[u + 1];
+        unsigned long long same = __ballot(key >= 0);
+        live += __popcll(same);
+#pragma unroll 1
+        for (int bit = 0; bit < key_bits; ++bit) {
+            const unsigned long long set = __ballot((key >> bit) & 1);
+            same &= ((key >> bit) & 1) ? set : ~set;
+        }
+        const int earlier = __popcll(same & below); // equal keys in lower lanes
+        int seen = 0;                                // equal keys in this wave's earlier groups
+        if (key >= 0) seen = bins[wave][key];
+        __builtin_amdgcn_wave_barrier();
+        if (key >= 0 && earlier == 0) bins[wave][key] = seen + __popcll(same);
+        const int k = wave_first + c * 64 + lane - own0;
+        if (k >= 0 && k < top_k) {
+            own_key[k] = key;
+            own_rank[k] = seen + earlier;
+            own_wave[k] = wave;
+        }
+    }
+    if (lane == 0) wave_live[wave] = live;
+    __syncthreads();
     // bucket sizes -> padded exclusive scan: 8 experts per thread, a shuffle scan
-    // inside each wave, the four wave totals through LDS
-    constexpr int PER = ROUTE_MAX_EXPERTS / (ROUTE_WAVES * 64);
+    // inside each wave, the wave totals through LDS
+    constexpr int PER = ROUTE_MAX_EXPERTS / 256;
+    const int Etot = E + a.shared;
     int sizes[PER];
     int local = 0;
+#pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int e = t * PER + j;
         int cnt = 0;
-        if (e < E) {
-            for (int w = 0; w < ROUTE_WAVES; ++w) cnt += bins[w][e];
-        } else if (e == E && a.shared) {
-            cnt = a.rows;
-        }
+        if (e < E) cnt = bins[0][e] + bins[1][e] + bins[2][e] + bins[3][e];
+        else if (e == E && a.shared) cnt = a.rows;
         sizes[j] = (cnt + 31) & ~31;
         local += sizes[j];
     }
     int incl = local;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
-        const int v = __shfl_up(incl, off);
-        if (lane >= off) incl += v;
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
     }
     if (lane == 63) wave_total[wave] = incl;
-    // live assignments (for the all-routes-dropped check)
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) assigned += __shfl_xor(assigned, off);
-    if (lane == 0) atomicAdd(&live_total, assigned);
     __syncthreads();
     int run = incl - local;
     for (int w = 0; w < wave; ++w) run += wave_total[w];
+#pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int e = t * PER + j;
         if (e <= Etot) start[e] = run;
-        if (e < Etot) {
-            for (int b = 0; b < sizes[j] / 32; ++b) {
-                const int blk = run / 32 + b;
+        if (m == 0 && e < Etot)
+            for (int blk = run / 32; blk < (run + sizes[j]) / 32; ++blk)
                 if (blk < a.max_blocks) a.blk_expert[blk] = e;
-            }
-        }
         run += sizes[j];
     }
-    if (t == ROUTE_WAVES * 64 - 1) {
+    if (m == 0 && t == 255) {
         a.num_blocks[0] = min(run / 32, a.max_blocks);
-        a.num_blocks[1] = live_total + (a.shared ? a.rows : 0);
+        a.num_blocks[1] = wave_live[0] + wave_live[1] + wave_live[2] + wave_live[3] + (a.shared ? a.rows : 0);
     }
     __syncthreads();
-    // per-wave running offsets
-    for (int e = t; e < E; e += ROUTE_WAVES * 64) {
-        int base = start[e];
-        for (int w = 0; w < ROUTE_WAVES; ++w) {
-            const int cnt = bins[w][e];
-            bins[w][e] = base;
-            base += cnt;
+    if (t < top_k) {
+        const int key = own_key[t];
+        int d = -1;
+        if (key >= 0) {
+            d = start[key] + own_rank[t];
+            for (int w = 0; w < own_wave[t]; ++w) d += bins[w][key];
         }
+        dest[t] = d;
+        a.dest_rows[(size_t)m * slots + t] = d;
+    } else if (t == top_k && a.shared) {
+        const int d = start[E] + m;
+        dest[t] = d;
+        a.dest_rows[(size_t)m * slots + t] = d;
     }
-    __syncthreads();
-    for (int c = 0; c < chunks_per_wave; ++c) {
-        const int i = first + c * 64 + lane;
-        int key = -1;
-        if (c < ROUTE_CACHE) {
+
+    // ---- the token into its sorted rows
+    if constexpr (sizeof(T) == 1) {
+        __syncthreads(); // dest[]
+        if (t < slots && dest[t] >= 0) a.scale_rows[dest[t]] = a.token_scale[m];
+        const int8_t* brow = reinterpret_cast<const int8_t*>(row);
+        for (int c = t; c < nchunks; c += 256) {
+            uint32_t w[4] = {0, 0, 0, 0};
+            if (vec && c * 16 + 16 <= K) {
+                const uint4 v4 = *reinterpret_cast<const uint4*>(brow + c * 16);
+                w[0] = v4.x; w[1] = v4.y; w[2] = v4.z; w[3] = v4.w;
+            } else {
+                for (int j = 0; j < 16; ++j)
+                    if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
+            }
+            const uint4 packed = make_uint4(w[0], w[1], w[2], w[3]);
+            for (int j = 0; j < slots; ++j) {
+                const int d = dest[j];
+                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+            }
+        }
+    } else {
+        float mx = 0.0f;
+        bool bad = false;
+        if (cached) {
 #pragma unroll
-            for (int u = 0; u < ROUTE_CACHE; ++u)
-                if (u == c) key = cached[u];
+            for (int i = 0; i < QR_CACHE; ++i)
+                if (t + i * 256 < nchunks) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        mx = fmaxf(mx, fabsf(v[i][j]));
+                        bad |= not_finite(v[i][j]);
+                    }
+                }
         } else {
-            key = key_of(c);
+            for (int c = t; c < nchunks; c += 256) {
+                float tmp[16];
+                RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    mx = fmaxf(mx, fabsf(tmp[j]));
+                    bad |= not_finite(tmp[j]);
+                }
+            }
         }
-        const unsigned long long mask = same_key_mask(key);
-        int dest = -1;
-        if (key >= 0) dest = bins[wave][key] + __popcll(mask & ((1ull << lane) - 1ull));
-        __builtin_amdgcn_wave_barrier();
-        if (key >= 0 && (mask & ((1ull << lane) - 1ull)) == 0ull) bins[wave][key] += __popcll(mask);
-        __builtin_amdgcn_wave_barrier();
-        if (i < n) a.dest_rows[(size_t)(i / a.top_k) * slots + (i % a.top_k)] = dest;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        const unsigned long long bad_mask = __ballot(bad);
+        if (lane == 0) {
+            wave_max[wave] = mx;
+            wave_bad[wave] = bad_mask != 0ull;
+        }
+        __syncthreads(); // also dest[]
+        mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+        if ((wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3]) && t == 0 && a.bad_flag) atomicOr(a.bad_flag, 1);
+        const float scale = mx > 0.0f ? mx / 127.0f : 1.0f;
+        const float inv = 1.0f / scale;
+        if (t == 0) a.token_scale[m] = scale;
+        if (t < slots && dest[t] >= 0) a.scale_rows[dest[t]] = scale;
+        auto emit = [&](int c, const float* vals) {
+            const uint4 packed = quantize16<true>(vals, inv);
+            for (int j = 0; j < slots; ++j) {
+                const int d = dest[j];
+                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+            }
+        };
+        if (cached) {
+#pragma unroll
+            for (int i = 0; i < QR_CACHE; ++i)
+                if (t + i * 256 < nchunks) emit(t + i * 256, v[i]);
+        } else {
+            for (int c = t; c < nchunks; c += 256) {
+                float tmp[16];
+                RowLoader<T>::load16(row, c * 16, K, vec, tmp);
+                emit(c, tmp);
+            }
+        }
     }
-    if (a.shared)
-        for (int r = t; r < a.rows; r += ROUTE_WAVES * 64) a.dest_rows[(size_t)r * slots + a.top_k] = start[E] + r;
 }
 
 // out[t, n] = sum over slots, in slot order, of fma(Y[dest, n], w, out); the
@@ -1749,7 +1807,7 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 // The decode path can quantize inside the GEMV when the rows fit the kernel's
 // LDS staging and per-thread register cache.
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g) {
-    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU || q.dest_rows) return false;
+    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU) return false;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
     const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
@@ -1906,7 +1964,7 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     if (args->M <= 0) return RKH_OK;
     const dim3 block(256);
     const int mode = args->mode;
-    if (args->M >= 256 && !args->dest_rows && !args->active_blocks && args->in_dtype != RKH_I8 &&
+    if (args->M >= 256 && !args->active_blocks && args->in_dtype != RKH_I8 &&
         (mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_W8_STATIC)) {
         const bool rows4 = args->M < 8 * 2 * 256; // 8 rows would give fewer than two workgroups per compute unit
         const dim3 grid(rows4 ? (args->M + 3) / 4 : (args->M + 7) / 8);
@@ -1924,7 +1982,7 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     // Re-quantization of a few long rows: several workgroups per row, about 256 chunks
     // each, until the grid has a few hundred workgroups.
     int split = 1;
-    if ((mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) && !args->dest_rows) {
+    if (mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) {
         const int row_chunks = (args->K + 15) / 16;
         while (split < 8 && args->M * split < 512 && row_chunks / (split * 2) >= 128) split *= 2;
     }
@@ -2007,9 +2065,18 @@ int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_arg
     return rc ? rc : rkh_gemm(stream, gargs);
 }
 
-int rkh_moe_route(void* stream, const rkh_moe_route_args* args) {
-    if (args->experts + args->shared > ROUTE_MAX_EXPERTS) return RKH_ERR_RUNTIME;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(ROUTE_WAVES * 64), 0, (hipStream_t)stream, *args);
+int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args) {
+    if (args->rows <= 0) return RKH_OK;
+    if (args->experts + args->shared > ROUTE_MAX_EXPERTS || args->top_k > ROUTE_MAX_TOPK ||
+        (long)args->rows * args->top_k > ROUTE_MAX_ASSIGNMENTS)
+        return RKH_ERR_RUNTIME;
+    const dim3 grid(args->rows), block(256);
+    if (args->in_dtype == RKH_F32)
+        hipLaunchKernelGGL(moe_scatter_kernel<float>, grid, block, 0, (hipStream_t)stream, *args);
+    else if (args->in_dtype == RKH_I8)
+        hipLaunchKernelGGL(moe_scatter_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args);
+    else
+        return RKH_ERR_RUNTIME;
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }

@@ -129,7 +129,7 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     void* stream = ws->owner.ctx->stream;
     auto mark = [&] { if (timer) timer->mark(); };
 
-    rkh_moe_route_args r{};
+    rkh_moe_scatter_args r{};
     r.ids = d_ids;
     r.routes = d_routes;
     r.rows = rows;
@@ -140,23 +140,15 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     r.blk_expert = ws->blk_expert.as<int>();
     r.num_blocks = ws->num_blocks.as<int>();
     r.max_blocks = ws->max_blocks;
-    int rc = rkh_moe_route(stream, &r);
-    if (rc) return map_error(rc);
-    mark(); // 1: schedule
-
-    rkh_quant_args q{};
-    q.src = d_input;
-    q.in_dtype = f32 ? RKH_F32 : RKH_I8;
-    q.mode = f32 ? RKH_Q_MOE : RKH_Q_COPY_I8;
-    q.M = rows;
-    q.K = H;
-    q.scale = f32 ? ws->token_scale.as<float>() : const_cast<float*>(d_scales);
-    q.dst = ws->a_tiled.as<>();
-    q.bad_flag = ws->flag.device();
-    q.dest_rows = ws->dest_rows.as<int>();
-    q.dest_stride = ws->slots;
-    q.scale_rows = ws->a_scale.as<float>();
-    rc = rkh_quant_rows(stream, &q);
+    r.src = d_input;
+    r.in_dtype = f32 ? RKH_F32 : RKH_I8;
+    r.K = H;
+    r.token_scale = f32 ? ws->token_scale.as<float>() : const_cast<float*>(d_scales);
+    r.dst = ws->a_tiled.as<>();
+    r.scale_rows = ws->a_scale.as<float>();
+    r.bad_flag = ws->flag.device();
+    mark(); // 1: schedule (routing is part of the scatter launch)
+    int rc = rkh_moe_scatter(stream, &r);
     if (rc) return map_error(rc);
     mark(); // 2: input
 
