@@ -185,24 +185,46 @@ __device__ __forceinline__ size_t tiled_chunk_offset(int row, int c, int KB) {
     return ((size_t)(row >> 5) * KB + kb) * 1024 + (size_t)((row & 31) + 32 * half) * 16;
 }
 
+// 16 quantized codes into the tiled matrix.  A plain store on purpose: the next
+// kernel reads these tiles, and with streaming (non-temporal) stores it found
+// them in HBM instead of the memory-side cache -- the quantization got 1 us
+// shorter and the GEMM behind it 1.5 us longer.
+__device__ __forceinline__ void store_codes(uint8_t* dst, uint4 codes) {
+    *reinterpret_cast<uint4*>(dst) = codes;
+}
+
+// int8 code of v * inv as the low byte of the result.
+//   EVEN:  rint(clamp(q, -127, 127))            (ties to even)
+//   else:  clamp(roundf(q), -127, 127)          (ties away from zero; NaN -> 127, as the chain of
+//          comparisons in the reference gives).  v_cvt_rpi_i32_f32 is floor(x + 0.5) computed
+//          exactly, i.e. round-half-away on |q|; checked against roundf over all 2^32 bit patterns.
+template <bool EVEN>
+__device__ __forceinline__ int quantize_code(float v, float inv) {
+    const float q = v * inv;
+    if (EVEN) {
+        return (int)rintf(fmaxf(fminf(q, 127.0f), -127.0f));
+    } else {
+        const float a = fminf(fabsf(q), 127.0f); // NaN -> 127
+        int r;
+        asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(r) : "v"(a));
+        return q < 0.0f ? -r : r;
+    }
+}
+
+// The low bytes of four dwords as one dword (c0 lowest).
+__device__ __forceinline__ uint32_t pack_low_bytes(int c0, int c1, int c2, int c3) {
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)c1, (uint32_t)c0, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)c3, (uint32_t)c2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 template <bool EVEN>
 __device__ __forceinline__ uint4 quantize16(const float* v, float inv) {
-    uint32_t w[4] = {0, 0, 0, 0};
+    uint32_t w[4];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        float q = v[j] * inv;
-        if (EVEN) {
-            q = fminf(q, 127.0f);
-            q = fmaxf(q, -127.0f);
-            q = rintf(q);
-        } else {
-            q = roundf(q);
-            q = q < 127.0f ? q : 127.0f;   // NaN -> 127, as the reference's std::min/std::max chain
-            q = q > -127.0f ? q : -127.0f;
-        }
-        const int code = (int)q;
-        w[j >> 2] |= (uint32_t)(code & 255) << ((j & 3) * 8);
-    }
+    for (int j = 0; j < 4; ++j)
+        w[j] = pack_low_bytes(quantize_code<EVEN>(v[4 * j], inv), quantize_code<EVEN>(v[4 * j + 1], inv),
+                              quantize_code<EVEN>(v[4 * j + 2], inv), quantize_code<EVEN>(v[4 * j + 3], inv));
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
@@ -240,7 +262,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
                 for (int j = 0; j < 16; ++j)
                     if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
             }
-            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = make_uint4(w[0], w[1], w[2], w[3]);
+            store_codes(a.dst + tiled_chunk_offset(m, c, KB), make_uint4(w[0], w[1], w[2], w[3]));
         }
         return;
     }
@@ -325,7 +347,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
 
     auto emit = [&](int c, const float* vals) {
         const uint4 packed = even ? quantize16<true>(vals, inv) : quantize16<false>(vals, inv);
-        *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = packed;
+        store_codes(a.dst + tiled_chunk_offset(m, c, KB), packed);
     };
     if (cached) {
 #pragma unroll
@@ -340,6 +362,48 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
             emit(c, tmp);
         }
     }
+}
+
+// Re-quantization of many short fp32 rows (the MoE middle: a thousand-odd rows of
+// 1024): one wave per row, four rows per workgroup.  The row maximum comes from
+// the partial maxima the SwiGLU epilogue left behind, so a row needs no
+// workgroup-wide reduction; with a workgroup per row three of its four waves
+// had nothing to do.  Rows of up to 64 * QR_CACHE chunks.
+__global__ __launch_bounds__(256) void requant_rows_wave_kernel(rkh_quant_args a) {
+    const int lane = lane_id(), m = blockIdx.x * 4 + wave_id();
+    if (m >= a.M || (a.active_blocks && m >= a.active_blocks[0] * 32)) return;
+    const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
+    const int nchunks = (K + 15) >> 4;
+    const float* row = static_cast<const float*>(a.src) + (size_t)m * K;
+    const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    float v[QR_CACHE][16];
+#pragma unroll
+    for (int i = 0; i < QR_CACHE; ++i)
+        if (lane + 64 * i < nchunks) RowLoader<float>::load16(row, (lane + 64 * i) * 16, K, vec, v[i]);
+    uint32_t bits = 0; // unsigned compare of |x| bit patterns
+    for (int i = lane; i < a.row_max_parts; i += 64) bits = max(bits, a.row_max_bits[(size_t)m * a.row_max_parts + i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+    const float mx = __uint_as_float(bits);
+    float scale;
+    if (a.mode == RKH_Q_REUSE_BITS) {
+        if (bits >= 0x7f800000u) {
+            if (lane == 0 && a.bad_flag) atomicOr(a.bad_flag, 1);
+            scale = 1.0f;
+        } else {
+            scale = mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN);
+        }
+    } else {
+        scale = mx != 0.0f ? mx / 127.0f : 1.0f;
+    }
+    if (lane == 0 && a.scale) a.scale[m] = scale;
+    const float inv = 1.0f / scale;
+    const bool even = a.mode == RKH_Q_REUSE_BITS_MOE;
+#pragma unroll
+    for (int i = 0; i < QR_CACHE; ++i)
+        if (lane + 64 * i < nchunks)
+            store_codes(a.dst + tiled_chunk_offset(m, lane + 64 * i, KB),
+                        even ? quantize16<true>(v[i], inv) : quantize16<false>(v[i], inv));
 }
 
 // Dense quantization of many rows: one workgroup per ROWS (8 or 4) consecutive
@@ -432,13 +496,13 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
         for (int i = 0; i < Q8_CACHE; ++i) {
             const int c = cl + CSTEP * i;
             if (c < nchunks)
-                *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(v[i], inv);
+                store_codes(a.dst + tiled_chunk_offset(m, c, KB), quantize16<false>(v[i], inv));
         }
     } else {
         for (int c = cl; c < nchunks; c += CSTEP) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
-            *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(m, c, KB)) = quantize16<false>(tmp, inv);
+            store_codes(a.dst + tiled_chunk_offset(m, c, KB), quantize16<false>(tmp, inv));
         }
     }
 }
@@ -1625,7 +1689,7 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
             const uint4 packed = make_uint4(w[0], w[1], w[2], w[3]);
             for (int j = 0; j < slots; ++j) {
                 const int d = dest[j];
-                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+                if (d >= 0) store_codes(a.dst + tiled_chunk_offset(d, c, KB), packed);
             }
         }
     } else {
@@ -1670,7 +1734,7 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
             const uint4 packed = quantize16<true>(vals, inv);
             for (int j = 0; j < slots; ++j) {
                 const int d = dest[j];
-                if (d >= 0) *reinterpret_cast<uint4*>(a.dst + tiled_chunk_offset(d, c, KB)) = packed;
+                if (d >= 0) store_codes(a.dst + tiled_chunk_offset(d, c, KB), packed);
             }
         };
         if (cached) {
@@ -1979,10 +2043,16 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
+    const bool reuse = mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE;
+    if (reuse && args->in_dtype == RKH_F32 && args->M >= 64 && (args->K + 15) / 16 <= 64 * QR_CACHE) {
+        hipLaunchKernelGGL(requant_rows_wave_kernel, dim3((args->M + 3) / 4), block, 0, (hipStream_t)stream, *args);
+        RKH_CHECK(hipGetLastError());
+        return RKH_OK;
+    }
     // Re-quantization of a few long rows: several workgroups per row, about 256 chunks
     // each, until the grid has a few hundred workgroups.
     int split = 1;
-    if (mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE) {
+    if (reuse) {
         const int row_chunks = (args->K + 15) / 16;
         while (split < 8 && args->M * split < 512 && row_chunks / (split * 2) >= 128) split *= 2;
     }
