@@ -124,6 +124,60 @@ def test_f32i8f32_dynamic_and_static(sess, oracle, M, N, K):
             op.close()
 
 
+def test_rounding_ties_neighbours_saturation_and_nan(sess, oracle):
+    """Static scale 1 makes the code round-half-away(x) itself: every tie k + 0.5, the floats on either
+    side of it, the largest float below 0.5 (where x + 0.5 rounds up to 1.0 in fp32), saturation beyond
+    +-127, infinities and NaNs of both signs (the reference's comparison chain turns every NaN into 127).
+    Rows with a dynamic scale of exactly 1 (max |x| = 127) go through the same values."""
+    ties = np.arange(-128, 128, dtype=np.float32) + np.float32(0.5)
+    vals = np.concatenate([ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+                           np.arange(-130, 131, dtype=np.float32),
+                           np.array([0.49999997, -0.49999997, 0.0, -0.0, 126.99999, 127.00001, -127.00001, 1e30,
+                                     -1e30, 1e-30, -1e-30, 127.0], np.float32)]).astype(np.float32)
+    K = (vals.size + 31) // 32 * 32
+    row = np.zeros(K, np.float32)
+    row[:vals.size] = vals
+    special = row.copy()
+    special[:6] = np.array([np.inf, -np.inf, np.nan, -np.nan, 3.5, -3.5], np.float32)
+    special[2:4].view(np.uint32)[:] = [0x7fc00001, 0xffc00001]
+    M = 300                                   # many-row quantization kernel; 5 rows go through the per-row one below
+    A = np.tile(row, (M, 1))
+    A[1::2] = row[::-1]
+    A[7] = special
+    N = 64
+    B = np.zeros((K, N), np.int8)
+    B[np.arange(K), np.arange(K) % N] = 1     # column n sums the codes at k = n (mod N)
+    ws = np.ones(N, np.float32)
+    for rows in (M, 5):
+        Ain = A[:rows] if rows == M else A[[0, 1, 7, 2, 3]]
+        scale = np.ones(rows, np.float32)
+        with np.errstate(over="ignore"):      # 1e30 -> inf in fp16, on purpose
+            halves = Ain.astype(np.float16).view(np.uint16)
+        for kind, x in ((capi.F32I8F32_STATIC, Ain), (capi.F16I8F16_STATIC, halves)):
+            op = ops.W8A8Linear(sess, kind, rows, B, ws)
+            try:
+                rc, got = op.run(x, scale)
+                want = oracle.w8a8(x, B, ws, a_scale_static=scale)
+                assert rc == 0
+                q, _ = op.read_quantized()
+                assert np.array_equal(q, want["q"]), np.argwhere(q != want["q"])[:5].tolist()
+                assert np.array_equal(got.view(np.uint8), want["C"].view(np.uint8))
+            finally:
+                op.close()
+        clipped = np.clip(Ain, -127, 127)      # max |x| = 127 -> dynamic scale exactly 1
+        clipped[np.isnan(clipped)] = 0
+        op = ops.W8A8Linear(sess, capi.F32I8F32_DYNAMIC, rows, B, ws)
+        try:
+            rc, got = op.run(clipped)
+            want = oracle.w8a8(clipped, B, ws)
+            assert rc == 0 and (want["a_scale"] == 1.0).all()
+            q, _ = op.read_quantized()
+            assert np.array_equal(q, want["q"])
+            assert np.array_equal(got.view(np.uint32), want["C"].view(np.uint32))
+        finally:
+            op.close()
+
+
 def test_config0_full(sess, oracle):
     """BASELINE config 0: M=64, K=2048, N=2048, seeds 0/1."""
     c = workloads.CONFIGS[0]()
