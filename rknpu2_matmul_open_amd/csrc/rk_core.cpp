@@ -7,6 +7,8 @@
 #include <cstdlib>
 #include <new>
 
+#include <cstring>
+
 #include "rk_host.h"
 #include "rk_npu_hip.h"
 
@@ -71,6 +73,24 @@ double StageTimer::span_us(int from, int to) {
     double us = 0.0;
     if (rkh_event_elapsed_us(events_[from], events_[to], &us)) return 0.0;
     return us;
+}
+
+HostStage::~HostStage() { rkh_host_free(ptr_); }
+void HostStage::init(size_t bytes) {
+    if (!bytes || bytes > kLimit) return;
+    void* p = nullptr;
+    if (rkh_host_alloc(&p, bytes) == RKH_OK) {
+        ptr_ = p;
+        bytes_ = bytes;
+    }
+}
+void HostStage::init_capped(size_t bytes) { init(bytes < kLimit ? bytes : kLimit); }
+const void* HostStage::fill(const void* user, size_t bytes) const {
+    std::memcpy(ptr_, user, bytes <= bytes_ ? bytes : bytes_);
+    return ptr_;
+}
+void HostStage::finish(void* user, size_t bytes) const {
+    if (ptr_ && bytes <= bytes_) std::memcpy(user, ptr_, bytes);
 }
 
 BadFlag::~BadFlag() { rkh_host_free(host_); }

@@ -123,6 +123,10 @@ typedef struct rkh_quant_args {
     int row_max_parts;
     /* If non-NULL, rows at or beyond active_blocks[0] * 32 are skipped. */
     const int* active_blocks;
+    /* src is pinned host memory read over the bus: every row must be read once,
+     * so the quantization is not folded into a GEMV whose workgroups would each
+     * fetch the rows again. */
+    int src_is_host;
 } rkh_quant_args;
 int rkh_quant_rows(void* stream, const rkh_quant_args* args);
 

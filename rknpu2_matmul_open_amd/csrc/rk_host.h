@@ -143,6 +143,38 @@ private:
     DeviceBuffer dev_;
     int* host_ = nullptr;
 };
+// Pinned, device-visible mirror of a caller's host buffer for the blocking
+// host-pointer entry points.  A copy between pageable memory and the device is
+// staged and waited for inside the runtime, once per direction (~15-20 us
+// each); a copy from pinned memory still costs a DMA round of ~8-12 us.  The
+// kernels can instead read the mirror of a small input directly (each row is
+// read once, by the quantization kernel) and write a small result straight into
+// the mirror of the output, which adds ~1.5 us to a call.  Only for buffers up
+// to kLimit: beyond that the bus transfer itself dominates and the DMA engines
+// do it without occupying compute units.  A failed allocation leaves the stage
+// off (the call then copies from / to the caller's buffer as before).
+class HostStage {
+public:
+    static constexpr size_t kLimit = size_t(1) << 20;
+    HostStage() = default;
+    HostStage(const HostStage&) = delete;
+    HostStage& operator=(const HostStage&) = delete;
+    ~HostStage();
+    void init(size_t bytes);        // stays off for 0 or more than kLimit bytes
+    void init_capped(size_t bytes); // min(bytes, kLimit): for buffers whose use varies from call to call
+    explicit operator bool() const { return ptr_ != nullptr; }
+    bool fits(size_t bytes) const { return ptr_ && bytes <= bytes_; }
+    // The mirror, filled with `bytes` from `user` (kernels read it in place).
+    const void* fill(const void* user, size_t bytes) const;
+    // The mirror as a kernel's output; finish() copies it on to `user` after the wait.
+    void* data() const { return ptr_; }
+    void finish(void* user, size_t bytes) const;
+
+private:
+    void* ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
 // Blocking check of one raw device flag (used by rk_npu_hip_sync).
 bool consume_device_flag(rk_npu_ctx* ctx, int* flag);
 void note_pending_flag(rk_npu_ctx* ctx, int* flag);

@@ -70,6 +70,7 @@ struct rk_npu_i4_workspace {
     DeviceBuffer a_tiled;         // the same, MFMA-tiled
     DeviceBuffer c_out;           // [M, N] int32
     DeviceBuffer splitk;
+    HostStage stage_a, stage_c;   // pinned mirrors of small codes / results, used in place by the kernels
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
 };
 
@@ -87,13 +88,22 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
             rk_npu_i4_timings* t) {
     const rk_npu_i4_config& c = ws->config;
     rk_npu_ctx* ctx = ws->owner.ctx;
+    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
+    const size_t c_bytes = (size_t)c.M * c.N * sizeof(int32_t);
     int rc;
     auto start = Clock::now();
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), codes, (size_t)c.M * c.K));
+        const size_t a_bytes = (size_t)c.M * c.K;
         rkh_quant_args q{};
         q.src = ws->a_raw.as<>();
+        if (direct_in) {
+            q.src = ws->stage_a.fill(codes, a_bytes);
+            q.src_is_host = 1;
+            rc = RK_NPU_OK;
+        } else {
+            rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), codes, a_bytes));
+        }
         q.in_dtype = RKH_I8;
         q.mode = RKH_Q_COPY_I8;
         q.M = c.M;
@@ -107,7 +117,7 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
         g.N = c.N;
         g.K = c.K;
         g.epilogue = RKH_EPI_I32;
-        g.C = ws->c_out.as<>();
+        g.C = direct_out ? ws->stage_c.data() : ws->c_out.as<>();
         g.ldc = c.N;
         g.splitk_acc = ws->splitk ? ws->splitk.as<int32_t>() : nullptr;
         if (!rc) rc = map_error(rkh_quant_gemm(ctx->stream, &q, &g));
@@ -116,9 +126,10 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
         if (!rc) rc = map_error(rkh_sync(ctx->stream));
         t->sync_us += elapsed_us(start);
         start = Clock::now();
-        if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), (size_t)c.M * c.N * sizeof(int32_t)));
+        if (!rc && direct_out) ws->stage_c.finish(C, c_bytes);
+        else if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }
-    const int wait = map_error(rkh_sync(ctx->stream));
+    const int wait = direct_out ? RK_NPU_OK : map_error(rkh_sync(ctx->stream));
     t->reduce_us += elapsed_us(start);
     return rc ? rc : wait;
 }
@@ -215,6 +226,8 @@ rk_npu_i4_workspace* rk_npu_i4_workspace_create(rk_npu_iommu_domain* domain, con
         return nullptr;
     const size_t scratch = splitk_scratch_bytes(M, N, K, true);
     if (scratch && ws->splitk.alloc(ws->owner, scratch)) return nullptr;
+    ws->stage_a.init((size_t)M * K);
+    ws->stage_c.init((size_t)M * N * sizeof(int32_t));
     if (rkh_sync(domain->ctx->stream)) return nullptr;
     return ws.release();
 }

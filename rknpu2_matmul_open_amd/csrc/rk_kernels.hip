@@ -1871,7 +1871,7 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 // The decode path can quantize inside the GEMV when the rows fit the kernel's
 // LDS staging and per-thread register cache.
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g) {
-    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU) return false;
+    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU || q.src_is_host) return false;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
     const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;

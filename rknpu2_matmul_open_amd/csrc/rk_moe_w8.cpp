@@ -100,6 +100,10 @@ struct rk_npu_moe_w8_workspace {
     DeviceBuffer h_scale;      // [sorted_rows]
     DeviceBuffer y;            // [sorted_rows, H] fp32 expert outputs
     DeviceBuffer out;          // [max_rows, H] fp32
+    // pinned mirrors for the host-pointer entry points: tokens and result (read /
+    // written in place by the kernels when a call's share fits), routing table
+    // [ids | coefficients | token scales] for max_rows
+    HostStage stage_in, stage_out, stage_route;
     BadFlag flag;
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     uint64_t bytes() const {
@@ -271,24 +275,57 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
         return RK_NPU_OK;
     }
     StageTimer timer(ctx->stream, timings != nullptr);
+    // Where the copies go.  Tokens are read once each and the result is written
+    // once, so when they fit their pinned mirrors the kernels use those in place.
+    // The routing table is read by every token's workgroup: in place only for a
+    // decode-sized call, otherwise uploaded (from its mirror, without a wait).
+    const size_t in_bytes = values * (f32 ? 4 : 1), out_bytes = values * 4;
+    const bool direct_in = ws->stage_in.fits(in_bytes), direct_out = ws->stage_out.fits(out_bytes);
+    const bool direct_route = ws->stage_route && rows <= 16;
+    const void* d_input = ws->input.as<>();
+    const float* d_scales = ws->token_scale.as<float>();
+    const int32_t* d_ids = ws->ids.as<int32_t>();
+    const float* d_routes = ws->routes.as<float>();
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, values * (f32 ? 4 : 1)));
-        if (!rc && !f32) rc = map_error(rkh_h2d(ctx->stream, ws->token_scale.as<>(), scales, (size_t)rows * 4));
-        if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->ids.as<>(), ids, nslots * 4));
-        if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->routes.as<>(), routes, nslots * 4));
+        if (direct_in) d_input = ws->stage_in.fill(input, in_bytes);
+        else rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, in_bytes));
+        const void *h_ids = ids, *h_routes = routes, *h_scales = scales;
+        if (ws->stage_route) {
+            const size_t table = (size_t)ws->config.max_rows * top * 4;
+            uint8_t* mirror = static_cast<uint8_t*>(ws->stage_route.data());
+            std::memcpy(mirror, ids, nslots * 4);
+            std::memcpy(mirror + table, routes, nslots * 4);
+            if (!f32) std::memcpy(mirror + 2 * table, scales, (size_t)rows * 4);
+            h_ids = mirror;
+            h_routes = mirror + table;
+            h_scales = mirror + 2 * table;
+        }
+        if (direct_route) {
+            d_ids = static_cast<const int32_t*>(h_ids);
+            d_routes = static_cast<const float*>(h_routes);
+            if (!f32) d_scales = static_cast<const float*>(h_scales);
+        } else {
+            if (!rc && !f32) rc = map_error(rkh_h2d(ctx->stream, ws->token_scale.as<>(), h_scales, (size_t)rows * 4));
+            if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->ids.as<>(), h_ids, nslots * 4));
+            if (!rc) rc = map_error(rkh_h2d(ctx->stream, ws->routes.as<>(), h_routes, nslots * 4));
+        }
         timer.mark(); // 0
         if (!rc)
-            rc = enqueue(ws, w, rows, ws->input.as<>(), f32, ws->token_scale.as<float>(),
-                         ws->ids.as<int32_t>(), ws->routes.as<float>(), ws->out.as<float>(), &timer);
+            rc = enqueue(ws, w, rows, d_input, f32, d_scales, d_ids, d_routes,
+                         direct_out ? static_cast<float*>(ws->stage_out.data()) : ws->out.as<float>(), &timer);
         if (!rc) rc = ws->flag.enqueue_readback(ctx->stream);
     }
     const int wait = map_error(rkh_sync(ctx->stream));
     if (rc || wait) return rc ? rc : wait;
     if (ws->flag.consume(ctx->stream)) return RK_NPU_ERR_PARAM; // NaN / Inf token
     const auto t1 = Clock::now();
-    rc = map_error(rkh_d2h(ctx->stream, output, ws->out.as<>(), values * 4));
-    if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    if (direct_out) {
+        ws->stage_out.finish(output, out_bytes);
+    } else {
+        rc = map_error(rkh_d2h(ctx->stream, output, ws->out.as<>(), out_bytes));
+        if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    }
     if (timings) {
         timings->schedule_us = timer.span_us(0, 1);
         timings->input_us = timer.span_us(1, 2);
@@ -453,6 +490,9 @@ rk_npu_moe_w8_workspace* create_workspace(rk_npu_iommu_domain* domain, const rk_
         ws->h_scale.alloc(ws->owner, S * 4) || ws->y.alloc(ws->owner, S * H * 4) ||
         ws->out.alloc(ws->owner, (size_t)R * H * 4, false) || ws->flag.init(ws->owner))
         return nullptr;
+    ws->stage_in.init_capped((size_t)R * H * 4);
+    ws->stage_out.init_capped((size_t)R * H * 4);
+    ws->stage_route.init((size_t)routed * 8 + (size_t)R * 4);
     if (rkh_sync(domain->ctx->stream)) return nullptr;
     return ws.release();
 }

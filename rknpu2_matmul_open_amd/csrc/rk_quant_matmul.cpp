@@ -118,6 +118,7 @@ struct rk_npu_matmul_workspace {
     DeviceBuffer a_scale;  // [align128(M)] fp32
     DeviceBuffer c_out;    // [M, N] result before the copy back
     DeviceBuffer splitk;   // int32 scratch when the shape may split K
+    HostStage stage_a, stage_scale, stage_c; // pinned mirrors of small A / static scales / C
     BadFlag flag;
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
 };
@@ -142,12 +143,13 @@ rkh_gemm_args gemm_args(rk_npu_matmul_workspace* ws, const Weights& w, void* dC)
 }
 
 // Enqueue quantize + GEMM on the context's stream (one fused kernel for
-// decode-sized M).  dA / dC are device pointers; static scales are expected in
-// the workspace's a_scale buffer.
-int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA, void* dC) {
+// decode-sized M, unless A is a pinned host mirror).  dA / dC are device-
+// visible pointers; static scales are expected in the workspace's a_scale buffer.
+int enqueue(rk_npu_matmul_workspace* ws, const Weights& w, const void* dA, void* dC, bool a_is_host = false) {
     const auto& s = ws->strategy;
     rkh_quant_args q{};
     q.src = dA;
+    q.src_is_host = a_is_host ? 1 : 0;
     q.in_dtype = ws->t.in_dtype;
     q.mode = ws->t.quant == 0 ? RKH_Q_COPY_I8 : ws->t.quant == 1 ? RKH_Q_W8_DYNAMIC : RKH_Q_W8_STATIC;
     q.M = s.M;
@@ -184,15 +186,24 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
     rk_npu_ctx* ctx = ws->owner.ctx;
     const size_t a_bytes = (size_t)s.M * s.K * elem_bytes(ws->t.in_dtype);
     const size_t c_bytes = (size_t)s.M * s.N * elem_bytes(out_dtype(ws->t.out_epi));
+    // Small operands skip the copies: the kernels read A from / write C into the
+    // pinned mirrors.  Static scales are read by every workgroup of the GEMM, so
+    // they are always uploaded (from their mirror when there is one).
+    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
+    const size_t scale_bytes = (size_t)s.M * sizeof(float);
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        const void* src = ws->a_raw.as<>();
+        if (direct_in) src = ws->stage_a.fill(A, a_bytes);
+        else rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         if (!rc && ws->t.quant == 2)
-            rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(), a_scale, (size_t)s.M * sizeof(float)));
-        if (!rc) rc = enqueue(ws, *w, ws->a_raw.as<>(), ws->c_out.as<>());
-        if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
+            rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(),
+                                   ws->stage_scale ? ws->stage_scale.fill(a_scale, scale_bytes) : a_scale, scale_bytes));
+        if (!rc) rc = enqueue(ws, *w, src, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), direct_in);
+        if (!rc && !direct_out) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }
     const int wait = map_error(rkh_sync(ctx->stream));
+    if (!rc && !wait && direct_out) ws->stage_c.finish(C, c_bytes);
     return rc ? rc : wait;
 }
 
@@ -304,6 +315,9 @@ rk_npu_matmul_workspace* rk_npu_matmul_workspace_create(rk_npu_iommu_domain* dom
         return nullptr;
     const size_t scratch = splitk_scratch_bytes(M, N, K, false);
     if (scratch && ws->splitk.alloc(ws->owner, scratch)) return nullptr;
+    ws->stage_a.init((size_t)M * K * elem_bytes(ws->t.in_dtype));
+    if (ws->t.quant == 2) ws->stage_scale.init((size_t)M * sizeof(float));
+    ws->stage_c.init((size_t)M * N * elem_bytes(out_dtype(ws->t.out_epi)));
     if (rkh_sync(domain->ctx->stream)) return nullptr;
     return ws.release();
 }

@@ -233,6 +233,7 @@ struct rk_npu_w4a8_workspace {
     DeviceBuffer c_out;     // [M, N] fp32-sized result staging
     DeviceBuffer row_max;   // [align128(M)][N/64] partial row maxima of the SwiGLU middle
     DeviceBuffer splitk;
+    HostStage stage_a, stage_c; // pinned mirrors of a small A / C that the kernels read / write in place
     BadFlag flag;
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     ~rk_npu_w4a8_workspace() {
@@ -269,11 +270,12 @@ rkh_gemm_args gemm_args(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w,
 // row_max feeds the scale (reference run_locked(scale_source), :98-151).
 int enqueue(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void* dA, bool half,
             void* dC, Out out, bool collect, rk_npu_w4a8_workspace* scale_source,
-            StageTimer* timer) {
+            StageTimer* timer, bool a_is_host = false) {
     const auto& c = ws->config;
     void* stream = ws->owner.ctx->stream;
     rkh_quant_args q{};
     q.src = dA;
+    q.src_is_host = a_is_host ? 1 : 0;
     q.in_dtype = half ? RKH_F16 : RKH_F32;
     q.M = c.M;
     q.K = c.K;
@@ -366,11 +368,18 @@ int run_host(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void
     const size_t out_cols = swiglu ? (size_t)c.N / 2 : (size_t)c.N;
     const size_t c_bytes = (size_t)c.M * out_cols * (out == Out::F16 ? 2 : 4);
     StageTimer timer(ctx->stream, timings != nullptr);
+    // Small operands skip the copies: the kernels read A from / write the result
+    // into the pinned mirrors (the caller's C is only written after the checks).
+    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        const void* src = ws->a_raw.as<>();
+        if (direct_in) src = ws->stage_a.fill(A, a_bytes);
+        else rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         timer.mark();
-        if (!rc) rc = enqueue(ws, w, ws->a_raw.as<>(), half, ws->c_out.as<>(), out, false, nullptr, &timer);
+        if (!rc)
+            rc = enqueue(ws, w, src, half, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), out, false, nullptr,
+                         &timer, direct_in);
         if (!rc) rc = ws->flag.enqueue_readback(ctx->stream);
     }
     int wait = map_error(rkh_sync(ctx->stream));
@@ -384,8 +393,12 @@ int run_host(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void
         return RK_NPU_ERR_PARAM; // NaN / Inf activation: C is not written
     }
     const auto t1 = Clock::now();
-    rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
-    if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    if (direct_out) {
+        ws->stage_c.finish(C, c_bytes);
+    } else {
+        rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
+        if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    }
     fill_timings(timings, timer, 0, true, elapsed_us(t1), elapsed_us(t0));
     return rc;
 }
@@ -618,6 +631,8 @@ rk_npu_w4a8_workspace* rk_npu_w4a8_workspace_create_ex(rk_npu_iommu_domain* doma
         return nullptr;
     const size_t scratch = splitk_scratch_bytes(M, N, K, true);
     if (scratch && ws->splitk.alloc(ws->owner, scratch)) return nullptr;
+    ws->stage_a.init((size_t)M * K * 4);
+    ws->stage_c.init((size_t)M * N * 4);
     if (rkh_sync(domain->ctx->stream)) return nullptr;
     return ws.release();
 }
@@ -669,14 +684,21 @@ int rk_npu_w4a8_run_ffn_f32(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights
     const auto t0 = Clock::now();
     rk_npu_ctx* ctx = gu->owner.ctx;
     const int M = gu->config.M, F = gu->config.N / 2;
+    const size_t a_bytes = (size_t)M * gu->config.K * 4, c_bytes = (size_t)M * dn->config.N * 4;
+    const bool direct_in = (bool)gu->stage_a, direct_out = dn->stage_c && dn->config.M == M;
     StageTimer timer(ctx->stream, metrics != nullptr);
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        rc = map_error(rkh_h2d(ctx->stream, gu->a_raw.as<>(), A, (size_t)M * gu->config.K * 4));
+        const void* src = gu->a_raw.as<>();
+        if (direct_in) src = gu->stage_a.fill(A, a_bytes);
+        else rc = map_error(rkh_h2d(ctx->stream, gu->a_raw.as<>(), A, a_bytes));
         timer.mark();                                                                        // 0
-        // middle lives in the gate/up workspace's result buffer
-        if (!rc) rc = enqueue(gu, guw, gu->a_raw.as<>(), false, gu->c_out.as<>(), Out::SwiGLU, true, nullptr, &timer); // 1,2
-        if (!rc) rc = enqueue(dn, dnw, gu->c_out.as<>(), false, dn->c_out.as<>(), Out::F32, false, gu, &timer);        // 3,4
+        // middle lives in the gate/up workspace's result buffer (on the device: the
+        // re-quantization reads it back)
+        if (!rc) rc = enqueue(gu, guw, src, false, gu->c_out.as<>(), Out::SwiGLU, true, nullptr, &timer, direct_in); // 1,2
+        if (!rc)
+            rc = enqueue(dn, dnw, gu->c_out.as<>(), false, direct_out ? dn->stage_c.data() : dn->c_out.as<>(), Out::F32,
+                         false, gu, &timer);                                                                         // 3,4
         if (!rc) rc = gu->flag.enqueue_readback(ctx->stream);
         if (!rc) rc = dn->flag.enqueue_readback(ctx->stream);
     }
@@ -687,8 +709,9 @@ int rk_npu_w4a8_run_ffn_f32(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights
     if (bad_in || bad_mid) return RK_NPU_ERR_PARAM; // NaN/Inf input or non-finite middle
     const auto t1 = Clock::now();
     rc = map_error(rkh_d2h(ctx->stream, middle, gu->c_out.as<>(), (size_t)M * F * 4));
-    if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, dn->c_out.as<>(), (size_t)M * dn->config.N * 4));
+    if (!rc && !direct_out) rc = map_error(rkh_d2h(ctx->stream, C, dn->c_out.as<>(), c_bytes));
     if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    if (!rc && direct_out) dn->stage_c.finish(C, c_bytes);
     if (metrics) {
         const double copy = elapsed_us(t1);
         fill_timings(&metrics->gate_up, timer, 0, true, copy, 0.0);
