@@ -286,21 +286,22 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     const float* d_scales = ws->token_scale.as<float>();
     const int32_t* d_ids = ws->ids.as<int32_t>();
     const float* d_routes = ws->routes.as<float>();
+    // the mirrors are filled before the context's submission lock is taken
+    if (direct_in) d_input = ws->stage_in.fill(input, in_bytes);
+    const void *h_ids = ids, *h_routes = routes, *h_scales = scales;
+    if (ws->stage_route) {
+        const size_t table = (size_t)ws->config.max_rows * top * 4;
+        uint8_t* mirror = static_cast<uint8_t*>(ws->stage_route.data());
+        std::memcpy(mirror, ids, nslots * 4);
+        std::memcpy(mirror + table, routes, nslots * 4);
+        if (!f32) std::memcpy(mirror + 2 * table, scales, (size_t)rows * 4);
+        h_ids = mirror;
+        h_routes = mirror + table;
+        h_scales = mirror + 2 * table;
+    }
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        if (direct_in) d_input = ws->stage_in.fill(input, in_bytes);
-        else rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, in_bytes));
-        const void *h_ids = ids, *h_routes = routes, *h_scales = scales;
-        if (ws->stage_route) {
-            const size_t table = (size_t)ws->config.max_rows * top * 4;
-            uint8_t* mirror = static_cast<uint8_t*>(ws->stage_route.data());
-            std::memcpy(mirror, ids, nslots * 4);
-            std::memcpy(mirror + table, routes, nslots * 4);
-            if (!f32) std::memcpy(mirror + 2 * table, scales, (size_t)rows * 4);
-            h_ids = mirror;
-            h_routes = mirror + table;
-            h_scales = mirror + 2 * table;
-        }
+        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, in_bytes));
         if (direct_route) {
             d_ids = static_cast<const int32_t*>(h_ids);
             d_routes = static_cast<const float*>(h_routes);

@@ -191,14 +191,15 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
     // they are always uploaded (from their mirror when there is one).
     const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
     const size_t scale_bytes = (size_t)s.M * sizeof(float);
+    // the mirrors are filled before the context's submission lock is taken
+    const void* src = direct_in ? ws->stage_a.fill(A, a_bytes) : ws->a_raw.as<>();
+    const void* scale_src = a_scale;
+    if (ws->t.quant == 2 && ws->stage_scale) scale_src = ws->stage_scale.fill(a_scale, scale_bytes);
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        const void* src = ws->a_raw.as<>();
-        if (direct_in) src = ws->stage_a.fill(A, a_bytes);
-        else rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         if (!rc && ws->t.quant == 2)
-            rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(),
-                                   ws->stage_scale ? ws->stage_scale.fill(a_scale, scale_bytes) : a_scale, scale_bytes));
+            rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(), scale_src, scale_bytes));
         if (!rc) rc = enqueue(ws, *w, src, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), direct_in);
         if (!rc && !direct_out) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }

@@ -371,11 +371,10 @@ int run_host(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void
     // Small operands skip the copies: the kernels read A from / write the result
     // into the pinned mirrors (the caller's C is only written after the checks).
     const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
+    const void* src = direct_in ? ws->stage_a.fill(A, a_bytes) : ws->a_raw.as<>(); // before the submission lock
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        const void* src = ws->a_raw.as<>();
-        if (direct_in) src = ws->stage_a.fill(A, a_bytes);
-        else rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         timer.mark();
         if (!rc)
             rc = enqueue(ws, w, src, half, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), out, false, nullptr,
@@ -687,11 +686,10 @@ int rk_npu_w4a8_run_ffn_f32(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights
     const size_t a_bytes = (size_t)M * gu->config.K * 4, c_bytes = (size_t)M * dn->config.N * 4;
     const bool direct_in = (bool)gu->stage_a, direct_out = dn->stage_c && dn->config.M == M;
     StageTimer timer(ctx->stream, metrics != nullptr);
+    const void* src = direct_in ? gu->stage_a.fill(A, a_bytes) : gu->a_raw.as<>(); // before the submission lock
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        const void* src = gu->a_raw.as<>();
-        if (direct_in) src = gu->stage_a.fill(A, a_bytes);
-        else rc = map_error(rkh_h2d(ctx->stream, gu->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, gu->a_raw.as<>(), A, a_bytes));
         timer.mark();                                                                        // 0
         // middle lives in the gate/up workspace's result buffer (on the device: the
         // re-quantization reads it back)
