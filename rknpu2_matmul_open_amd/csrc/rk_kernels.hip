@@ -1428,13 +1428,20 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // row block and column tile; they run side by side and the second one finds
 // the weights in L2 (taking all row blocks of an expert into one workgroup was
 // measured slower: fewer workgroups than compute units remain).
-template <int EPI>
+// KSPLIT (decode-sized calls: a handful of row blocks would leave most compute
+// units without a workgroup): the tile is 64 columns, the four waves take a
+// quarter of K each and their accumulators are added through LDS before wave 0
+// runs the epilogue -- four times as many workgroups, each wave with its whole
+// share of the weights in flight at once.
+template <int EPI, bool KSPLIT>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
     constexpr int TN = 2, WAVES = 4;
-    constexpr int RING = 8;
+    constexpr int RING = 8; // (16 for the K-split variant, a wave's whole share in flight, was measured slower)
     constexpr int LPS = 1 + TN;
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
-    __shared__ __attribute__((aligned(16))) uint8_t stage_raw[WAVES * 32 * (32 * 4 + 8)];
+    constexpr int STAGE_BYTES = WAVES * 32 * (32 * 4 + 8);
+    constexpr int XCH_BYTES = KSPLIT ? (WAVES - 1) * TN * 16 * 64 * 4 : 0;
+    __shared__ __attribute__((aligned(16))) uint8_t stage_raw[STAGE_BYTES + XCH_BYTES];
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
@@ -1447,13 +1454,17 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     const uint8_t* Wb = g.W + (size_t)e * g.w_expert_stride;
     const float* w_scale = g.w_scale ? g.w_scale + (size_t)e * g.ws_expert_stride : nullptr;
 
-    const int pb0 = (nblk * WAVES + wave) * TN;
-    const uint8_t* asrc = g.A + (size_t)mblk * KB * 1024;
+    // this wave's column blocks and k-tiles [kt0, kt0 + kts)
+    const int pb0 = KSPLIT ? nblk * TN : (nblk * WAVES + wave) * TN;
+    const int share = KSPLIT ? (KB + WAVES - 1) / WAVES : KB;
+    const int kts = KSPLIT ? max(0, min(share, KB - wave * share)) : KB;
+    const int kt0 = KSPLIT ? min(wave * share, KB - 1) : 0; // (a wave without a share still loads in bounds)
+    const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * 1024;
     const uint8_t* wsrc[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) wsrc[j] = Wb + (size_t)(pb0 + j) * KB * 1024;
+    for (int j = 0; j < TN; ++j) wsrc[j] = Wb + ((size_t)(pb0 + j) * KB + kt0) * 1024;
     const unsigned lane_off = lane * 16;
-    int left = KB - 1; // how often the sources may still advance
+    int left = max(kts, 1) - 1; // how often the sources may still advance
 
     v16i acc[TN];
 #pragma unroll
@@ -1485,14 +1496,17 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
 
 #pragma unroll
     for (int t = 0; t < RING - 1; ++t) issue(ring[t]);
-    for (int s = 0; s < KB; s += RING)
+    for (int s = 0; s < kts; s += RING)
         static_for<RING>([&](auto slot_tag) {
             constexpr int SLOT = decltype(slot_tag)::value;
             issue(ring[(SLOT + RING - 1) % RING]);
             wait(ring[SLOT]);
+            // (a K share need not be a multiple of RING: the steps past its end reload the last tile and are skipped)
+            if (!KSPLIT || s + SLOT < kts) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][1 + j], ring[SLOT][0], acc[j], 0, 0, 0);
+                for (int j = 0; j < TN; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][1 + j], ring[SLOT][0], acc[j], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
     // The look-ahead loads beyond K are still in flight here and the compiler
@@ -1505,6 +1519,32 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
 #pragma unroll
         for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(ring[t][l]));
 
+    if constexpr (KSPLIT) {
+        // waves 1..3 hand their accumulators to wave 0: [wave - 1][tile][q][lane] x 4 ints
+        int* xch = reinterpret_cast<int*>(stage_raw + STAGE_BYTES);
+        if (wave > 0) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<v4i*>(xch + ((((wave - 1) * TN + j) * 4 + q) * 64 + lane) * 4) =
+                        v4i{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const v4i got = *reinterpret_cast<const v4i*>(xch + (((w * TN + j) * 4 + q) * 64 + lane) * 4);
+                    acc[j][q * 4] += got.x;
+                    acc[j][q * 4 + 1] += got.y;
+                    acc[j][q * 4 + 2] += got.z;
+                    acc[j][q * 4 + 3] += got.w;
+                }
+    }
     const int m_limit = g.num_blocks[0] * 32;
     uint8_t* stage_lds = stage_raw + wave * (32 * (32 * 4 + 8));
     const int m0 = mblk * 32;
@@ -1773,14 +1813,26 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 }
 
 // ------------------------------------------------------------- launchers
+// Workgroups of the 256-column grid below which the K-split variant is used.  Measured on a 32-expert
+// top-4 layer (H 2048, I 1024): 1 / 2 tokens 32.9 -> 27.1 / 37.7 -> 35.7 us; from 4 tokens (16 possible
+// row blocks) on the wide tile is faster again (41.4 vs 44.6 us).
+constexpr long GROUPED_KSPLIT_BELOW = 96;
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
-// 256-column tile); blocks beyond the live count exit at once.
+// 256-column tile); blocks beyond the live count exit at once.  When that grid
+// would leave compute units idle (max_blocks is the caller's bound for this
+// call, a handful for a decode step) the tile shrinks to 64 columns and the
+// waves split K instead.
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     if (g.w_int4) return RKH_ERR_RUNTIME;
     const int mblocks = g.max_blocks;
-    const int nblocks = (g.N + 255) / 256;
+    const bool ksplit = (long)mblocks * ((g.N + 255) / 256) < GROUPED_KSPLIT_BELOW;
+    const int nblocks = ksplit ? (g.N + 63) / 64 : (g.N + 255) / 256;
     const dim3 grid(mblocks * nblocks), block(256);
-#define RK_LAUNCH(EPI) hipLaunchKernelGGL((gemm_stream_kernel<EPI>), grid, block, 0, st, g, mblocks, nblocks)
+#define RK_LAUNCH(EPI)                                                                                        \
+    do {                                                                                                      \
+        if (ksplit) hipLaunchKernelGGL((gemm_stream_kernel<EPI, true>), grid, block, 0, st, g, mblocks, nblocks); \
+        else hipLaunchKernelGGL((gemm_stream_kernel<EPI, false>), grid, block, 0, st, g, mblocks, nblocks);   \
+    } while (0)
     switch (g.epilogue) {
     case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
     case RKH_EPI_F16: RK_LAUNCH(RKH_EPI_F16); break;

@@ -132,6 +132,10 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     const int H = wc.hidden, I = wc.intermediate;
     void* stream = ws->owner.ctx->stream;
     auto mark = [&] { if (timer) timer->mark(); };
+    // most row blocks this call can produce (the workspace's max_blocks is the same bound for max_rows)
+    const int routed = rows * ws->config.top_k;
+    const int call_blocks = std::min(ws->max_blocks, routed / 32 + std::min(wc.routed_experts, routed) +
+                                                         (wc.shared_expert ? (rows + 31) / 32 : 0));
 
     rkh_moe_scatter_args r{};
     r.ids = d_ids;
@@ -171,7 +175,7 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     g.row_max_bits = ws->row_max.as<uint32_t>();
     g.blk_expert = ws->blk_expert.as<int>();
     g.num_blocks = ws->num_blocks.as<int>();
-    g.max_blocks = ws->max_blocks;
+    g.max_blocks = call_blocks;
     g.w_expert_stride = w->gate_stride;
     g.ws_expert_stride = (size_t)2 * I;
     rc = rkh_gemm(stream, &g);
@@ -206,7 +210,7 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     d.ldc = H;
     d.blk_expert = ws->blk_expert.as<int>();
     d.num_blocks = ws->num_blocks.as<int>();
-    d.max_blocks = ws->max_blocks;
+    d.max_blocks = call_blocks;
     d.w_expert_stride = w->down_stride;
     d.ws_expert_stride = (size_t)H;
     rc = rkh_gemm(stream, &d);
