@@ -1428,19 +1428,21 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // row block and column tile; they run side by side and the second one finds
 // the weights in L2 (taking all row blocks of an expert into one workgroup was
 // measured slower: fewer workgroups than compute units remain).
-// KSPLIT (decode-sized calls: a handful of row blocks would leave most compute
-// units without a workgroup): the tile is 64 columns, the four waves take a
-// quarter of K each and their accumulators are added through LDS before wave 0
-// runs the epilogue -- four times as many workgroups, each wave with its whole
-// share of the weights in flight at once.
-template <int EPI, bool KSPLIT>
+// KS = 4 (decode-sized calls, whose handful of row blocks would leave most
+// compute units without a workgroup): the tile shrinks to 256 / KS columns and
+// KS waves share a column pair, taking 1/KS of K each; their accumulators are
+// added through LDS before the first of them runs the epilogue -- KS times as
+// many workgroups.
+template <int EPI, int KS>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
     constexpr int TN = 2, WAVES = 4;
-    constexpr int RING = 8; // (16 for the K-split variant, a wave's whole share in flight, was measured slower)
+    constexpr bool KSPLIT = KS > 1;
+    constexpr int CG = WAVES / KS; // column pairs per workgroup
+    constexpr int RING = 8; // (16 with K split four ways, a wave's whole share in flight, was measured slower)
     constexpr int LPS = 1 + TN;
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
     constexpr int STAGE_BYTES = WAVES * 32 * (32 * 4 + 8);
-    constexpr int XCH_BYTES = KSPLIT ? (WAVES - 1) * TN * 16 * 64 * 4 : 0;
+    constexpr int XCH_BYTES = KSPLIT ? CG * (KS - 1) * TN * 16 * 64 * 4 : 0;
     __shared__ __attribute__((aligned(16))) uint8_t stage_raw[STAGE_BYTES + XCH_BYTES];
 
     const int lane = lane_id();
@@ -1455,10 +1457,11 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     const float* w_scale = g.w_scale ? g.w_scale + (size_t)e * g.ws_expert_stride : nullptr;
 
     // this wave's column blocks and k-tiles [kt0, kt0 + kts)
-    const int pb0 = KSPLIT ? nblk * TN : (nblk * WAVES + wave) * TN;
-    const int share = KSPLIT ? (KB + WAVES - 1) / WAVES : KB;
-    const int kts = KSPLIT ? max(0, min(share, KB - wave * share)) : KB;
-    const int kt0 = KSPLIT ? min(wave * share, KB - 1) : 0; // (a wave without a share still loads in bounds)
+    const int cg = wave / KS, kq = wave % KS; // column pair, part of K
+    const int pb0 = (nblk * CG + cg) * TN;
+    const int share = (KB + KS - 1) / KS;
+    const int kts = max(0, min(share, KB - kq * share));
+    const int kt0 = min(kq * share, KB - 1); // (a wave without a share still loads in bounds)
     const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * 1024;
     const uint8_t* wsrc[TN];
 #pragma unroll
@@ -1520,20 +1523,20 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
         for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(ring[t][l]));
 
     if constexpr (KSPLIT) {
-        // waves 1..3 hand their accumulators to wave 0: [wave - 1][tile][q][lane] x 4 ints
-        int* xch = reinterpret_cast<int*>(stage_raw + STAGE_BYTES);
-        if (wave > 0) {
+        // the other parts of K hand their accumulators to part 0: [column pair][part - 1][tile][q][lane] x 4 ints
+        int* xch = reinterpret_cast<int*>(stage_raw + STAGE_BYTES) + cg * (KS - 1) * TN * 16 * 64;
+        if (kq > 0) {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<v4i*>(xch + ((((wave - 1) * TN + j) * 4 + q) * 64 + lane) * 4) =
+                    *reinterpret_cast<v4i*>(xch + ((((kq - 1) * TN + j) * 4 + q) * 64 + lane) * 4) =
                         v4i{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
         }
         __syncthreads();
-        if (wave > 0) return;
+        if (kq > 0) return;
 #pragma unroll
-        for (int w = 0; w < WAVES - 1; ++w)
+        for (int w = 0; w < KS - 1; ++w)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -1816,7 +1819,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 // Workgroups of the 256-column grid below which the K-split variant is used.  Measured on a 32-expert
 // top-4 layer (H 2048, I 1024): 1 / 2 tokens 32.9 -> 27.1 / 37.7 -> 35.7 us; from 4 tokens (16 possible
 // row blocks) on the wide tile is faster again (41.4 vs 44.6 us).
-constexpr long GROUPED_KSPLIT_BELOW = 96;
+// (Splitting K two ways over 128-column tiles for 4 .. 64 tokens was measured too: 1 - 3 us slower than
+// the wide tile at every size.)
+constexpr long GROUPED_KS4_BELOW = 96;
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
 // 256-column tile); blocks beyond the live count exit at once.  When that grid
 // would leave compute units idle (max_blocks is the caller's bound for this
@@ -1825,13 +1830,15 @@ constexpr long GROUPED_KSPLIT_BELOW = 96;
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     if (g.w_int4) return RKH_ERR_RUNTIME;
     const int mblocks = g.max_blocks;
-    const bool ksplit = (long)mblocks * ((g.N + 255) / 256) < GROUPED_KSPLIT_BELOW;
-    const int nblocks = ksplit ? (g.N + 63) / 64 : (g.N + 255) / 256;
+    const long wide = (long)mblocks * ((g.N + 255) / 256);
+    const int ks = wide < GROUPED_KS4_BELOW ? 4 : 1;
+    const int cols = 256 / ks;
+    const int nblocks = (g.N + cols - 1) / cols;
     const dim3 grid(mblocks * nblocks), block(256);
-#define RK_LAUNCH(EPI)                                                                                        \
-    do {                                                                                                      \
-        if (ksplit) hipLaunchKernelGGL((gemm_stream_kernel<EPI, true>), grid, block, 0, st, g, mblocks, nblocks); \
-        else hipLaunchKernelGGL((gemm_stream_kernel<EPI, false>), grid, block, 0, st, g, mblocks, nblocks);   \
+#define RK_LAUNCH(EPI)                                                                                         \
+    do {                                                                                                       \
+        if (ks == 4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4>), grid, block, 0, st, g, mblocks, nblocks); \
+        else hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1>), grid, block, 0, st, g, mblocks, nblocks);        \
     } while (0)
     switch (g.epilogue) {
     case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
