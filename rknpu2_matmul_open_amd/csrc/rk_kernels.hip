@@ -1433,13 +1433,18 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // KS waves share a column pair, taking 1/KS of K each; their accumulators are
 // added through LDS before the first of them runs the epilogue -- KS times as
 // many workgroups.
-template <int EPI, int KS>
+// W4 (dense int4 weights only): a step is one 64-deep super-tile -- two
+// activation tiles and 1 KiB of packed weights per column block, unpacked in
+// registers into the two operands (every code times 16, undone by one shift of
+// the accumulators, so K may not exceed 2^17).
+template <int EPI, int KS, bool W4>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
     constexpr int TN = 2, WAVES = 4;
     constexpr bool KSPLIT = KS > 1;
     constexpr int CG = WAVES / KS; // column pairs per workgroup
     constexpr int RING = 8; // (16 with K split four ways, a wave's whole share in flight, was measured slower)
-    constexpr int LPS = 1 + TN;
+    constexpr int AT = W4 ? 2 : 1;   // activation tiles per step
+    constexpr int LPS = AT + TN;
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
     constexpr int STAGE_BYTES = WAVES * 32 * (32 * 4 + 8);
     constexpr int XCH_BYTES = KSPLIT ? CG * (KS - 1) * TN * 16 * 64 * 4 : 0;
@@ -1447,7 +1452,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
-    const int KB = (int)rkh_align_up(g.K, RKH_K_ALIGN) / 32; // k-tiles: a multiple of 8 = RING
+    // steps over K: k-tiles (a multiple of 8 = RING) or, for int4 weights, super-tiles (a multiple of 4)
+    const int KB = (int)rkh_align_up(g.K, RKH_K_ALIGN) / (32 * AT);
 
     const int logical = xcd_remap(blockIdx.x, mblocks * nblocks);
     const int mblk = logical % mblocks, nblk = logical / mblocks;
@@ -1464,7 +1470,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     const int share = (KB + KS - 1) / KS;
     const int kts = max(0, min(share, KB - kq * share));
     const int kt0 = min(kq * share, KB - 1); // (a wave without a share still loads in bounds)
-    const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * 1024;
+    const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * (1024 * AT);
     const uint8_t* wsrc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) wsrc[j] = Wb + ((size_t)(pb0 + j) * KB + kt0) * 1024;
@@ -1476,19 +1482,19 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[j][r] = 0;
-    v4i ring[RING][LPS]; // [0] = activations, [1 + j] = weights of column block j
+    v4i ring[RING][LPS]; // [0 .. AT) = activation tiles, [AT + j] = weights of column block j
 
     auto issue = [&](v4i* regs) {
         static_for<LPS>([&](auto l_tag) {
             constexpr int L = decltype(l_tag)::value;
             const unsigned off = lane_off; // (locals: asm operands cannot name captures of an enclosing lambda)
-            const uint8_t* base = L == 0 ? asrc : wsrc[L == 0 ? 0 : L - 1];
+            const uint8_t* base = L < AT ? asrc + L * 1024 : wsrc[L < AT ? 0 : L - AT];
             v4i r;
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
             regs[L] = r;
         });
         const int step = left > 0 ? 1024 : 0;
-        asrc += step;
+        asrc += step * AT;
 #pragma unroll
         for (int j = 0; j < TN; ++j) wsrc[j] += step;
         --left;
@@ -1507,10 +1513,21 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
             issue(ring[(SLOT + RING - 1) % RING]);
             wait(ring[SLOT]);
             // (a K share need not be a multiple of RING: the steps past its end reload the last tile and are skipped)
-            if (!KSPLIT || s + SLOT < kts) {
+            if ((!KSPLIT && !W4) || s + SLOT < kts) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][1 + j], ring[SLOT][0], acc[j], 0, 0, 0);
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (W4) {
+                        const v4i raw = ring[SLOT][AT + j];
+                        const v4i lo = v4i{(raw.x << 4) & (int)0xF0F0F0F0, raw.x & (int)0xF0F0F0F0,
+                                           (raw.y << 4) & (int)0xF0F0F0F0, raw.y & (int)0xF0F0F0F0};
+                        const v4i hi = v4i{(raw.z << 4) & (int)0xF0F0F0F0, raw.z & (int)0xF0F0F0F0,
+                                           (raw.w << 4) & (int)0xF0F0F0F0, raw.w & (int)0xF0F0F0F0};
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, ring[SLOT][0], acc[j], 0, 0, 0);
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, ring[SLOT][AT - 1], acc[j], 0, 0, 0);
+                    } else {
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][AT + j], ring[SLOT][0], acc[j], 0, 0, 0);
+                    }
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -1549,6 +1566,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
                     acc[j][q * 4 + 2] += got.z;
                     acc[j][q * 4 + 3] += got.w;
                 }
+    }
+    if constexpr (W4) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[j][r] >>= 4;
     }
     const int m_limit = g.blk_expert ? live_blocks * 32 : g.M;
     uint8_t* stage_lds = stage_raw + wave * (32 * (32 * 4 + 8));
@@ -1824,23 +1847,30 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 // (Splitting K two ways over 128-column tiles for 4 .. 64 tokens was measured too: 1 - 3 us slower than
 // the wide tile at every size.)
 constexpr long GROUPED_KS4_BELOW = 96;
+constexpr long DENSE_KS4_BELOW = 128; // dense use of the same kernel: every row block is live
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
 // 256-column tile); blocks beyond the live count exit at once.  When that grid
 // would leave compute units idle (max_blocks is the caller's bound for this
 // call, a handful for a decode step) the tile shrinks to 64 columns and the
 // waves split K instead.
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
-    if (g.w_int4) return RKH_ERR_RUNTIME;
+    if (g.w_int4 && (g.blk_expert || g.K > 131072)) return RKH_ERR_RUNTIME;
     const int mblocks = g.blk_expert ? g.max_blocks : (g.M + 31) / 32;
     const long wide = (long)mblocks * ((g.N + 255) / 256);
-    const int ks = wide < GROUPED_KS4_BELOW ? 4 : 1;
+    const int ks = wide < (g.blk_expert ? GROUPED_KS4_BELOW : DENSE_KS4_BELOW) ? 4 : 1;
     const int cols = 256 / ks;
     const int nblocks = (g.N + cols - 1) / cols;
     const dim3 grid(mblocks * nblocks), block(256);
 #define RK_LAUNCH(EPI)                                                                                         \
     do {                                                                                                       \
-        if (ks == 4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4>), grid, block, 0, st, g, mblocks, nblocks); \
-        else hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1>), grid, block, 0, st, g, mblocks, nblocks);        \
+        if (g.w_int4 && ks == 4)                                                                               \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true>), grid, block, 0, st, g, mblocks, nblocks);   \
+        else if (g.w_int4)                                                                                     \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true>), grid, block, 0, st, g, mblocks, nblocks);   \
+        else if (ks == 4)                                                                                      \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, false>), grid, block, 0, st, g, mblocks, nblocks);  \
+        else                                                                                                   \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false>), grid, block, 0, st, g, mblocks, nblocks);  \
     } while (0)
     switch (g.epilogue) {
     case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
@@ -2167,17 +2197,24 @@ static DensePlan effective_plan(int M, int N, int K, int w_int4) {
     return plan;
 }
 
-// A dense int8 GEMM of up to four row blocks is a weight stream like a MoE
-// expert's: it runs on the grouped kernel (one "expert"; for few column tiles K
-// is split over the waves of a workgroup and summed through LDS) instead of
-// splitting K over workgroups and finishing in a second launch.  Measured
-// against the large-tile kernel with fp16 in / out, quantization included:
-// M 64, 2048 x 2048: 10.2 vs 15.3 us; M 128, 4096 x 4096: 12.6 vs 20.2 us; M 128, K 14336, N 4096: 25.5 vs
-// 28.9 us; M 128, K 4096, N 14336: 20.9 vs 20.9 us.  From about 160 rows on the large tile wins for wide N
-// (each row block streams the weights again).
-constexpr int DENSE_STREAM_MAX_M = 128;
+// A dense GEMM of up to four row blocks is a weight stream like a MoE expert's:
+// it runs on the grouped kernel (one "expert"; for few column tiles K is split
+// over the waves of a workgroup and summed through LDS) instead of splitting K
+// over workgroups and finishing in a second launch.  Measured against the
+// large-tile kernel, fp16 in / out, quantization included (us):
+//   int8  M 64, 2048 x 2048: 10.2 vs 15.3   M 128, 4096 x 4096: 12.6 vs 20.2   M 128, K 14336, N 4096: 25.5 vs 28.9
+//         M 128, K 4096, N 14336: 20.9 vs 20.9
+//   int4  M 64, 2048 x 2048:  9.9 vs 14.1   M 128, 4096 x 4096: 11.9 vs 19.4   M 128, K 14336, N 4096: 22.2 vs 25.7
+//         M 32, K 4096, N 14336: 11.4 vs 18.4
+// From about 160 rows on the large tile wins for wide N (each row block streams
+// the weights again).  The same holds earlier for the gate/up + SwiGLU GEMM of
+// an FFN, whose N is twice as wide: the whole FFN (4096 -> 14336 -> 4096, weights
+// from HBM) takes 47.4 vs 53.9 us at 16 rows, 49.4 vs 47.0 at 64, 63.0 vs 56.3 at 128.
+constexpr int DENSE_STREAM_MAX_M = 128, DENSE_STREAM_SWIGLU_MAX_M = 32;
 static bool dense_streams(const rkh_gemm_args& g) {
-    return !g.w_int4 && !g.blk_expert && g.M > 8 && g.M <= DENSE_STREAM_MAX_M && g.epilogue != RKH_EPI_SWIGLU;
+    if (g.blk_expert || g.M <= 8 || g.M > DENSE_STREAM_MAX_M) return false;
+    if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
+    return !g.w_int4 || g.K <= 131072;
 }
 
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
