@@ -29,6 +29,9 @@ def _bits32(x):
 
 SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), (9, 200, 96),
           (40, 130, 257), (64, 256, 1024), (100, 320, 640), (130, 1000, 300),
+          # weight-streaming kernel without the in-workgroup K split (>= 128 column tiles x row blocks),
+          # K a single / an odd number of 64-deep super-tiles
+          (70, 11000, 192), (33, 33000, 40),
           # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
           (650, 6900, 1000), (641, 6912, 200)]
 
@@ -147,6 +150,7 @@ def test_w4a8_rejections(sess):
 
 SWIGLU_SHAPES = [(1, 64, 64), (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
                  (128, 1024, 512),
+                 (20, 32896, 128), (32, 2048, 700),  # weight-streaming kernel: wide grid / K split inside the workgroup
                  (650, 6912, 520), (641, 7040, 300)]  # large-tile kernel (F a multiple of 64 / only of 32)
 
 

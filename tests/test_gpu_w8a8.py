@@ -21,6 +21,8 @@ def _rand_i8(rng, shape, lo=-127, hi=127):
 I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96), (17, 40, 33),
               (33, 130, 70), (64, 256, 256), (65, 257, 129), (128, 512, 384), (300, 48, 33),
               (200, 1000, 520),
+              # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
+              (100, 8448, 160), (128, 96, 3000),
               # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
               (641, 6900, 200), (700, 6900, 1100)]
 
