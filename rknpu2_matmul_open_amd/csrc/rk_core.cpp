@@ -75,22 +75,68 @@ double StageTimer::span_us(int from, int to) {
     return us;
 }
 
-HostStage::~HostStage() { rkh_host_free(ptr_); }
+HostStage::~HostStage() {
+    for (void* e : events_) rkh_event_destroy(e);
+    rkh_host_free(ptr_);
+}
 void HostStage::init(size_t bytes) {
-    if (!bytes || bytes > kLimit) return;
+    if (!bytes || bytes > kPipeLimit) return;
     void* p = nullptr;
-    if (rkh_host_alloc(&p, bytes) == RKH_OK) {
-        ptr_ = p;
-        bytes_ = bytes;
+    if (rkh_host_alloc(&p, bytes) != RKH_OK) return;
+    ptr_ = p;
+    bytes_ = bytes;
+    if (bytes > kLimit) {
+        const size_t chunks = (bytes + kChunk - 1) / kChunk;
+        for (size_t i = 0; i < chunks; ++i) {
+            void* e = nullptr;
+            if (rkh_event_create(&e) != RKH_OK) { // without its events the mirror only serves uploads
+                for (void* made : events_) rkh_event_destroy(made);
+                events_.clear();
+                break;
+            }
+            events_.push_back(e);
+        }
     }
 }
-void HostStage::init_capped(size_t bytes) { init(bytes < kLimit ? bytes : kLimit); }
 const void* HostStage::fill(const void* user, size_t bytes) const {
     std::memcpy(ptr_, user, bytes <= bytes_ ? bytes : bytes_);
     return ptr_;
 }
 void HostStage::finish(void* user, size_t bytes) const {
     if (ptr_ && bytes <= bytes_) std::memcpy(user, ptr_, bytes);
+}
+int HostStage::upload(void* stream, void* device, const void* user, size_t bytes) const {
+    if (!ptr_ || bytes > bytes_) return rkh_h2d(stream, device, user, bytes);
+    for (size_t off = 0; off < bytes; off += kChunk) {
+        const size_t n = bytes - off < kChunk ? bytes - off : kChunk;
+        std::memcpy(static_cast<uint8_t*>(ptr_) + off, static_cast<const uint8_t*>(user) + off, n);
+        const int rc = rkh_h2d(stream, static_cast<uint8_t*>(device) + off, static_cast<uint8_t*>(ptr_) + off, n);
+        if (rc) return rc;
+    }
+    return RKH_OK;
+}
+int HostStage::download(void* stream, void* user, const void* device, size_t bytes) {
+    staged_ = ptr_ && bytes <= bytes_ && events_.size() * kChunk >= bytes;
+    if (!staged_) return rkh_d2h(stream, user, device, bytes);
+    size_t i = 0;
+    for (size_t off = 0; off < bytes; off += kChunk, ++i) {
+        const size_t n = bytes - off < kChunk ? bytes - off : kChunk;
+        int rc = rkh_d2h(stream, static_cast<uint8_t*>(ptr_) + off, static_cast<const uint8_t*>(device) + off, n);
+        if (!rc) rc = rkh_event_record(events_[i], stream);
+        if (rc) return rc;
+    }
+    return RKH_OK;
+}
+int HostStage::finish_download(void* stream, void* user, size_t bytes) {
+    if (!staged_) return rkh_sync(stream);
+    size_t i = 0;
+    for (size_t off = 0; off < bytes; off += kChunk, ++i) {
+        const size_t n = bytes - off < kChunk ? bytes - off : kChunk;
+        const int rc = rkh_event_sync(events_[i]);
+        if (rc) return rc;
+        std::memcpy(static_cast<uint8_t*>(user) + off, static_cast<uint8_t*>(ptr_) + off, n);
+    }
+    return RKH_OK;
 }
 
 BadFlag::~BadFlag() { rkh_host_free(host_); }

@@ -86,6 +86,7 @@ void rkh_fail_malloc_after(int n);
 int rkh_event_create(void** event);
 void rkh_event_destroy(void* event);
 int rkh_event_record(void* event, void* stream);
+int rkh_event_sync(void* event);                                /* blocks until the event has happened */
 int rkh_event_elapsed_us(void* start, void* stop, double* us); /* waits for stop */
 
 /* ---- weight re-tiling at upload ---- */

@@ -88,8 +88,8 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
             rk_npu_i4_timings* t) {
     const rk_npu_i4_config& c = ws->config;
     rk_npu_ctx* ctx = ws->owner.ctx;
-    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
     const size_t c_bytes = (size_t)c.M * c.N * sizeof(int32_t);
+    const bool direct_in = ws->stage_a.direct((size_t)c.M * c.K), direct_out = ws->stage_c.direct(c_bytes);
     int rc;
     auto start = Clock::now();
     {
@@ -102,7 +102,7 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
             q.src_is_host = 1;
             rc = RK_NPU_OK;
         } else {
-            rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), codes, a_bytes));
+            rc = map_error(ws->stage_a.upload(ctx->stream, ws->a_raw.as<>(), codes, a_bytes));
         }
         q.in_dtype = RKH_I8;
         q.mode = RKH_Q_COPY_I8;
@@ -127,9 +127,9 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
         t->sync_us += elapsed_us(start);
         start = Clock::now();
         if (!rc && direct_out) ws->stage_c.finish(C, c_bytes);
-        else if (!rc) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
+        else if (!rc) rc = map_error(ws->stage_c.download(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }
-    const int wait = direct_out ? RK_NPU_OK : map_error(rkh_sync(ctx->stream));
+    const int wait = direct_out || rc ? RK_NPU_OK : map_error(ws->stage_c.finish_download(ctx->stream, C, c_bytes));
     t->reduce_us += elapsed_us(start);
     return rc ? rc : wait;
 }

@@ -2086,6 +2086,10 @@ int rkh_event_record(void* event, void* stream) {
     RKH_CHECK(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
     return RKH_OK;
 }
+int rkh_event_sync(void* event) {
+    RKH_CHECK(hipEventSynchronize((hipEvent_t)event));
+    return RKH_OK;
+}
 int rkh_event_elapsed_us(void* start, void* stop, double* us) {
     RKH_CHECK(hipEventSynchronize((hipEvent_t)stop));
     float ms = 0.0f;

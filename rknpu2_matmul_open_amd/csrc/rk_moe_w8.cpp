@@ -284,7 +284,7 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     // The routing table is read by every token's workgroup: in place only for a
     // decode-sized call, otherwise uploaded (from its mirror, without a wait).
     const size_t in_bytes = values * (f32 ? 4 : 1), out_bytes = values * 4;
-    const bool direct_in = ws->stage_in.fits(in_bytes), direct_out = ws->stage_out.fits(out_bytes);
+    const bool direct_in = ws->stage_in.direct(in_bytes), direct_out = ws->stage_out.direct(out_bytes);
     const bool direct_route = ws->stage_route && rows <= 16;
     const void* d_input = ws->input.as<>();
     const float* d_scales = ws->token_scale.as<float>();
@@ -305,7 +305,7 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     }
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->input.as<>(), input, in_bytes));
+        if (!direct_in) rc = map_error(ws->stage_in.upload(ctx->stream, ws->input.as<>(), input, in_bytes));
         if (direct_route) {
             d_ids = static_cast<const int32_t*>(h_ids);
             d_routes = static_cast<const float*>(h_routes);
@@ -328,8 +328,8 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     if (direct_out) {
         ws->stage_out.finish(output, out_bytes);
     } else {
-        rc = map_error(rkh_d2h(ctx->stream, output, ws->out.as<>(), out_bytes));
-        if (!rc) rc = map_error(rkh_sync(ctx->stream));
+        rc = map_error(ws->stage_out.download(ctx->stream, output, ws->out.as<>(), out_bytes));
+        if (!rc) rc = map_error(ws->stage_out.finish_download(ctx->stream, output, out_bytes));
     }
     if (timings) {
         timings->schedule_us = timer.span_us(0, 1);
@@ -495,8 +495,8 @@ rk_npu_moe_w8_workspace* create_workspace(rk_npu_iommu_domain* domain, const rk_
         ws->h_scale.alloc(ws->owner, S * 4) || ws->y.alloc(ws->owner, S * H * 4) ||
         ws->out.alloc(ws->owner, (size_t)R * H * 4, false) || ws->flag.init(ws->owner))
         return nullptr;
-    ws->stage_in.init_capped((size_t)R * H * 4);
-    ws->stage_out.init_capped((size_t)R * H * 4);
+    ws->stage_in.init((size_t)R * H * 4);
+    ws->stage_out.init((size_t)R * H * 4);
     ws->stage_route.init((size_t)routed * 8 + (size_t)R * 4);
     if (rkh_sync(domain->ctx->stream)) return nullptr;
     return ws.release();

@@ -189,7 +189,7 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
     // Small operands skip the copies: the kernels read A from / write C into the
     // pinned mirrors.  Static scales are read by every workgroup of the GEMM, so
     // they are always uploaded (from their mirror when there is one).
-    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
+    const bool direct_in = ws->stage_a.direct(a_bytes), direct_out = ws->stage_c.direct(c_bytes);
     const size_t scale_bytes = (size_t)s.M * sizeof(float);
     // the mirrors are filled before the context's submission lock is taken
     const void* src = direct_in ? ws->stage_a.fill(A, a_bytes) : ws->a_raw.as<>();
@@ -197,15 +197,18 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
     if (ws->t.quant == 2 && ws->stage_scale) scale_src = ws->stage_scale.fill(a_scale, scale_bytes);
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(ws->stage_a.upload(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         if (!rc && ws->t.quant == 2)
             rc = map_error(rkh_h2d(ctx->stream, ws->a_scale.as<>(), scale_src, scale_bytes));
         if (!rc) rc = enqueue(ws, *w, src, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), direct_in);
-        if (!rc && !direct_out) rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
+        if (!rc && !direct_out) rc = map_error(ws->stage_c.download(ctx->stream, C, ws->c_out.as<>(), c_bytes));
     }
-    const int wait = map_error(rkh_sync(ctx->stream));
-    if (!rc && !wait && direct_out) ws->stage_c.finish(C, c_bytes);
-    return rc ? rc : wait;
+    if (rc || direct_out) {
+        const int wait = map_error(rkh_sync(ctx->stream));
+        if (!rc && !wait) ws->stage_c.finish(C, c_bytes);
+        return rc ? rc : wait;
+    }
+    return map_error(ws->stage_c.finish_download(ctx->stream, C, c_bytes));
 }
 
 int run_device(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kind kind,

@@ -370,11 +370,11 @@ int run_host(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void
     StageTimer timer(ctx->stream, timings != nullptr);
     // Small operands skip the copies: the kernels read A from / write the result
     // into the pinned mirrors (the caller's C is only written after the checks).
-    const bool direct_in = (bool)ws->stage_a, direct_out = (bool)ws->stage_c;
+    const bool direct_in = ws->stage_a.direct(a_bytes), direct_out = ws->stage_c.direct(c_bytes);
     const void* src = direct_in ? ws->stage_a.fill(A, a_bytes) : ws->a_raw.as<>(); // before the submission lock
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(ws->stage_a.upload(ctx->stream, ws->a_raw.as<>(), A, a_bytes));
         timer.mark();
         if (!rc)
             rc = enqueue(ws, w, src, half, direct_out ? ws->stage_c.data() : ws->c_out.as<>(), out, false, nullptr,
@@ -395,8 +395,8 @@ int run_host(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w, const void
     if (direct_out) {
         ws->stage_c.finish(C, c_bytes);
     } else {
-        rc = map_error(rkh_d2h(ctx->stream, C, ws->c_out.as<>(), c_bytes));
-        if (!rc) rc = map_error(rkh_sync(ctx->stream));
+        rc = map_error(ws->stage_c.download(ctx->stream, C, ws->c_out.as<>(), c_bytes));
+        if (!rc) rc = map_error(ws->stage_c.finish_download(ctx->stream, C, c_bytes));
     }
     fill_timings(timings, timer, 0, true, elapsed_us(t1), elapsed_us(t0));
     return rc;
@@ -684,12 +684,13 @@ int rk_npu_w4a8_run_ffn_f32(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights
     rk_npu_ctx* ctx = gu->owner.ctx;
     const int M = gu->config.M, F = gu->config.N / 2;
     const size_t a_bytes = (size_t)M * gu->config.K * 4, c_bytes = (size_t)M * dn->config.N * 4;
-    const bool direct_in = (bool)gu->stage_a, direct_out = dn->stage_c && dn->config.M == M;
+    const size_t mid_bytes = (size_t)M * F * 4;
+    const bool direct_in = gu->stage_a.direct(a_bytes), direct_out = dn->stage_c.direct(c_bytes);
     StageTimer timer(ctx->stream, metrics != nullptr);
     const void* src = direct_in ? gu->stage_a.fill(A, a_bytes) : gu->a_raw.as<>(); // before the submission lock
     {
         std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-        if (!direct_in) rc = map_error(rkh_h2d(ctx->stream, gu->a_raw.as<>(), A, a_bytes));
+        if (!direct_in) rc = map_error(gu->stage_a.upload(ctx->stream, gu->a_raw.as<>(), A, a_bytes));
         timer.mark();                                                                        // 0
         // middle lives in the gate/up workspace's result buffer (on the device: the
         // re-quantization reads it back)
@@ -706,9 +707,11 @@ int rk_npu_w4a8_run_ffn_f32(rk_npu_w4a8_workspace* gu, const rk_npu_w4a8_weights
     const bool bad_mid = dn->flag.consume(ctx->stream);
     if (bad_in || bad_mid) return RK_NPU_ERR_PARAM; // NaN/Inf input or non-finite middle
     const auto t1 = Clock::now();
-    rc = map_error(rkh_d2h(ctx->stream, middle, gu->c_out.as<>(), (size_t)M * F * 4));
-    if (!rc && !direct_out) rc = map_error(rkh_d2h(ctx->stream, C, dn->c_out.as<>(), c_bytes));
-    if (!rc) rc = map_error(rkh_sync(ctx->stream));
+    // the middle goes through the gate/up workspace's output mirror (unused by the kernels in this call)
+    rc = map_error(gu->stage_c.download(ctx->stream, middle, gu->c_out.as<>(), mid_bytes));
+    if (!rc && !direct_out) rc = map_error(dn->stage_c.download(ctx->stream, C, dn->c_out.as<>(), c_bytes));
+    if (!rc) rc = map_error(gu->stage_c.finish_download(ctx->stream, middle, mid_bytes));
+    if (!rc && !direct_out) rc = map_error(dn->stage_c.finish_download(ctx->stream, C, c_bytes));
     if (!rc && direct_out) dn->stage_c.finish(C, c_bytes);
     if (metrics) {
         const double copy = elapsed_us(t1);
