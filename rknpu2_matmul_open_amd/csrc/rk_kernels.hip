@@ -134,6 +134,33 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
 
 template <typename T> struct RowLoader;
 template <> struct RowLoader<uint16_t> {
+    // The 16 elements as they lie in memory (elements beyond K read as zero), so
+    // that a caller can put other loads between fetching and converting them.
+    struct Raw { uint32_t w[8]; };
+    static __device__ __forceinline__ Raw load16_raw(const uint16_t* row, int k0, int K, bool vec) {
+        Raw r;
+        if (vec && k0 + 16 <= K) {
+            const uint4 a = *reinterpret_cast<const uint4*>(row + k0);
+            const uint4 b = *reinterpret_cast<const uint4*>(row + k0 + 8);
+            r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
+            r.w[4] = b.x; r.w[5] = b.y; r.w[6] = b.z; r.w[7] = b.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t lo = k0 + 2 * j < K ? row[k0 + 2 * j] : 0u;
+                const uint32_t hi = k0 + 2 * j + 1 < K ? row[k0 + 2 * j + 1] : 0u;
+                r.w[j] = lo | (hi << 16);
+            }
+        }
+        return r;
+    }
+    static __device__ __forceinline__ void unpack(const Raw& r, float* out) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            out[2 * j] = half_bits_to_float((uint16_t)(r.w[j] & 0xffffu));
+            out[2 * j + 1] = half_bits_to_float((uint16_t)(r.w[j] >> 16));
+        }
+    }
     static __device__ __forceinline__ void load16(const uint16_t* row, int k0, int K, bool vec,
                                                   float* out) {
         if (vec && k0 + 16 <= K) {
@@ -152,6 +179,16 @@ template <> struct RowLoader<uint16_t> {
     }
 };
 template <> struct RowLoader<float> {
+    struct Raw { float v[16]; };
+    static __device__ __forceinline__ Raw load16_raw(const float* row, int k0, int K, bool vec) {
+        Raw r;
+        load16(row, k0, K, vec, r.v);
+        return r;
+    }
+    static __device__ __forceinline__ void unpack(const Raw& r, float* out) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) out[j] = r.v[j];
+    }
     static __device__ __forceinline__ void load16(const float* row, int k0, int K, bool vec,
                                                   float* out) {
         if (vec && k0 + 16 <= K) {
@@ -574,8 +611,13 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 //     workgroup quantizes the few rows itself -- they are L2 hits after the first
 //     -- which saves a kernel launch per decode step; workgroup 0 also writes the
 //     scales and the tiled int8 copy that the two-kernel path would have left).
+// Two workgroups must fit a compute unit (a grid of a few hundred workgroups
+// otherwise runs in two rounds), i.e. four waves per SIMD and at most 128
+// vector registers: stated as a requirement, because the int4 variants with the
+// fused quantization would otherwise be allocated more.
 template <int MR, bool W4, int QT>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
+__global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
+void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
     __shared__ uint32_t row_max[MR];
@@ -595,8 +637,26 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
 
     // Fused path: put the first batch of weight loads in flight before the
     // quantization prologue so that its latency hides behind them.
+    // The activation rows are requested FIRST: loads return in issue order, so
+    // behind the weight loads they would arrive with the last of those, and the
+    // prologue (and with it the second batch of weight loads) would start only
+    // then.  Fetched first they are back after one L2 round trip and the whole
+    // quantization runs under the weight loads' latency.
     v4i wpre[GEMV_UNROLL];
+    using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
+    typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
     if constexpr (QT != 0) {
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = (int)threadIdx.x + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const QT_T* row = static_cast<const QT_T*>(q.src) + (size_t)m * K;
+                araw[i] = RowLoader<QT_T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         const int tiles = W4 ? Kp >> 6 : Kp >> 5;
 #pragma unroll
         for (int u = 0; u < GEMV_UNROLL; ++u) {
@@ -605,27 +665,30 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
                                        wbase + (size_t)tt * 1024 + lane * 16))
                                  : v4i{0, 0, 0, 0};
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (QT != 0) {
-        using T = typename std::conditional<QT == 1, uint16_t, float>::type;
+        using T = QT_T;
         const int t = threadIdx.x;
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
         if (t < MR) row_max[t] = 0u;
         __syncthreads();
-        float v[GEMV_QCHUNKS][16];
+        // (the rows stay in registers as fetched and are converted once per pass:
+        // holding them as floats across the barriers costs the int4 variants their
+        // second workgroup per compute unit)
         bool bad = false;
 #pragma unroll
         for (int i = 0; i < GEMV_QCHUNKS; ++i) {
             const int pidx = t + i * GEMV_WAVES * 64;
             if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                const T* row = static_cast<const T*>(q.src) + (size_t)m * K;
-                RowLoader<T>::load16(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0, v[i]);
+                const int m = pidx / nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
                 float mx = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
-                    mx = fmaxf(mx, fabsf(v[i][j]));
-                    bad |= not_finite(v[i][j]);
+                    mx = fmaxf(mx, fabsf(v[j]));
+                    bad |= not_finite(v[j]);
                 }
                 atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
             }
@@ -650,7 +713,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
             const int pidx = t + i * GEMV_WAVES * 64;
             if (pidx < total) {
                 const int m = pidx / nchunks, c = pidx - m * nchunks;
-                const uint4 packed = quantize16<false>(v[i], 1.0f / row_scale[m]);
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
                 if (p == 0 && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
             }
@@ -672,77 +737,69 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
         }
         __syncthreads();
 
-        if (!W4) {
-            const int tiles = kc >> 5, tile0 = kc0 >> 5;
-            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
-                v4i w[GEMV_UNROLL];
+        // One group = GEMV_UNROLL tiles per wave.  Int4: a tile is a 64-deep super-tile.
+        const int tiles = W4 ? kc >> 6 : kc >> 5, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
+        auto fetch = [&](v4i* w, int tb) {
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) {
-                    const int tt = tb + u * GEMV_WAVES;
-                    if (QT != 0 && tb == wave) {
-                        w[u] = wpre[u];
-                    } else {
-                        w[u] = tt < tiles
-                                   ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                         wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
-                                   : v4i{0, 0, 0, 0};
+            for (int u = 0; u < GEMV_UNROLL; ++u) {
+                const int tt = tb + u * GEMV_WAVES;
+                w[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                        wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
+                                  : v4i{0, 0, 0, 0};
+            }
+        };
+        auto consume = [&](const v4i* w, int tb) {
+#pragma unroll
+            for (int u = 0; u < GEMV_UNROLL; ++u) {
+                const int tt = tb + u * GEMV_WAVES;
+                if (tt >= tiles) continue;
+                if constexpr (!W4) {
+#pragma unroll
+                    for (int m = 0; m < MR; ++m) {
+                        const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                        acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
                     }
-                }
+                } else {
+                    // The words pass through an empty asm statement so that their unpacking
+                    // stays here: moved up to where the prefetched group arrived (the compiler
+                    // does that) the sixteen operand words per tile of all eight tiles are live
+                    // across the prologue, more registers than two workgroups per compute unit leave.
+                    int wv[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) {
-                    const int tt = tb + u * GEMV_WAVES;
-                    if (tt < tiles) {
+                    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(wv[i]));
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {       // the two 32-k halves
+                        const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
+                        const int hi0 = wv[2 * s] & 0xF0F0F0F0;
+                        const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
+                        const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
 #pragma unroll
                         for (int m = 0; m < MR; ++m) {
-                            const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
-                            acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
+                            const v4i av = *reinterpret_cast<const v4i*>(
+                                a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                            acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
                         }
                     }
                 }
             }
-        } else {
-            const int tiles = kc >> 6, tile0 = kc0 >> 6; // super-tiles of 64 k
-            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
-                v4i w[GEMV_UNROLL];
-#pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) {
-                    const int tt = tb + u * GEMV_WAVES;
-                    if (QT != 0 && tb == wave) {
-                        w[u] = wpre[u];
-                    } else {
-                        w[u] = tt < tiles
-                                   ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                         wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
-                                   : v4i{0, 0, 0, 0};
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) {
-                    const int tt = tb + u * GEMV_WAVES;
-                    if (tt < tiles) {
-                        const int wv[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
-#pragma unroll
-                        for (int s = 0; s < 2; ++s) {       // the two 32-k halves
-                            const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
-                            const int hi0 = wv[2 * s] & 0xF0F0F0F0;
-                            const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
-                            const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
-#pragma unroll
-                            for (int m = 0; m < MR; ++m) {
-                                const v4i av = *reinterpret_cast<const v4i*>(
-                                    a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
-                                acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
-                                acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
-                                acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
-                                acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
-                            }
-                        }
-                    }
-                }
-            }
+        };
+        int tb = wave;
+        if constexpr (QT != 0) { // the group fetched ahead of the prologue (the fused path has a single K chunk)
+            consume(wpre, tb);
+            tb += GEMV_WAVES * GEMV_UNROLL;
+        }
+        for (; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+            v4i w[GEMV_UNROLL];
+            fetch(w, tb);
+            consume(w, tb);
+        }
+        if constexpr (W4) {
             // int4 operands are carried as 16 * code; fold each K chunk's exact
             // multiple-of-16 partial back so very long K cannot overflow int32.
 #pragma unroll
@@ -760,9 +817,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(rkh_gemm_args g, 
         if (lane < 32) red[wave][m][lane] = v;
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < MR * 32; idx += GEMV_WAVES * 64) {
-        const int m = idx >> 5, j = idx & 31;
-        if (m >= g.M) continue;
+    static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
+    if ((int)threadIdx.x < MR * 32) {
+        const int m = (int)threadIdx.x >> 5, j = (int)threadIdx.x & 31;
+        if (m >= g.M) return;
         int sum = 0;
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
