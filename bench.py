@@ -174,6 +174,44 @@ def bench_c2(sess, ops, capi, workloads, steps, warmup):
     return out
 
 
+def bench_c1w4(sess, ops, capi, workloads, steps, warmup):
+    """w4a8 decode GEMV at config 1's shape (M=1, K=4096, N=14336), int4 weights."""
+    M, K, N = 1, 4096, 14336
+    c = workloads.w4a8_case(M, K, N, seed_w=2, seed_a=3)
+    # as in bench_c1: the loop walks over several copies so that every step streams from HBM
+    # (16 copies of 29.4 MB = 470 MB)
+    copies = [ops.W4A8Weights(sess, c["B"], c["w_scale"]) for _ in range(2 * C1_COPIES)]
+    ws = ops.W4A8Workspace(sess, M, N, K)
+    dA = sess.to_device(c["A"])
+    dC = sess.empty_device(M * N * 2)
+    lib = sess.lib
+    turn = [0]
+
+    def step():
+        w = copies[turn[0] % len(copies)]
+        turn[0] += 1
+        rc = lib.rk_npu_w4a8_run_f16_device(ws.h, w.h, dA, dC)
+        if rc:
+            raise RuntimeError("run_device rc=%d" % rc)
+
+    sess.spin_up(step)
+    step_us = sess.time_us(step, steps, warmup)
+    weight_bytes = K * N // 2
+    algo_bytes = weight_bytes + K * 2 + N * 2 + N * 4
+    out = {"workload": "w4a8 decode GEMV M=1 K=4096 N=14336 (int4 weights, 29360128 B), fp16 in/out, seeds 2/3",
+           "weight_GBps": weight_bytes / step_us / 1e3, "ms_per_step": step_us / 1e3,
+           "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,true,1> (fused per-token quantize + int4 GEMV)",
+                        "achieved": algo_bytes / step_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": algo_bytes / step_us / 1e3 / HBM_PEAK_GBS, "kernel_us": step_us,
+                        "algorithmic_bytes": algo_bytes, "traffic": None}}
+    sess.free_device(dA)
+    sess.free_device(dC)
+    ws.close()
+    for w in copies:
+        w.close()
+    return out
+
+
 def bench_c2w8(sess, ops, capi, workloads, steps, warmup):
     """w8a8 prefill GEMM at the same shape as config 2 (M=2048, K=4096, N=4096), int8 weights."""
     M, K, N = 2048, 4096, 4096
@@ -305,7 +343,7 @@ def main():
     ap.add_argument("--workload", default="c1", choices=["c1", "all"],
                     help="c1: headline line (+ c2 TOPS); all: also time configs 0, 3 and 4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default=None, choices=["c0", "c1", "c2", "c2w8", "c3", "c4", "copy"],
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c1w4", "c2", "c2w8", "c3", "c4", "copy"],
                     help="profiling aid: run one configuration's loop only")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -323,7 +361,7 @@ def main():
         sess.close()
         return
     if args.only:
-        fn = {"c0": bench_c0, "c2": bench_c2, "c2w8": bench_c2w8, "c3": bench_c3, "c4": bench_c4}.get(args.only)
+        fn = {"c0": bench_c0, "c1w4": bench_c1w4, "c2": bench_c2, "c2w8": bench_c2w8, "c3": bench_c3, "c4": bench_c4}.get(args.only)
         res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)
                if args.only == "c1" else fn(sess, ops, capi, workloads, args.steps, args.warmup))
         print(json.dumps(res))
@@ -335,6 +373,8 @@ def main():
     log("config 2 (prefill GEMM)")
     r2 = bench_c2(sess, ops, capi, workloads, args.steps, args.warmup)
     also = {"c2": r2}
+    log("w4a8 decode GEMV")
+    also["c1w4"] = bench_c1w4(sess, ops, capi, workloads, args.steps, args.warmup)
     if args.workload == "all":
         for name, fn in (("c2w8", bench_c2w8), ("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
             log("config %s" % name)
