@@ -108,7 +108,7 @@ def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
         "config": {"workload": "c1: w8a8 decode GEMV M=1 K=4096 N=14336, fp16 in/out, seeds 2/3",
                    "value_is": "int8 weight bytes (58720256) / step time; step = one fused quantize+GEMV kernel; "
                                "the loop cycles through %d copies of the matrix so that every step reads HBM" % C1_COPIES},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,false,1> (fused per-token quantize + GEMV)",
+        "roofline": {"bound": "hbm", "kernel": "gemv_wide8_kernel<1> (fused per-token quantize + GEMV)",
                      "achieved": algo_bytes / kernel_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": algo_bytes / kernel_us / 1e3 / HBM_PEAK_GBS,
                      "kernel_us": kernel_us, "algorithmic_bytes": algo_bytes,
@@ -200,7 +200,7 @@ def bench_c1w4(sess, ops, capi, workloads, steps, warmup):
     algo_bytes = weight_bytes + K * 2 + N * 2 + N * 4
     out = {"workload": "w4a8 decode GEMV M=1 K=4096 N=14336 (int4 weights, 29360128 B), fp16 in/out, seeds 2/3",
            "weight_GBps": weight_bytes / step_us / 1e3, "ms_per_step": step_us / 1e3,
-           "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,true,1> (fused per-token quantize + int4 GEMV)",
+           "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,true,1,32> (fused per-token quantize + int4 GEMV)",
                         "achieved": algo_bytes / step_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": algo_bytes / step_us / 1e3 / HBM_PEAK_GBS, "kernel_us": step_us,
                         "algorithmic_bytes": algo_bytes, "traffic": None}}

@@ -615,9 +615,333 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 // otherwise runs in two rounds), i.e. four waves per SIMD and at most 128
 // vector registers: stated as a requirement, because the int4 variants with the
 // fused quantization would otherwise be allocated more.
-template <int MR, bool W4, int QT>
+// CW < 32 (narrow matrices, where one workgroup per 32-column block leaves compute
+// units without work -- 128 workgroups for a 4096-column projection): 32 / CW
+// workgroups share a column block, CW = 16 or 8 columns each.  A load instruction
+// then covers the workgroup's part of 32 / CW consecutive k-tiles (pieces of
+// 16 * CW bytes): lane = column % CW + CW * k-half + 2 * CW * (tile of the group),
+// and the cross-lane reduction takes two or three xor-shuffles instead of one.
+template <int MR, bool W4, int QT, int CW>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
+    static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
+    constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
+    // (padding for the single-row variants of narrow matrices: their look-ahead of GEMV_UNROLL loads per wave, and
+    // one more step for the activations, runs up to that many load instructions past the end
+    // of a chunk, 32 / CW tiles of 32 -- int4: 64 -- staged bytes each)
+    constexpr bool ROLLING = MR == 1 && CW < 32; // see the K loop
+    constexpr int A_PAD = ROLLING ? GEMV_WAVES * (GEMV_UNROLL + 1) * TPL * (W4 ? 64 : 32) : 0;
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
+    __shared__ int red[GEMV_WAVES][MR][CW];
+    __shared__ uint32_t row_max[MR];
+    __shared__ float row_scale[MR];
+    const int lane = lane_id(), wave = wave_id();
+    const int half = (lane / CW) & 1;                       // which 16 k of a 32-k tile
+    const int sub = lane / (2 * CW);                        // which tile of the group one load covers
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int p = (int)blockIdx.x / TPL;
+    const int col0 = ((int)blockIdx.x % TPL) * CW;          // first column of the block this workgroup owns
+    const bool first_wg = blockIdx.x == 0;
+    // byte of this lane inside a 1 KiB tile
+    const unsigned lane_byte = (unsigned)((col0 + lane % CW) + 32 * half) * 16u;
+    // chunk of K staged in LDS at a time (multiple of 64)
+    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
+    int acc[MR], folded[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = folded[m] = 0;
+
+    const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
+    const uint8_t* wbase = g.W + (size_t)p * block_bytes;
+    // Weight loads go through a buffer descriptor over this column block: a load whose offset
+    // lies beyond it returns zeros without touching memory, so the loop below needs no branch
+    // around the loads past the end of K -- and without branches the compiler counts the
+    // outstanding loads exactly (it waits for the one it needs, not for all of them).
+    const __amdgpu_buffer_rsrc_t wrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)block_bytes, 0x00020000);
+    auto load_tile = [&](int unit, int units, int first_tile) -> v4i { // `unit` counts this wave's load instructions
+        const unsigned off = unit < units ? (unsigned)(first_tile + unit * TPL + sub) * 1024u + lane_byte : 0xFFFFFFF0u;
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+    };
+
+    // Fused path: put the first batch of weight loads in flight before the
+    // quantization prologue so that its latency hides behind them.
+    // The activation rows are requested FIRST: loads return in issue order, so
+    // behind the weight loads they would arrive with the last of those, and the
+    // prologue (and with it the second batch of weight loads) would start only
+    // then.  Fetched first they are back after one L2 round trip and the whole
+    // quantization runs under the weight loads' latency.
+    v4i wpre[GEMV_UNROLL];
+    using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
+    typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
+    if constexpr (QT != 0) {
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = (int)threadIdx.x + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const QT_T* row = static_cast<const QT_T*>(q.src) + (size_t)m * K;
+                araw[i] = RowLoader<QT_T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
+#pragma unroll
+        for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (QT != 0) {
+        using T = QT_T;
+        const int t = threadIdx.x;
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+        if (t < MR) row_max[t] = 0u;
+        __syncthreads();
+        // (the rows stay in registers as fetched and are converted once per pass:
+        // holding them as floats across the barriers costs the int4 variants their
+        // second workgroup per compute unit)
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                float mx = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    mx = fmaxf(mx, fabsf(v[j]));
+                    bad |= not_finite(v[j]);
+                }
+                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
+            }
+        }
+        __syncthreads();
+        if (t < g.M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            if (first_wg && q.scale) q.scale[t] = sc;
+        }
+        if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
+        // zero the K padding of the staged rows
+        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) {
+            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
+                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            }
+        }
+        // a_scale of the epilogue comes from LDS in this path
+    }
+
+    for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
+        const int kc = min(kc_max, Kp - kc0);
+        // stage activations: row-major [MR][kc] in LDS from the tiled buffer
+        const int chunks = kc >> 4;
+        if (kc0) __syncthreads();
+        if constexpr (QT == 0) {
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks;
+                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+            }
+        }
+        __syncthreads();
+
+        // One group = GEMV_UNROLL tiles per wave.  Int4: a tile is a 64-deep super-tile.
+        // (counted in load instructions: one of them spans 32 / CW tiles; K is padded to 256 and a
+        // chunk but the last holds a multiple of 4096 k, so the tile count is a multiple of that)
+        const int tiles = (W4 ? kc >> 6 : kc >> 5) / TPL, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
+        auto load_unit = [&](int unit) -> v4i { return load_tile(unit, tiles, tile0); };
+        auto consume_unit = [&](const v4i& wu, int unit) {
+            {
+                // This lane's tile within the chunk.  Past the end of the chunk the weights are
+                // zeros, so whatever the activation read returns does not matter: it lands in the
+                // next row or in the padding behind the last one.
+                const int tt = unit * TPL + sub;
+                if constexpr (!W4) {
+#pragma unroll
+                    for (int m = 0; m < MR; ++m) {
+                        const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                        acc[m] = __builtin_amdgcn_sdot4(av.x, wu.x, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.y, wu.y, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.z, wu.z, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.w, wu.w, acc[m], false);
+                    }
+                } else {
+                    // The words pass through an empty asm statement so that their unpacking
+                    // stays here: moved up to where the prefetched group arrived (the compiler
+                    // does that) the sixteen operand words per tile of all eight tiles are live
+                    // across the prologue, more registers than two workgroups per compute unit leave.
+                    int wv[4] = {wu.x, wu.y, wu.z, wu.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(wv[i]));
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {       // the two 32-k halves
+                        const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
+                        const int hi0 = wv[2 * s] & 0xF0F0F0F0;
+                        const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
+                        const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
+#pragma unroll
+                        for (int m = 0; m < MR; ++m) {
+                            const v4i av = *reinterpret_cast<const v4i*>(
+                                a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                            acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
+                            acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
+                        }
+                    }
+                }
+            }
+        };
+        if constexpr (ROLLING) {
+            // A rolling window of GEMV_UNROLL loads per wave: as soon as a tile is used, the
+            // register it sat in takes the load of the tile GEMV_UNROLL places further on, so the
+            // number of loads in flight does not drain between groups (a workgroup of a narrow
+            // matrix walks a long K alone on its compute unit).  The fused path starts from the
+            // group fetched ahead of the prologue (it has a single K chunk).
+            // The staged activations of a tile are read one step ahead of its use, so that
+            // their LDS latency does not sit between the arrival of a tile and the next load.
+            struct ActTile { v4i a[W4 ? 2 : 1]; };
+            auto read_act = [&](int unit) {
+                const int tt = unit * TPL + sub; // (past the end of the chunk: the next row or the padding)
+                ActTile r;
+                if constexpr (!W4) {
+                    r.a[0] = *reinterpret_cast<const v4i*>(a_lds + (size_t)(tt * 2 + half) * 16);
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        r.a[s] = *reinterpret_cast<const v4i*>(a_lds + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                }
+                return r;
+            };
+            auto dot_tile = [&](const v4i& wu, const ActTile& t) {
+                if constexpr (!W4) {
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].x, wu.x, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].y, wu.y, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].z, wu.z, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].w, wu.w, acc[0], false);
+                } else {
+                    const int wv[4] = {wu.x, wu.y, wu.z, wu.w};
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].x, (wv[2 * s] << 4) & 0xF0F0F0F0, acc[0], false);
+                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].y, wv[2 * s] & 0xF0F0F0F0, acc[0], false);
+                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].z, (wv[2 * s + 1] << 4) & 0xF0F0F0F0, acc[0], false);
+                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].w, wv[2 * s + 1] & 0xF0F0F0F0, acc[0], false);
+                    }
+                }
+            };
+            v4i w[GEMV_UNROLL];
+#pragma unroll
+            for (int u = 0; u < GEMV_UNROLL; ++u) {
+                if constexpr (QT != 0) w[u] = wpre[u];
+                else w[u] = load_unit(wave + u * GEMV_WAVES);
+            }
+            ActTile cur = read_act(wave);
+            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                    const ActTile nxt = read_act(tb + (u + 1) * GEMV_WAVES);
+                    dot_tile(w[u], cur);
+                    w[u] = load_unit(tb + (GEMV_UNROLL + u) * GEMV_WAVES);
+                    // (each load stays behind the use of its register; gathered at the end of the
+                    // iteration, as the scheduler would have them, the window drains every time)
+                    __builtin_amdgcn_sched_barrier(0);
+                    cur = nxt;
+                }
+            }
+        } else {
+            // A group of GEMV_UNROLL loads at a time.  Several rows: the rolling window above costs
+            // those variants more registers than two workgroups per compute unit leave.  Wide
+            // matrices: they are bound by memory throughput, not by a workgroup's own latency, and
+            // a workgroup that asks for its next 64 KiB in one go is served faster than one that
+            // trickles the requests out a tile at a time (4096 x 14336, int8: 11.5 against 11.9 us).
+            int tb = wave;
+            if constexpr (QT != 0) {
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u)
+                    if (tb + u * GEMV_WAVES < tiles) consume_unit(wpre[u], tb + u * GEMV_WAVES);
+                tb += GEMV_WAVES * GEMV_UNROLL;
+            }
+            for (; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+                v4i w[GEMV_UNROLL];
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u) w[u] = load_unit(tb + u * GEMV_WAVES);
+#pragma unroll
+                for (int u = 0; u < GEMV_UNROLL; ++u)
+                    if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
+            }
+        }
+        if constexpr (W4) {
+            // int4 operands are carried as 16 * code; fold each K chunk's exact
+            // multiple-of-16 partial back so very long K cannot overflow int32.
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                folded[m] += acc[m] >> 4;
+                acc[m] = 0;
+            }
+        }
+    }
+
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        int v = W4 ? folded[m] : acc[m];
+        v += __shfl_xor(v, 32);
+        if (CW <= 16) v += __shfl_xor(v, 16);
+        if (CW <= 8) v += __shfl_xor(v, 8);
+        if (lane < CW) red[wave][m][lane] = v;
+    }
+    __syncthreads();
+    static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
+    if ((int)threadIdx.x < MR * CW) {
+        const int m = (int)threadIdx.x / CW, j = (int)threadIdx.x % CW;
+        if (m >= g.M) return;
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
+        const int n = block_first_col(p, g.interleave_F) + col0 + j;
+        if (n < g.N)
+            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
+                      QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
+                      g.w_scale ? g.w_scale[n] : 1.0f);
+    }
+}
+
+
+// ---- single-row int8 GEMV of a wide matrix (more than 256 column blocks) ----
+// The same workgroup layout as gemv_kernel<1, false, QT, 32>, but with the
+// loads past the end of K skipped by branches instead of being sent through a
+// bounds-checked descriptor.  With the branches the compiler no longer counts
+// the outstanding loads exactly and waits for ALL of a wave's loads wherever it
+// needs one of them -- so every wave of a workgroup has its whole group of tiles
+// before the quantization prologue starts, passes the prologue's barriers with
+// nothing outstanding, uses the group at once and asks for the next group in
+// one burst together with the other seven waves.  For a matrix that is bound
+// by memory throughput that is the faster order, measured on one box for
+// 4096 x 14336 (the decode shape of the benchmark): 11.05 us against 11.5 us for
+// gemv_kernel's exact waits (11.4 with an explicit wait for the whole group in
+// front of the prologue or of the K loop).  Int4 matrices of the same shape are
+// faster on gemv_kernel (7.8 against 8.3 us) and stay there.
+template <int QT>
+__global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
+void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
+    constexpr int MR = 1;
+    constexpr bool W4 = false;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
     __shared__ uint32_t row_max[MR];
@@ -831,6 +1155,7 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
                       g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
+
 
 // ------------------------------------------------------------------ GEMM
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
@@ -1996,10 +2321,32 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
 template <int MR>
 int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
     const int pblocks = (int)(rkh_align_up(g.N, 32) / 32);
-    const dim3 grid(pblocks), block(GEMV_WAVES * 64);
+    // Narrow matrices: several workgroups per column block (16 columns each up to 256 blocks =
+    // 8192 columns, 8 columns each up to 64 blocks), so that a 4096-column projection has a
+    // workgroup for every compute unit; all of them still run at once.  (Measured per shape on
+    // one box, M = 1, int8 / int4 us: 4096 x 4096: 7.7 / 6.1 with 32 columns, 6.6 / 5.5 with 16,
+    // 6.9 / 6.0 with 8; 14336 x 4096: 16.6 / 12.3, 14.5 / 10.5, 13.7 / 11.3; 8192 x 1024:
+    // 10.6 / 8.1, 7.9 / 6.4, 6.4 / 5.7; a 14336-column matrix loses a quarter with 16.)
+    // (RK_NPU_HIP_GEMV_COLS = 8 / 16 / 32 forces the choice: tuning aid)
+    static const char* forced = getenv("RK_NPU_HIP_GEMV_COLS");
+    const int want = forced ? atoi(forced) : 0;
+    const int cw = want == 8 || want == 16 || want == 32 ? want : pblocks <= 64 ? 8 : pblocks <= 256 ? 16 : 32;
+    const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
-#define RK_GEMV(W4, QT) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT>), grid, block, 0, st, g, q)
+    if (MR == 1 && !g.w_int4 && cw == 32) { // (see gemv_wide8_kernel)
+        if (qt == 0) hipLaunchKernelGGL((gemv_wide8_kernel<0>), grid, block, 0, st, g, q);
+        else if (qt == 1) hipLaunchKernelGGL((gemv_wide8_kernel<1>), grid, block, 0, st, g, q);
+        else hipLaunchKernelGGL((gemv_wide8_kernel<2>), grid, block, 0, st, g, q);
+        RKH_CHECK(hipGetLastError());
+        return RKH_OK;
+    }
+#define RK_GEMV(W4, QT)                                                                        \
+    do {                                                                                       \
+        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, g, q);        \
+        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, g, q); \
+        else hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, g, q);               \
+    } while (0)
     if (g.w_int4) {
         if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
     } else {
