@@ -33,7 +33,10 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           # K a single / an odd number of 64-deep super-tiles
           (70, 11000, 192), (33, 33000, 40),
           # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
-          (650, 6900, 1000), (641, 6912, 200)]
+          (650, 6900, 1000), (641, 6912, 200),
+          # decode GEMV variants: 16 columns per workgroup (one row: rolling load window; several rows),
+          # 32 columns per workgroup on a wide matrix, K staged in several chunks
+          (1, 4096, 4096), (3, 2500, 1000), (1, 9000, 520), (8, 8200, 5000)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

@@ -24,7 +24,9 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
               (100, 8448, 160), (128, 96, 3000),
               # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
-              (641, 6900, 200), (700, 6900, 1100)]
+              (641, 6900, 200), (700, 6900, 1100),
+              # decode GEMV: 16 columns per workgroup (65 .. 256 column blocks) / 32 columns (more)
+              (1, 2100, 257), (5, 8300, 100)]
 
 
 @pytest.mark.parametrize("M,N,K", I32_SHAPES)
@@ -64,7 +66,10 @@ def test_i8i8i32_extremes_wrap(sess, oracle):
 
 F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64, 128),
               (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024),
-              (650, 7000, 1100)]  # large-tile kernel
+              (650, 7000, 1100),  # large-tile kernel
+              # decode GEMV variants: 16 columns per workgroup with the rolling load window (one row),
+              # with several rows, with K staged in several chunks; wide matrices with one / several rows
+              (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300)]
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
