@@ -1,0 +1,133 @@
+"""GPU parity of the device-pointer entry points (include/rk_npu_hip.h) against the CPU oracle.
+
+These calls take operands that already lie in device memory and only enqueue
+work, so for decode-sized M they reach the one-launch path in which the GEMV
+quantizes its rows itself -- a path the host-pointer calls never take (they
+quantize from the pinned mirror with a kernel of its own).  Same bar as the
+host-pointer tests: quantized codes, scales and outputs bit-exact.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from rknpu2_matmul_open_amd import capi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits32(x):
+    return np.ascontiguousarray(x, np.float32).view(np.uint32)
+
+
+def _special_rows(A, as_f16):
+    """A zero row (scale 1) and a row of exact ties at scale 1 where the row count allows."""
+    M, K = A.shape
+    if M > 2:
+        A[1, :] = 0
+        ties = np.array([127, -127, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32)[: min(K, 8)]
+        A[2, :] = 0
+        A[2, : len(ties)] = ties.astype(np.float16).view(np.uint16) if as_f16 else ties
+    return A
+
+
+# M <= 8 with rows that fit the fused GEMV (one launch), every column width of the kernel
+# (<= 64 / 65..256 / > 256 column blocks), ragged N and K; the last ones do not fit the fused
+# path (rows too long) or have more than 8 rows and take the two-kernel route.
+W8_SHAPES = [(1, 64, 64), (1, 200, 200), (1, 513, 1000), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520),
+             (2, 3000, 700), (3, 65, 33), (4, 9000, 300), (4, 4100, 8000), (8, 128, 4096), (8, 8300, 2000),
+             (7, 5000, 4100), (2, 2500, 20003), (16, 300, 500)]
+
+
+@pytest.mark.parametrize("M,N,K", W8_SHAPES)
+@pytest.mark.parametrize("f16", [True, False])
+def test_w8a8_dynamic_device(sess, oracle, M, N, K, f16):
+    c = workloads.w8a8_case(M, K, N, seed_w=M + N + 1, seed_a=K + 11)
+    if f16:
+        A = _special_rows(c["A"].copy(), True)
+        kind, out_dtype = capi.F16I8F16_DYNAMIC, np.uint16
+    else:
+        A = _special_rows(oracle.half_to_float(c["A"]).astype(np.float32).reshape(M, K) * 3.0, False)
+        kind, out_dtype = capi.F32I8F32_DYNAMIC, np.float32
+    op = ops.W8A8Linear(sess, kind, M, c["B"], c["w_scale"])
+    dA = sess.to_device(A)
+    dC = sess.empty_device(M * N * np.dtype(out_dtype).itemsize)
+    try:
+        for _ in range(2):  # a second call on the same workspace must give the same answer
+            assert op.run_device(dA, dC) == 0
+            assert sess.sync() == 0
+            got = sess.from_device(dC, (M, N), out_dtype)
+            want = oracle.w8a8(A, c["B"], c["w_scale"])
+            q, s = op.read_quantized()
+            assert np.array_equal(_bits32(s), _bits32(want["a_scale"]))
+            assert np.array_equal(q, want["q"])
+            if f16:
+                assert np.array_equal(got, want["C"])
+            else:
+                assert np.array_equal(_bits32(got), _bits32(want["C"]))
+    finally:
+        sess.free_device(dA)
+        sess.free_device(dC)
+        op.close()
+
+
+W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520), (2, 65, 20003),
+             (3, 2500, 1000), (4, 9000, 300), (8, 128, 512), (8, 8200, 2000), (5, 4100, 5000), (12, 200, 300)]
+
+
+@pytest.mark.parametrize("M,N,K", W4_SHAPES)
+def test_w4a8_device(sess, oracle, M, N, K):
+    rng = np.random.default_rng(M * 7919 + N * 31 + K + 5)
+    B = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.02
+    A = _special_rows((rng.standard_normal((M, K)) * 2).astype(np.float32), False)
+    A16 = A.astype(np.float16).view(np.uint16)
+    lib = sess.lib
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    dA, dA16 = sess.to_device(A), sess.to_device(A16)
+    dC, dC16 = sess.empty_device(M * N * 4), sess.empty_device(M * N * 2)
+    try:
+        want = oracle.w4a8(A, B, ws)
+        assert lib.rk_npu_w4a8_run_f32_device(wsp.h, w.h, dA, dC) == 0
+        assert sess.sync() == 0
+        q, s = wsp.read_quantized()
+        assert np.array_equal(_bits32(s), _bits32(want["a_scale"]))
+        assert np.array_equal(q, want["q"])
+        assert np.array_equal(_bits32(sess.from_device(dC, (M, N), np.float32)), _bits32(want["C"]))
+        want16 = oracle.w4a8(A16, B, ws)
+        assert lib.rk_npu_w4a8_run_f16_device(wsp.h, w.h, dA16, dC16) == 0
+        assert sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC16, (M, N), np.uint16), want16["C"])
+    finally:
+        for d in (dA, dA16, dC, dC16):
+            sess.free_device(d)
+        wsp.close()
+        w.close()
+
+
+def test_w4a8_device_rejects_nonfinite_rows(sess):
+    """NaN / Inf in a row: the enqueue succeeds, the next sync reports RK_NPU_ERR_PARAM."""
+    M, N, K = 2, 96, 200
+    rng = np.random.default_rng(3)
+    B = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    ws = np.full(N, 0.01, np.float32)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    A[1, 17] = np.inf
+    dA, dC = sess.to_device(A), sess.empty_device(M * N * 4)
+    try:
+        assert sess.lib.rk_npu_w4a8_run_f32_device(wsp.h, w.h, dA, dC) == 0
+        assert sess.sync() == capi.RK_NPU_ERR_PARAM
+        # the context is usable again afterwards
+        A[1, 17] = 1.0
+        sess.free_device(dA)
+        dA = sess.to_device(A)
+        assert sess.lib.rk_npu_w4a8_run_f32_device(wsp.h, w.h, dA, dC) == 0
+        assert sess.sync() == 0
+    finally:
+        sess.free_device(dA)
+        sess.free_device(dC)
+        wsp.close()
+        w.close()
