@@ -151,7 +151,8 @@ def test_w4a8_rejections(sess):
         w.close()
 
 
-SWIGLU_SHAPES = [(1, 64, 64), (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
+SWIGLU_SHAPES = [(1, 64, 64), (1, 4160, 1000), (2, 192, 20003),  # one / two rows: the SwiGLU GEMV (ragged K, K in chunks)
+                 (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
                  (128, 1024, 512),
                  (20, 32896, 128), (32, 2048, 700),  # weight-streaming kernel: wide grid / K split inside the workgroup
                  (650, 6912, 520), (641, 7040, 300)]  # large-tile kernel (F a multiple of 64 / only of 32)
@@ -181,7 +182,7 @@ def test_swiglu_bit_exact_poly_and_close_to_libm(sess, oracle, M, N, K):
         w.close()
 
 
-FFN_SHAPES = [(1, 64, 64, 64), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
+FFN_SHAPES = [(1, 64, 64, 64), (2, 256, 2048, 300), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
               (128, 384, 2048, 256)]
 
 
