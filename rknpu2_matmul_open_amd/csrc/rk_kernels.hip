@@ -2820,6 +2820,18 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
 
 int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_args* gargs) {
     if (gemv_can_fuse(*qargs, *gargs)) return dispatch_gemv((hipStream_t)stream, *gargs, qargs);
+    if (qargs->mode == RKH_Q_REUSE_BITS) {
+        // A decode-sized re-quantization (the down projection of an FFN with a few rows) is
+        // folded into the GEMV as well: the kernel scans its rows itself instead of reading the
+        // partial maxima the SwiGLU epilogue left.  Same result -- the maximum of the partial
+        // maxima IS the row maximum, the scale rule and the rejection of non-finite rows are
+        // those of RKH_Q_W4A8 -- and one launch less.
+        rkh_quant_args scan = *qargs;
+        scan.mode = RKH_Q_W4A8;
+        scan.row_max_bits = nullptr;
+        scan.row_max_parts = 0;
+        if (gemv_can_fuse(scan, *gargs)) return dispatch_gemv((hipStream_t)stream, *gargs, &scan);
+    }
     const int rc = rkh_quant_rows(stream, qargs);
     return rc ? rc : rkh_gemm(stream, gargs);
 }
