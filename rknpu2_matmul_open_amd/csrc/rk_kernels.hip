@@ -1169,11 +1169,15 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
 // gate/up projection of a 4096 -> 14336 FFN took 14.9 us.
 constexpr int GEMV_SWIGLU_UNROLL = 4; // load instructions per wave and block in flight (two blocks)
 
-template <int MR, bool W4>
+// QT as in gemv_kernel: 0 = quantized rows in g.A, 1 / 2 = the kernel quantizes the fp16 / fp32
+// rows q.src itself (same prologue: rows requested first, then the first group of weights).
+template <int MR, bool W4, int QT>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
-void gemv_swiglu_kernel(rkh_gemm_args g) {
+void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[2][GEMV_WAVES][MR][32];
+    __shared__ uint32_t row_max[MR];
+    __shared__ float row_scale[MR];
     const int lane = lane_id(), wave = wave_id();
     const int half = lane >> 5;
     const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
@@ -1192,30 +1196,100 @@ void gemv_swiglu_kernel(rkh_gemm_args g) {
     // (bounds-checked descriptor over the two blocks: see gemv_kernel)
     const __amdgpu_buffer_rsrc_t wrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)(2 * block_bytes), 0x00020000);
+    v4i w[2][GEMV_SWIGLU_UNROLL];
+    auto load_group = [&](int tb, int tiles, int tile0) {
+#pragma unroll
+        for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int tt = tb + u * GEMV_WAVES;
+                const unsigned off = tt < tiles ? (unsigned)(b * block_bytes) + (unsigned)(tile0 + tt) * 1024u + (unsigned)lane * 16u
+                                                : 0xFFFFFFF0u;
+                w[b][u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+            }
+    };
+
+    if constexpr (QT != 0) { // (the fused path has a single K chunk: rows fit the staging area)
+        using T = typename std::conditional<QT == 2, float, uint16_t>::type;
+        const int t = threadIdx.x;
+        const bool first_wg = blockIdx.x == 0;
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+        typename RowLoader<T>::Raw araw[GEMV_QCHUNKS];
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const T* row = static_cast<const T*>(q.src) + (size_t)m * K;
+                araw[i] = RowLoader<T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_group(wave, W4 ? Kp >> 6 : Kp >> 5, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t < MR) row_max[t] = 0u;
+        __syncthreads();
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                float mx = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    mx = fmaxf(mx, fabsf(v[e]));
+                    bad |= not_finite(v[e]);
+                }
+                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
+            }
+        }
+        __syncthreads();
+        if (t < g.M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            if (first_wg && q.scale) q.scale[t] = sc;
+        }
+        if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
+        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) { // zero the K padding
+            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
+                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            }
+        }
+    }
 
     for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
         const int kc = min(kc_max, Kp - kc0);
         const int chunks = kc >> 4;
         if (kc0) __syncthreads();
-        for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
-            const int m = idx / chunks, c = idx - m * chunks;
-            const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-            *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+        if constexpr (QT == 0) {
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks;
+                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+            }
         }
         __syncthreads();
 
         const int tiles = W4 ? kc >> 6 : kc >> 5, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
         for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_SWIGLU_UNROLL) {
-            v4i w[2][GEMV_SWIGLU_UNROLL];
-#pragma unroll
-            for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u)
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    const int tt = tb + u * GEMV_WAVES;
-                    const unsigned off = tt < tiles ? (unsigned)(b * block_bytes) + (unsigned)(tile0 + tt) * 1024u + (unsigned)lane * 16u
-                                                    : 0xFFFFFFF0u;
-                    w[b][u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
-                }
+            if (QT == 0 || tb != wave) load_group(tb, tiles, tile0); // (fused: the first group is on its way)
 #pragma unroll
             for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u) {
                 const int tt = tb + u * GEMV_WAVES;
@@ -1288,7 +1362,7 @@ void gemv_swiglu_kernel(rkh_gemm_args g) {
         }
         uint32_t bits = 0;
         if (live) {
-            const float as = g.a_scale ? g.a_scale[m] : 1.0f;
+            const float as = QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f);
             const float gf = dequant(gate, as, g.w_scale ? g.w_scale[n] : 1.0f);
             const float uf = dequant(up, as, g.w_scale ? g.w_scale[F + n] : 1.0f);
             const float y = __fmul_rn(silu_poly(gf), uf);
@@ -2502,10 +2576,17 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
 }
 
 template <int MR>
-int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g) {
+int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
     const dim3 grid(g.interleave_F / 32), block(GEMV_WAVES * 64);
-    if (g.w_int4) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, true>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemv_swiglu_kernel<MR, false>), grid, block, 0, st, g);
+    const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
+    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+#define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, g, q)
+    if (g.w_int4) {
+        if (qt == 0) RK_SWI(true, 0); else if (qt == 1) RK_SWI(true, 1); else RK_SWI(true, 2);
+    } else {
+        if (qt == 0) RK_SWI(false, 0); else if (qt == 1) RK_SWI(false, 1); else RK_SWI(false, 2);
+    }
+#undef RK_SWI
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
@@ -2519,9 +2600,9 @@ bool gemv_swiglu_applies(const rkh_gemm_args& g) {
            g.interleave_F % 32 == 0 && g.N == 2 * g.interleave_F && g.K <= (1 << 24);
 }
 
-int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g) {
-    if (g.M == 1) return launch_gemv_swiglu<1>(st, g);
-    return launch_gemv_swiglu<2>(st, g);
+int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    if (g.M == 1) return launch_gemv_swiglu<1>(st, g, fuse);
+    return launch_gemv_swiglu<2>(st, g, fuse);
 }
 
 int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
@@ -2533,8 +2614,8 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 
 // The decode path can quantize inside the GEMV when the rows fit the kernel's
 // LDS staging and per-thread register cache.
-bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g) {
-    if (g.blk_expert || g.M > 8 || g.epilogue == RKH_EPI_SWIGLU || q.src_is_host) return false;
+bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
+    if (g.blk_expert || g.M > 8 || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
     const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
@@ -2804,7 +2885,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     hipStream_t st = (hipStream_t)stream;
     const bool grouped = g.blk_expert != nullptr;
     if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) return dispatch_gemv(st, g, nullptr);
-    if (gemv_swiglu_applies(g)) return dispatch_gemv_swiglu(st, g);
+    if (gemv_swiglu_applies(g)) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
     const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);
@@ -2820,6 +2901,8 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
 
 int rkh_quant_gemm(void* stream, const rkh_quant_args* qargs, const rkh_gemm_args* gargs) {
     if (gemv_can_fuse(*qargs, *gargs)) return dispatch_gemv((hipStream_t)stream, *gargs, qargs);
+    if (gemv_swiglu_applies(*gargs) && gemv_can_fuse(*qargs, *gargs, true))
+        return dispatch_gemv_swiglu((hipStream_t)stream, *gargs, qargs);
     if (qargs->mode == RKH_Q_REUSE_BITS) {
         // A decode-sized re-quantization (the down projection of an FFN with a few rows) is
         // folded into the GEMV as well: the kernel scans its rows itself instead of reading the

@@ -6,8 +6,6 @@ quantizes its rows itself -- a path the host-pointer calls never take (they
 quantize from the pinned mirror with a kernel of its own).  Same bar as the
 host-pointer tests: quantized codes, scales and outputs bit-exact.
 """
-import ctypes as C
-
 import numpy as np
 import pytest
 
@@ -131,3 +129,66 @@ def test_w4a8_device_rejects_nonfinite_rows(sess):
         sess.free_device(dC)
         wsp.close()
         w.close()
+
+
+# one / two rows: gate/up + SwiGLU as a GEMV that quantizes its rows itself, and a down GEMV that
+# re-quantizes the middle itself; more rows: the MFMA kernels with kernels of their own for both
+FFN_SHAPES = [(1, 64, 64, 64), (1, 1000, 4160, 300), (2, 256, 2048, 300), (2, 20003, 96, 65),
+              (5, 128, 96, 65), (8, 512, 1024, 4100), (33, 256, 160, 128)]
+
+
+@pytest.mark.parametrize("M,H,I,Nout", FFN_SHAPES)
+def test_w4a8_ffn_device(sess, oracle, M, H, I, Nout):
+    rng = np.random.default_rng(M + H + I + 17)
+    B_gu = rng.integers(-7, 8, (H, 2 * I)).astype(np.int8)
+    s_gu = (rng.random(2 * I).astype(np.float32) + 0.5) * 0.01
+    B_dn = rng.integers(-7, 8, (I, Nout)).astype(np.int8)
+    s_dn = (rng.random(Nout).astype(np.float32) + 0.5) * 0.01
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    if M > 2:
+        x[1] = 0.0  # zero token -> zero middle row -> Down scale 1
+    gw, dw = ops.W4A8Weights(sess, B_gu, s_gu), ops.W4A8Weights(sess, B_dn, s_dn)
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, Nout, I)
+    dA = sess.to_device(x)
+    dmid, dC = sess.empty_device(M * I * 4), sess.empty_device(M * Nout * 4)
+    try:
+        want = oracle.w4a8_ffn(x, B_gu, s_gu, B_dn, s_dn, oracle.EXP_POLY)
+        assert want["rc"] == 0
+        for _ in range(2):
+            assert sess.lib.rk_npu_w4a8_run_ffn_f32_device(gws.h, gw.h, dws.h, dw.h, dA, dmid, dC) == 0
+            assert sess.sync() == 0
+            assert np.array_equal(_bits32(sess.from_device(dmid, (M, I), np.float32)), _bits32(want["middle"]))
+            qd, sd = dws.read_quantized()
+            assert np.array_equal(_bits32(sd), _bits32(want["down_scale"]))
+            assert np.array_equal(qd, want["q_down"])
+            assert np.array_equal(_bits32(sess.from_device(dC, (M, Nout), np.float32)), _bits32(want["C"]))
+    finally:
+        for d in (dA, dmid, dC):
+            sess.free_device(d)
+        for o in (gws, dws, gw, dw):
+            o.close()
+
+
+def test_w4a8_ffn_device_nonfinite_middle_is_rejected(sess):
+    """A middle that overflows to Inf (huge scales) must surface as RK_NPU_ERR_PARAM at the next
+    sync, also when the down GEMV scans the middle itself (one row)."""
+    M, H, I, Nout = 1, 64, 64, 64
+    B_gu = np.full((H, 2 * I), 7, np.int8)
+    s_gu = np.full(2 * I, 1e18, np.float32)
+    B_dn = np.ones((I, Nout), np.int8)
+    s_dn = np.ones(Nout, np.float32)
+    x = np.full((M, H), 1e18, np.float32)
+    gw, dw = ops.W4A8Weights(sess, B_gu, s_gu), ops.W4A8Weights(sess, B_dn, s_dn)
+    gws, dws = ops.W4A8Workspace(sess, M, 2 * I, H), ops.W4A8Workspace(sess, M, Nout, I)
+    dA = sess.to_device(x)
+    dmid, dC = sess.empty_device(M * I * 4), sess.empty_device(M * Nout * 4)
+    try:
+        assert sess.lib.rk_npu_w4a8_run_ffn_f32_device(gws.h, gw.h, dws.h, dw.h, dA, dmid, dC) == 0
+        assert sess.sync() == capi.RK_NPU_ERR_PARAM
+        mid = sess.from_device(dmid, (M, I), np.float32)
+        assert not np.isfinite(mid).all()
+    finally:
+        for d in (dA, dmid, dC):
+            sess.free_device(d)
+        for o in (gws, dws, gw, dw):
+            o.close()
