@@ -941,7 +941,6 @@ template <int QT>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
     constexpr int MR = 1;
-    constexpr bool W4 = false;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
     __shared__ uint32_t row_max[MR];
@@ -953,11 +952,11 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
     const int p = blockIdx.x;
     // chunk of K staged in LDS at a time (multiple of 64)
     const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
-    int acc[MR], folded[MR];
+    int acc[MR];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = folded[m] = 0;
+    for (int m = 0; m < MR; ++m) acc[m] = 0;
 
-    const uint8_t* wbase = g.W + (W4 ? (size_t)p * (Kp / 64) * 1024 : (size_t)p * KB * 1024);
+    const uint8_t* wbase = g.W + (size_t)p * KB * 1024;
 
     // Fused path: put the first batch of weight loads in flight before the
     // quantization prologue so that its latency hides behind them.
@@ -981,7 +980,7 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        const int tiles = W4 ? Kp >> 6 : Kp >> 5;
+        const int tiles = Kp >> 5;
 #pragma unroll
         for (int u = 0; u < GEMV_UNROLL; ++u) {
             const int tt = wave + u * GEMV_WAVES;
@@ -1061,8 +1060,8 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
         }
         __syncthreads();
 
-        // One group = GEMV_UNROLL tiles per wave.  Int4: a tile is a 64-deep super-tile.
-        const int tiles = W4 ? kc >> 6 : kc >> 5, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
+        // One group = GEMV_UNROLL tiles per wave.
+        const int tiles = kc >> 5, tile0 = kc0 >> 5;
         auto fetch = [&](v4i* w, int tb) {
 #pragma unroll
             for (int u = 0; u < GEMV_UNROLL; ++u) {
@@ -1077,39 +1076,13 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
             for (int u = 0; u < GEMV_UNROLL; ++u) {
                 const int tt = tb + u * GEMV_WAVES;
                 if (tt >= tiles) continue;
-                if constexpr (!W4) {
 #pragma unroll
-                    for (int m = 0; m < MR; ++m) {
-                        const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
-                        acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
-                    }
-                } else {
-                    // The words pass through an empty asm statement so that their unpacking
-                    // stays here: moved up to where the prefetched group arrived (the compiler
-                    // does that) the sixteen operand words per tile of all eight tiles are live
-                    // across the prologue, more registers than two workgroups per compute unit leave.
-                    int wv[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(wv[i]));
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {       // the two 32-k halves
-                        const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
-                        const int hi0 = wv[2 * s] & 0xF0F0F0F0;
-                        const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
-                        const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
-#pragma unroll
-                        for (int m = 0; m < MR; ++m) {
-                            const v4i av = *reinterpret_cast<const v4i*>(
-                                a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
-                            acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
-                        }
-                    }
+                for (int m = 0; m < MR; ++m) {
+                    const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                    acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
+                    acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
+                    acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
+                    acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
                 }
             }
         };
@@ -1123,20 +1096,11 @@ void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
             fetch(w, tb);
             consume(w, tb);
         }
-        if constexpr (W4) {
-            // int4 operands are carried as 16 * code; fold each K chunk's exact
-            // multiple-of-16 partial back so very long K cannot overflow int32.
-#pragma unroll
-            for (int m = 0; m < MR; ++m) {
-                folded[m] += acc[m] >> 4;
-                acc[m] = 0;
-            }
-        }
     }
 
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-        int v = W4 ? folded[m] : acc[m];
+        int v = acc[m];
         v += __shfl_xor(v, 32);
         if (lane < 32) red[wave][m][lane] = v;
     }
