@@ -106,6 +106,34 @@ int rk_npu_w4a8_workspace_read_quantized(rk_npu_w4a8_workspace* workspace, int8_
 int rk_npu_w4a8_run_i32(rk_npu_w4a8_workspace* workspace, const rk_npu_w4a8_weights* weights,
                         const float* A, int32_t* acc);
 
+/* Measurement probes: what the memory system and the matrix pipes of the box at hand give,
+ * to put beside the datasheet peaks.  Each call enqueues ONE kernel on the context's stream
+ * (time it with the events above):
+ *   - a read-only pass over [src_device, src_device + bytes), 16 bytes per lane, every wave
+ *     slot of the chip issuing loads;
+ *   - a pure int8 MFMA loop (v_mfma_i32_32x32x32_i8, eight waves per compute unit, four
+ *     independent accumulators per wave, operands in registers, no memory traffic) on the
+ *     32 KiB at operands_device -- the clock the chip sustains depends on the operands' bit
+ *     patterns, so pass data like the workload's; *ops receives the operation count
+ *     (2 * 32 * 32 * 32 per MFMA). */
+int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes);
+int rk_npu_hip_probe_mfma_i8(rk_npu_ctx* ctx, const void* operands_device, int iterations, double* ops);
+
+/* Stream capture: the *_device calls made between capture_begin and capture_end on this
+ * context (from the calling thread) are recorded instead of executed -- they only launch
+ * kernels, no copy or memset node is ever recorded -- and graph_launch replays the recorded
+ * sequence with one submission.  For decode loops, whose kernels are short enough that the
+ * per-launch submission cost shows.  Run the sequence once eagerly before capturing it (first
+ * use of a kernel may set function attributes); do not call rk_npu_hip_sync, blocking
+ * reference calls or allocation calls on the context while capturing.  Rejected input is
+ * reported by rk_npu_hip_sync after a replay as after eager calls, provided the sequence was
+ * also enqueued eagerly since the previous sync (that registers the workspaces' flags). */
+typedef struct rk_npu_hip_graph rk_npu_hip_graph;
+int rk_npu_hip_capture_begin(rk_npu_ctx* ctx);
+rk_npu_hip_graph* rk_npu_hip_capture_end(rk_npu_ctx* ctx);
+int rk_npu_hip_graph_launch(rk_npu_ctx* ctx, rk_npu_hip_graph* graph);
+void rk_npu_hip_graph_free(rk_npu_hip_graph* graph);
+
 /* Test hook: make the n-th next device allocation fail (1 = the next one,
  * 0 = off), to exercise RK_NPU_ERR_NOMEM / NULL-return paths from the host. */
 void rk_npu_hip_fail_alloc_after(int n);

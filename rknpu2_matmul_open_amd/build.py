@@ -25,8 +25,34 @@ FLAGS = [
 ]
 
 
+# gemm_wk_kernel and gemm_stream_kernel issue their loads from inline assembly and place every
+# s_waitcnt by hand: they rely on this compiler not copying or re-using a load's destination
+# register between the load and the wait that covers it.  The kernels were validated (parity
+# suite on an MI355X) with the compiler named here; any other one may schedule differently, so
+# a build with it says so loudly and the parity suite has to be run again before its results
+# are trusted.
+VALIDATED_HIPCC = "HIP version: 7.2.26015"
+
+
+def check_toolchain(hipcc):
+    """Returns the compiler's version line; warns on stderr when it is not the validated one."""
+    try:
+        out = subprocess.run([hipcc, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                             text=True, check=False).stdout
+    except OSError as e:
+        raise RuntimeError("cannot run %s: %s" % (hipcc, e))
+    line = next((l.strip() for l in out.splitlines() if l.startswith("HIP version:")), "")
+    if not line.startswith(VALIDATED_HIPCC):
+        sys.stderr.write(
+            "\n[build] WARNING: %s reports %r, the inline-assembly load kernels (gemm_wk_kernel,\n"
+            "[build] gemm_stream_kernel) were validated with %r.  Run `pytest tests -m gpu` on an\n"
+            "[build] MI355X before trusting results of this build.\n\n" % (hipcc, line or out[:80], VALIDATED_HIPCC))
+    return line
+
+
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    check_toolchain(hipcc)
     objs = []
     procs = []
     for src in SOURCES:

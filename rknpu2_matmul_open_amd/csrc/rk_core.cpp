@@ -354,4 +354,53 @@ int rk_npu_hip_event_elapsed_us(rk_npu_hip_event* start, rk_npu_hip_event* stop,
 
 void rk_npu_hip_fail_alloc_after(int n) { rkh_fail_malloc_after(n); }
 
+/* ---- measurement probes ---- */
+int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes) {
+    if (!ctx || !src_device || bytes < 16) return RK_NPU_ERR_PARAM;
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    // eight workgroups of 512 lanes per compute unit: every wave slot of the chip issues loads
+    return rkhost::map_error(rkh_probe_stream_read(ctx->stream, src_device, bytes, ctx->cu_count * 8, nullptr));
+}
+int rk_npu_hip_probe_mfma_i8(rk_npu_ctx* ctx, const void* operands_device, int iterations, double* ops) {
+    if (!ctx || !operands_device || iterations < 1) return RK_NPU_ERR_PARAM;
+    const int workgroups = ctx->cu_count; // one workgroup of eight waves per compute unit, as the GEMM runs
+    if (ops) *ops = (double)workgroups * 8.0 * iterations * 4.0 * 2.0 * 32 * 32 * 32;
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    return rkhost::map_error(rkh_probe_mfma_i8(ctx->stream, operands_device, workgroups, iterations, nullptr));
+}
+
+/* ---- stream capture ---- */
+struct rk_npu_hip_graph {
+    void* exec = nullptr;
+};
+int rk_npu_hip_capture_begin(rk_npu_ctx* ctx) {
+    if (!ctx) return RK_NPU_ERR_PARAM;
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    return rkhost::map_error(rkh_capture_begin(ctx->stream));
+}
+rk_npu_hip_graph* rk_npu_hip_capture_end(rk_npu_ctx* ctx) {
+    if (!ctx) return nullptr;
+    auto* g = new (std::nothrow) rk_npu_hip_graph();
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    void* exec = nullptr;
+    const int rc = rkh_capture_end(ctx->stream, &exec); // (always ends the capture, also when g is null)
+    if (rc || !g) {
+        rkh_graph_destroy(exec);
+        delete g;
+        return nullptr;
+    }
+    g->exec = exec;
+    return g;
+}
+int rk_npu_hip_graph_launch(rk_npu_ctx* ctx, rk_npu_hip_graph* graph) {
+    if (!ctx || !graph || !graph->exec) return RK_NPU_ERR_PARAM;
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    return rkhost::map_error(rkh_graph_launch(graph->exec, ctx->stream));
+}
+void rk_npu_hip_graph_free(rk_npu_hip_graph* graph) {
+    if (!graph) return;
+    rkh_graph_destroy(graph->exec);
+    delete graph;
+}
+
 } // extern "C"

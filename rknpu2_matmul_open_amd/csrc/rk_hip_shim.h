@@ -11,7 +11,7 @@
  * -------------------
  * "Tiled int8" (activations and int8 weights): a matrix X[R, K] is stored as
  * 1 KiB tiles of 32 rows x 32 k.  Tile (rb, kb) starts at byte
- * (rb * KB + kb) * 1024 with KB = Kp / 32 and Kp = K rounded up to 64.
+ * (rb * KB + kb) * 1024 with KB = Kp / 32 and Kp = K rounded up to 256 (RKH_K_ALIGN).
  * Inside a tile, lane l = (row % 32) + 32 * ((k % 32) / 16) owns 16
  * consecutive bytes at l * 16, holding k % 16 = 0..15.  One wavefront reads a
  * tile with a single 16-byte-per-lane load and has the int8 MFMA operand of
@@ -118,7 +118,7 @@ typedef struct rkh_quant_args {
     int mode;            /* rkh_quant_mode                                         */
     int M, K;
     float* scale;        /* [M] out (in for STATIC)                                */
-    uint8_t* dst;        /* tiled int8, Kp = align64(K)                            */
+    uint8_t* dst;        /* tiled int8, Kp = align256(K)                           */
     int* bad_flag;       /* OR 1: non-finite input (modes with a check), may be NULL */
     const uint32_t* row_max_bits; /* REUSE modes: [M][row_max_parts] partial maxima of |x| bits */
     int row_max_parts;
@@ -175,7 +175,7 @@ size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4);
 /* Routing + token scatter in one launch: assignments with a non-zero
  * coefficient are bucketed by expert, stably, each bucket padded to 32 sorted
  * rows (the shared expert, id == experts, takes every token); each token is
- * quantized per row (s = max ? max/127 : 1, ties even, non-finite -> bad_flag)
+ * quantized per row (s = max ? max/127 : 1, ties even, rejected input -> bad_flag)
  * or, for int8 input, copied, into the sorted rows of its assignments. */
 typedef struct rkh_moe_scatter_args {
     const int32_t* ids;    /* [rows, top_k] device                                 */
@@ -191,7 +191,10 @@ typedef struct rkh_moe_scatter_args {
     float* token_scale;    /* [rows]: out for fp32 tokens, in for int8 codes       */
     uint8_t* dst;          /* tiled int8 sorted rows                               */
     float* scale_rows;     /* [sorted rows] out: scale of the token in that row    */
-    int* bad_flag;         /* OR 1 on a non-finite fp32 token, may be NULL         */
+    int* bad_flag;         /* OR 1 on rejected input, may be NULL: a non-finite fp32 token or one
+                            * whose scale underflows, a token scale that is not finite and
+                            * positive, an expert id outside [0, experts), a coefficient that is
+                            * negative or not finite                                            */
 } rkh_moe_scatter_args;
 int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args);
 
@@ -203,6 +206,20 @@ typedef struct rkh_moe_combine_args {
     float* out;            /* [rows, H]                                            */
 } rkh_moe_combine_args;
 int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args);
+
+
+/* ---- measurement probes (practical ceilings beside the datasheet peaks) ---- */
+/* One read-only pass over [src, src + bytes) with `workgroups` workgroups of 512 lanes. */
+int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, int workgroups, void* sink);
+/* `workgroups` x 8 waves x `iterations` x 4 int8 MFMAs (32x32x32) on operands read once from
+ * `operands` (32 KiB: 4 x 512 lanes x 16 bytes). */
+int rkh_probe_mfma_i8(void* stream, const void* operands, int workgroups, int iterations, void* sink);
+
+/* ---- stream capture ---- */
+int rkh_capture_begin(void* stream);
+int rkh_capture_end(void* stream, void** graph_exec);
+int rkh_graph_launch(void* graph_exec, void* stream);
+void rkh_graph_destroy(void* graph_exec);
 
 #ifdef __cplusplus
 }

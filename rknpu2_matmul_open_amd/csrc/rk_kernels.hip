@@ -2,12 +2,21 @@
 // launchers declared in rk_hip_shim.h.  Data layouts are described there.
 //
 // Kernel inventory (what bounds each one):
-//   pack_w8 / pack_w4     weight re-tiling at upload            (one-time)
-//   quant_rows            per-token absmax + int8 quantize      (HBM, tiny)
-//   gemv                  M <= 8 decode path, dot4, no MFMA     (HBM)
-//   gemm                  int8 MFMA 32x32x32, LDS double buffer (MFMA / HBM)
-//   splitk_epilogue       dequant / SwiGLU of split-K sums      (HBM, tiny)
-//   moe_route / combine   sort by expert, weighted sum          (latency)
+//   pack_w8_kernel / pack_w4_kernel     weight re-tiling at upload                      (one-time)
+//   quant_rows_kernel                   per-token absmax + int8 codes, workgroup per row (HBM, small)
+//   quant_rows8_kernel                  the same for many rows, 8 / 4 rows per workgroup (HBM)
+//   requant_rows_wave_kernel            re-quantize short fp32 rows, wave per row        (HBM, small)
+//   gemv_kernel / gemv_wide8_kernel     M <= 8 decode path: dot4, no MFMA, optional fused
+//                                       per-token quantization                           (HBM)
+//   gemv_swiglu_kernel                  gate/up + SwiGLU of one or two rows              (HBM)
+//   gemm_wk_kernel                      int8 MFMA 32x32x32, (32..128) x 256 tiles, activations
+//                                       through an LDS ring, waves split K               (MFMA)
+//   gemm_wk_reduce_kernel               sum of K-split partial tiles + epilogue          (L2, small)
+//   gemm_stream_kernel                  32 x 256 tiles, operands straight to registers: MoE
+//                                       (grouped by expert) and dense GEMMs of 9..128 rows (HBM)
+//   moe_scatter_kernel                  route by expert + quantize tokens into sorted rows (latency)
+//   moe_combine_kernel                  weighted sum of expert outputs in slot order     (HBM, small)
+//   stream_read_probe_kernel / mfma_i8_probe_kernel   measurement probes (practical ceilings)
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
@@ -2197,15 +2206,21 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
     const int per_wave = ((n + 63) / 64 + 3) / 4;
     const int wave_first = wave * per_wave * 64;
     int keys[PER_WAVE]; // expert of a live assignment, -1 if dropped or beyond the table
+    bool bad_route = false; // an id outside [0, E) or a coefficient that is negative or not finite
 #pragma unroll
     for (int c = 0; c < PER_WAVE; ++c) {
         const int i = wave_first + c * 64 + lane;
         keys[c] = -1;
         if (c < per_wave && i < n) {
             const int id = a.ids[i];
-            keys[c] = (a.routes[i] != 0.0f && (unsigned)id < (unsigned)E) ? id : -1;
+            const float coeff = a.routes[i];
+            const bool id_ok = (unsigned)id < (unsigned)E;
+            bad_route |= !id_ok || not_finite(coeff) || coeff < 0.0f;
+            keys[c] = (coeff != 0.0f && id_ok) ? id : -1;
         }
     }
+    // (every workgroup sees the whole table: the first one reports for all)
+    if (m == 0 && bad_route && a.bad_flag) atomicOr(a.bad_flag, 1);
     float v[QR_CACHE][16];
     if constexpr (sizeof(T) == 4) {
         if (cached) {
@@ -2308,6 +2323,10 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
     // ---- the token into its sorted rows
     if constexpr (sizeof(T) == 1) {
         __syncthreads(); // dest[]
+        if (t == 0 && a.bad_flag) { // given scales must be finite and positive (reference :595)
+            const float given = a.token_scale[m];
+            if (!(given > 0.0f) || not_finite(given)) atomicOr(a.bad_flag, 1);
+        }
         if (t < slots && dest[t] >= 0) a.scale_rows[dest[t]] = a.token_scale[m];
         const int8_t* brow = reinterpret_cast<const int8_t*>(row);
         for (int c = t; c < nchunks; c += 256) {
@@ -2361,6 +2380,9 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
         if ((wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3]) && t == 0 && a.bad_flag) atomicOr(a.bad_flag, 1);
         const float scale = mx > 0.0f ? mx / 127.0f : 1.0f;
         const float inv = 1.0f / scale;
+        // a maximum so small that the scale underflows to zero or its inverse overflows is
+        // rejected like a non-finite token (reference src/rk_npu_moe_w8.cpp:323-324)
+        if (t == 0 && a.bad_flag && (!(scale > 0.0f) || not_finite(inv))) atomicOr(a.bad_flag, 1);
         if (t == 0) a.token_scale[m] = scale;
         if (t < slots && dest[t] >= 0) a.scale_rows[dest[t]] = scale;
         auto emit = [&](int c, const float* vals) {
@@ -2404,6 +2426,69 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
     }
     *reinterpret_cast<float4*>(a.out + (size_t)tkn * a.H + n) = sum;
 }
+
+
+// ------------------------------------------------------ measurement probes
+// What the memory system and the matrix pipes give on the box the benchmark runs
+// on, to put beside the datasheet peaks: a read-only stream over a footprint and
+// a pure-MFMA loop with operands in registers.
+//
+// Read-only stream: every step of the grid reads one slab of adjacent 1 KiB
+// pieces (16 bytes per lane), workgroup after workgroup, so that the whole grid
+// sweeps memory front to back -- the access order that gave the highest rate of
+// those tried.  The xor of everything read is written only if it equals a value
+// it never takes, which keeps the loads alive.
+__global__ __launch_bounds__(512) void stream_read_probe_kernel(const uint4* __restrict__ src, size_t chunks,
+                                                                uint32_t* sink) {
+    const size_t stride = (size_t)gridDim.x * 512;
+    uint32_t x = 0;
+    size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
+    for (; i + 3 * stride < chunks; i += 4 * stride) { // four loads in flight per lane
+        const v4i a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i));
+        const v4i b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + stride));
+        const v4i c = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + 2 * stride));
+        const v4i d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + 3 * stride));
+        x ^= (uint32_t)(a.x ^ a.y ^ a.z ^ a.w) ^ (uint32_t)(b.x ^ b.y ^ b.z ^ b.w) ^
+             (uint32_t)(c.x ^ c.y ^ c.z ^ c.w) ^ (uint32_t)(d.x ^ d.y ^ d.z ^ d.w);
+    }
+    for (; i < chunks; i += stride) {
+        const v4i a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i));
+        x ^= (uint32_t)(a.x ^ a.y ^ a.z ^ a.w);
+    }
+    if (x == 0x9e3779b9u && sink) atomicAdd(sink, 1u); // (a value chosen to be improbable, not impossible: the sink is scratch)
+}
+
+// Pure int8 MFMA: every wave keeps four independent 32x32 accumulators busy with
+// v_mfma_i32_32x32x32_i8 on operands it loaded once (so their bit patterns -- and
+// the switching activity in the multipliers, which sets the clock the chip
+// sustains -- are those of the caller's data), `iterations` times.  Eight waves
+// per workgroup, as in the GEMM kernels.  2 * 32 * 32 * 32 operations per MFMA.
+__global__ __launch_bounds__(512) void mfma_i8_probe_kernel(const v4i* __restrict__ operands, int iterations,
+                                                            int* sink) {
+    const int t = threadIdx.x;
+    v4i a[2], b[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        a[i] = operands[(size_t)(2 * i) * 512 + t];
+        b[i] = operands[(size_t)(2 * i + 1) * 512 + t];
+    }
+    v16i acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[j & 1], b[j >> 1], acc[j], 0, 0, 0);
+    }
+    int x = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x ^= acc[j][r];
+    if (x == 0x5bd1e995 && sink) atomicAdd(sink, 1);
+}
+
 
 // ------------------------------------------------------------- launchers
 // Workgroups of the 256-column grid below which the K-split variant is used.  Measured on a 32-expert
@@ -2905,5 +2990,46 @@ int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args) {
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
+
+int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, int workgroups, void* sink) {
+    if (!src || bytes < 16 || workgroups < 1) return RKH_ERR_RUNTIME;
+    hipLaunchKernelGGL(stream_read_probe_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream,
+                       static_cast<const uint4*>(src), bytes / 16, static_cast<uint32_t*>(sink));
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int rkh_probe_mfma_i8(void* stream, const void* operands, int workgroups, int iterations, void* sink) {
+    if (!operands || workgroups < 1 || iterations < 1) return RKH_ERR_RUNTIME;
+    hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream,
+                       static_cast<const v4i*>(operands), iterations, static_cast<int*>(sink));
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+// ---- stream capture: a sequence of launches recorded once and replayed ----
+int rkh_capture_begin(void* stream) {
+    RKH_CHECK(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return RKH_OK;
+}
+int rkh_capture_end(void* stream, void** graph_exec) {
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    RKH_CHECK(hipStreamEndCapture((hipStream_t)stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return e == hipErrorOutOfMemory ? RKH_ERR_NOMEM : RKH_ERR_RUNTIME;
+    *graph_exec = exec;
+    return RKH_OK;
+}
+int rkh_graph_launch(void* graph_exec, void* stream) {
+    RKH_CHECK(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    return RKH_OK;
+}
+void rkh_graph_destroy(void* graph_exec) {
+    if (graph_exec) (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+}
+
 
 } // extern "C"

@@ -72,8 +72,8 @@ struct rk_npu_moe_w8_weights {
     int count = 0;              // routed + shared
     size_t gate_stride = 0;     // bytes between experts in gate_up
     size_t down_stride = 0;
-    DeviceBuffer gate_up;       // count x tiled int8 [align256(2I) x align64(H)], gate/up interleaved
-    DeviceBuffer down;          // count x tiled int8 [align256(H) x align64(I)]
+    DeviceBuffer gate_up;       // count x tiled int8 [align256(2I) x align256(H)], gate/up interleaved
+    DeviceBuffer down;          // count x tiled int8 [align256(H) x align256(I)]
     DeviceBuffer gate_scales;   // count x [2I]
     DeviceBuffer down_scales;   // count x [H]
     uint64_t bytes() const {
@@ -92,11 +92,11 @@ struct rk_npu_moe_w8_workspace {
     DeviceBuffer dest_rows;    // [max_rows, slots]
     DeviceBuffer blk_expert;   // [max_blocks]
     DeviceBuffer num_blocks;   // [2]
-    DeviceBuffer a_tiled;      // sorted token rows, tiled int8 [sorted_rows x align64(H)]
+    DeviceBuffer a_tiled;      // sorted token rows, tiled int8 [sorted_rows x align256(H)]
     DeviceBuffer a_scale;      // [sorted_rows]
     DeviceBuffer hidden;       // [sorted_rows, I] fp32
     DeviceBuffer row_max;      // [sorted_rows][I/32] partial row maxima of hidden
-    DeviceBuffer h_tiled;      // re-quantized hidden, tiled int8 [sorted_rows x align64(I)]
+    DeviceBuffer h_tiled;      // re-quantized hidden, tiled int8 [sorted_rows x align256(I)]
     DeviceBuffer h_scale;      // [sorted_rows]
     DeviceBuffer y;            // [sorted_rows, H] fp32 expert outputs
     DeviceBuffer out;          // [max_rows, H] fp32

@@ -77,7 +77,7 @@ bool valid_strategy(const rk_npu_matmul_strategy* s) {
 struct Weights {
     Owner owner;
     int K = 0, N = 0, k_tile = 0;
-    DeviceBuffer tiled;   // tiled int8, align256(N) x align64(K)
+    DeviceBuffer tiled;   // tiled int8, align256(N) x align256(K)
     DeviceBuffer w_scale; // [N] fp32 (absent for i8i8i32)
 };
 

@@ -82,50 +82,79 @@ uint64_t affinity_mask() {
     return mask ? mask : 1;
 }
 
-// RK_NPU_W4A8_CHAIN_MAX_M: 0..64, default 8, -1 when malformed (reference policy.cpp:25-36)
+// ---- request, resource and strategy rules ---------------------------------------
+// The rules themselves are API contract (reference src/rk_npu_w4a8_tune_policy.cpp:14-79,
+// 140-164: which requests, schedules and cached strategies are acceptable); they are
+// stated here as small predicates over named facts so that a rejected request can be
+// traced to the rule that failed (RK_NPU_W4A8_TUNE_TRACE=1 prints it).
+
+bool trace_rules() {
+    static const bool on = [] {
+        const char* v = std::getenv("RK_NPU_W4A8_TUNE_TRACE");
+        return v && *v && *v != '0';
+    }();
+    return on;
+}
+
+struct Rule {
+    const char* what;
+    bool holds;
+};
+bool all_hold(const char* subject, std::initializer_list<Rule> rules) {
+    for (const Rule& rule : rules)
+        if (!rule.holds) {
+            if (trace_rules()) std::fprintf(stderr, "[rk_npu_w4a8_tune] %s rejected: %s\n", subject, rule.what);
+            return false;
+        }
+    return true;
+}
+
+// Row count up to which a problem may run chained: RK_NPU_W4A8_CHAIN_MAX_M, a decimal
+// number 0..64; 8 when unset; -1 (nothing is valid) for anything else.
 int chain_limit() {
     const char* text = std::getenv("RK_NPU_W4A8_CHAIN_MAX_M");
     if (!text) return 8;
-    if (!*text) return -1;
-    int value = 0;
-    for (const char* p = text; *p; ++p) {
-        if (*p < '0' || *p > '9') return -1;
-        value = value * 10 + (*p - '0');
-        if (value > 64) return -1;
-    }
-    return value;
+    const size_t len = std::strlen(text);
+    if (len == 0 || std::strspn(text, "0123456789") != len) return -1;
+    const char* digits = text + std::strspn(text, "0"); // leading zeros carry no value
+    if (std::strlen(digits) > 2) return -1;             // three significant digits exceed 64
+    const int rows = *digits ? std::atoi(digits) : 0;
+    return rows <= 64 ? rows : -1;
 }
 
-// reference policy.cpp:37-45
 bool valid_config(const rk_npu_w4a8_autotune_config& c) {
-    return c.M > 0 && c.M <= INT_MAX / 2 && c.K > 0 && c.K <= INT32_MAX / 1024 && c.N > 0 && c.N <= INT_MAX - 63 &&
-           (c.activation_type == RK_NPU_W4A8_F32 || c.activation_type == RK_NPU_W4A8_F16) &&
-           !(c.allowed_npu_core_mask & ~7u) && c.warmup >= 0 && c.loops > 0 && c.repeats > 0 && c.timeout_ms &&
-           c.required_k_tile >= 0 && c.required_k_tile <= std::min(2048, align_up_i(c.K, 32)) &&
-           c.required_k_tile % 32 == 0 && std::isfinite(c.k_tile_multiplier) &&
-           (c.k_tile_multiplier == 0 || c.k_tile_multiplier >= 1);
+    const int widest_tile = std::min(2048, align_up_i(std::max(c.K, 0), 32));
+    const double mult = c.k_tile_multiplier;
+    return all_hold("request", {
+        {"1 <= M <= INT_MAX / 2", c.M >= 1 && c.M <= INT_MAX / 2},
+        {"1 <= K <= INT32_MAX / 1024", c.K >= 1 && c.K <= INT32_MAX / 1024},
+        {"1 <= N <= INT_MAX - 63", c.N >= 1 && c.N <= INT_MAX - 63},
+        {"activations are fp32 or fp16", c.activation_type == RK_NPU_W4A8_F32 || c.activation_type == RK_NPU_W4A8_F16},
+        {"NPU core mask within cores 0..2", (c.allowed_npu_core_mask & ~7u) == 0},
+        {"warmup >= 0, loops >= 1, repeats >= 1", c.warmup >= 0 && c.loops >= 1 && c.repeats >= 1},
+        {"timeout set", c.timeout_ms != 0},
+        {"required K tile is 0 or a multiple of 32 up to min(2048, align32(K))",
+         c.required_k_tile >= 0 && c.required_k_tile <= widest_tile && c.required_k_tile % 32 == 0},
+        {"K tile multiplier is 0 (environment) or a finite number >= 1", std::isfinite(mult) && (mult == 0 || mult >= 1)},
+    });
 }
 
-// Config checks + the weight scan (reference policy.cpp:46-70).
+// Request checks, then the scan of the weights.
 int make_profile(const rk_npu_w4a8_autotune_config& c, const int8_t* B, const float* w_scale, W4Profile* out) {
-    if (!valid_config(c) || !B || !w_scale) return RK_NPU_ERR_PARAM;
-    double factor = c.k_tile_multiplier;
-    if (factor == 0) {
-        factor = rkhost::w4a8_env_multiplier();
-        if (factor < 1) return RK_NPU_ERR_PARAM;
-    }
-    W4Profile p;
-    const int rc = rkhost::w4a8_make_profile(c.K, c.N, factor, B, w_scale, &p);
-    if (rc) return rc;
-    if (c.required_k_tile && !p.permits(c.required_k_tile)) return RK_NPU_ERR_PARAM;
-    *out = p;
+    if (!B || !w_scale || !valid_config(c)) return RK_NPU_ERR_PARAM;
+    const double factor = c.k_tile_multiplier != 0 ? c.k_tile_multiplier : rkhost::w4a8_env_multiplier();
+    if (factor < 1) return RK_NPU_ERR_PARAM; // malformed environment value
+    W4Profile scanned;
+    if (const int rc = rkhost::w4a8_make_profile(c.K, c.N, factor, B, w_scale, &scanned)) return rc;
+    if (c.required_k_tile != 0 && !scanned.permits(c.required_k_tile)) return RK_NPU_ERR_PARAM;
+    *out = scanned;
     return RK_NPU_OK;
 }
 
-// Core and CPU sets fixed once from the masks (reference policy.cpp:71-79,
-// src/rk_npu_autotune_common.cpp:46-63): the largest supported NPU core set
-// with no more cores than N has 64-wide groups; up to four permitted CPUs,
-// cores 4..7 first.
+// What a request is tuned on, fixed once from its masks and the process affinity: the NPU
+// core set (the widest of {0,1,2}, {0,1}, {0}, {1}, {2} that the mask allows and that has
+// no more cores than N has 64-column groups), and a team of up to four permitted CPUs,
+// the RK3588's big cores 4..7 ahead of the others.
 struct Resources {
     uint32_t npu = 0;
     uint64_t cpu = 0, allowed_cpu = 0;
@@ -133,66 +162,94 @@ struct Resources {
     int chain_max_m = 8;
 };
 
+uint32_t pick_npu_cores(uint32_t allowed, int N) {
+    static const uint32_t kPreference[] = {7u, 3u, 1u, 2u, 4u};
+    const int column_groups = ceil_div_i(N, 64);
+    for (uint32_t set : kPreference)
+        if ((allowed & set) == set && __builtin_popcount(set) <= column_groups) return set;
+    return 0;
+}
+
 Resources make_resources(const rk_npu_w4a8_autotune_config& c) {
     Resources r;
-    const uint64_t affinity = affinity_mask();
     r.chain_max_m = chain_limit();
     if (r.chain_max_m < 0) return r;
-    r.allowed_cpu = (c.allowed_cpu_core_mask ? c.allowed_cpu_core_mask : affinity) & affinity;
-    std::vector<int> order;
-    for (int cpu = 4; cpu <= 7; ++cpu)
-        if (r.allowed_cpu & (1ull << cpu)) order.push_back(cpu);
-    for (int cpu = 0; cpu < 64; ++cpu)
-        if ((cpu < 4 || cpu > 7) && (r.allowed_cpu & (1ull << cpu))) order.push_back(cpu);
-    r.threads = std::min<int>(4, (int)order.size());
-    for (int i = 0; i < r.threads; ++i) r.cpu |= 1ull << order[(size_t)i];
-    const uint32_t allowed = c.allowed_npu_core_mask ? c.allowed_npu_core_mask : 7u;
-    const int groups = ceil_div_i(c.N, 64);
-    for (uint32_t mask : {7u, 3u, 1u, 2u, 4u})
-        if ((mask & allowed) == mask && __builtin_popcount(mask) <= groups) {
-            r.npu = mask;
-            break;
+    const uint64_t affinity = affinity_mask();
+    r.allowed_cpu = affinity & (c.allowed_cpu_core_mask ? c.allowed_cpu_core_mask : affinity);
+    const uint64_t big = r.allowed_cpu & 0xf0ull;
+    for (uint64_t pool : {big, r.allowed_cpu & ~big}) // each pool in ascending CPU order
+        while (pool && r.threads < 4) {
+            const uint64_t lowest = pool & (~pool + 1);
+            r.cpu |= lowest;
+            pool ^= lowest;
+            ++r.threads;
         }
+    r.npu = pick_npu_cores(c.allowed_npu_core_mask ? c.allowed_npu_core_mask : 7u, c.N);
     return r;
 }
 
-// reference policy.cpp:14-23
-bool valid_cpu_policy(const rk_npu_w4a8_config& c, int maximum_threads, int chain_max_m) {
-    if (maximum_threads < 1 || maximum_threads > 4 || chain_max_m < 0) return false;
-    const bool small = c.M <= std::max(kSmallBatch, chain_max_m);
-    if (c.cpu_threads != maximum_threads && !(small && c.cpu_threads == 1)) return false;
-    if (c.pipeline == RK_NPU_W4A8_CHAIN) return c.M <= chain_max_m && c.K > c.k_tile;
-    return c.pipeline == RK_NPU_W4A8_PIPELINED || (small && c.pipeline == RK_NPU_W4A8_SERIAL);
+// Which CPU team size and submission scheme a strategy may name, given the team the
+// resources provide and the chaining limit.  Problems of few rows may also run on one
+// thread and serially; chaining needs few enough rows and more than one K tile.
+bool schedule_allowed(const rk_npu_w4a8_config& cfg, int team, int chain_rows) {
+    if (team < 1 || team > 4 || chain_rows < 0) return false;
+    const bool few_rows = cfg.M <= std::max(kSmallBatch, chain_rows);
+    bool scheme_ok = false;
+    switch (cfg.pipeline) {
+    case RK_NPU_W4A8_PIPELINED: scheme_ok = true; break;
+    case RK_NPU_W4A8_SERIAL: scheme_ok = few_rows; break;
+    case RK_NPU_W4A8_CHAIN: scheme_ok = cfg.M <= chain_rows && cfg.k_tile < cfg.K; break;
+    default: break;
+    }
+    const bool team_ok = cfg.cpu_threads == team || (few_rows && cfg.cpu_threads == 1);
+    return team_ok && scheme_ok;
 }
 
-// reference policy.cpp:140-148
+// A strategy taken on its own (tuned constructors, before any request is known).
 bool valid_execution(const Strategy& s, bool panel8) {
-    const rk_npu_w4a8_options& o = s.execution;
-    if (!valid_cpu_policy(s.base.config, __builtin_popcountll(s.base.cpu_core_mask), chain_limit()) ||
-        o.struct_size != sizeof(o) || o.reduce_backend != RK_NPU_W4A8_REDUCE_CPU ||
-        (o.input_layout != RK_NPU_W4A8_INPUT_NATIVE && (!panel8 || o.input_layout != RK_NPU_W4A8_INPUT_PANEL8)))
+    const rk_npu_w4a8_options& opt = s.execution;
+    const bool layout_ok = opt.input_layout == RK_NPU_W4A8_INPUT_NATIVE ||
+                           (panel8 && opt.input_layout == RK_NPU_W4A8_INPUT_PANEL8);
+    if (!all_hold("strategy", {
+            {"schedule fits its own CPU mask", schedule_allowed(s.base.config, __builtin_popcountll(s.base.cpu_core_mask), chain_limit())},
+            {"options struct size", opt.struct_size == sizeof(opt)},
+            {"CPU reduction", opt.reduce_backend == RK_NPU_W4A8_REDUCE_CPU},
+            {"input layout", layout_ok},
+        }))
         return false;
-    rk_npu_w4a8_memory_info_ex info{};
-    return rk_npu_w4a8_memory_query_ex(&s.base.config, &o, &info) == RK_NPU_OK;
+    rk_npu_w4a8_memory_info_ex unused{};
+    return rk_npu_w4a8_memory_query_ex(&s.base.config, &opt, &unused) == RK_NPU_OK;
 }
 
-// reference policy.cpp:149-164
+// A strategy against the request, weight profile and resources it claims to answer.
 bool valid_strategy(const Strategy& strategy, const rk_npu_w4a8_autotune_config& c, const W4Profile& p,
                     const Resources& r, bool panel8) {
-    const rk_npu_w4a8_strategy& s = strategy.base;
     if (!valid_execution(strategy, panel8)) return false;
-    const rk_npu_w4a8_config& a = s.config;
-    const rk_npu_w4a8_weight_info& w = s.weights;
-    if (s.tuning_revision != kRevision || s.activation_type != c.activation_type ||
-        s.weight_fingerprint != p.fingerprint || a.M != c.M || a.N != c.N || a.K != c.K || a.npu_core_mask != r.npu ||
-        !valid_cpu_policy(a, r.threads, r.chain_max_m) || s.cpu_core_mask != r.cpu || a.timeout_ms != c.timeout_ms ||
-        !p.permits(a.k_tile) || (c.required_k_tile && a.k_tile != c.required_k_tile) || w.config.K != c.K ||
-        w.config.N != c.N || w.config.k_tile != a.k_tile || w.safe_k_tile != p.safe || w.multiplier != p.multiplier ||
-        w.bound_relaxed != !p.certified(a.k_tile))
-        return false;
-    for (double t : {s.input_us, s.npu_us, s.sync_us, s.output_us, s.total_us, s.jitter_pct, s.robust_us})
-        if (!std::isfinite(t) || t < 0) return false;
-    return true;
+    const rk_npu_w4a8_strategy& s = strategy.base;
+    const rk_npu_w4a8_config& run = s.config;
+    const rk_npu_w4a8_weight_info& wi = s.weights;
+    static double rk_npu_w4a8_strategy::* const kTimes[] = {
+        &rk_npu_w4a8_strategy::input_us, &rk_npu_w4a8_strategy::npu_us,     &rk_npu_w4a8_strategy::sync_us,
+        &rk_npu_w4a8_strategy::output_us, &rk_npu_w4a8_strategy::total_us, &rk_npu_w4a8_strategy::jitter_pct,
+        &rk_npu_w4a8_strategy::robust_us};
+    bool times_ok = true;
+    for (auto field : kTimes) times_ok = times_ok && std::isfinite(s.*field) && s.*field >= 0;
+    return all_hold("strategy", {
+        {"tuning revision", s.tuning_revision == kRevision},
+        {"activation type", s.activation_type == c.activation_type},
+        {"weight fingerprint", s.weight_fingerprint == p.fingerprint},
+        {"shape", run.M == c.M && run.N == c.N && run.K == c.K},
+        {"NPU core set", run.npu_core_mask == r.npu},
+        {"CPU set", s.cpu_core_mask == r.cpu},
+        {"schedule fits the resources", schedule_allowed(run, r.threads, r.chain_max_m)},
+        {"timeout", run.timeout_ms == c.timeout_ms},
+        {"K tile permitted by the weights", p.permits(run.k_tile)},
+        {"K tile is the required one", c.required_k_tile == 0 || run.k_tile == c.required_k_tile},
+        {"weight key", wi.config.K == c.K && wi.config.N == c.N && wi.config.k_tile == run.k_tile},
+        {"weight bound", wi.safe_k_tile == p.safe && wi.multiplier == p.multiplier &&
+                             wi.bound_relaxed == (p.certified(run.k_tile) ? 0 : 1)},
+        {"timings finite and non-negative", times_ok},
+    });
 }
 
 uint64_t double_bits(double d) {

@@ -418,3 +418,19 @@ def test_i4_host_side(lib):
     assert lib.rk_npu_i4i4i32_run(None, None, capi.ptr(B), capi.ptr(B), None) == P
     lib.rk_npu_i4i4i32_weights_free(None)
     lib.rk_npu_i4_workspace_free(None)
+
+
+def test_build_names_the_compiler_it_was_validated_with(tmp_path, capsys):
+    """The inline-assembly load kernels depend on how one hipcc schedules around hand-placed
+    waits: the build records that compiler's version and warns loudly about any other."""
+    from rknpu2_matmul_open_amd import build
+    line = build.check_toolchain(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"))
+    assert line.startswith("HIP version:")
+    quiet = capsys.readouterr().err
+    assert ("WARNING" in quiet) == (not line.startswith(build.VALIDATED_HIPCC))
+    other = tmp_path / "hipcc"
+    other.write_text("#!/bin/sh\necho 'HIP version: 9.9.99999-deadbeef'\n")
+    other.chmod(0o755)
+    assert build.check_toolchain(str(other)) == "HIP version: 9.9.99999-deadbeef"
+    err = capsys.readouterr().err
+    assert "WARNING" in err and "gemm_wk_kernel" in err and build.VALIDATED_HIPCC in err

@@ -31,8 +31,11 @@ def _special_rows(A, as_f16):
 
 # M <= 8 with rows that fit the fused GEMV (one launch), every column width of the kernel
 # (<= 64 / 65..256 / > 256 column blocks), ragged N and K; the last ones do not fit the fused
-# path (rows too long) or have more than 8 rows and take the two-kernel route.
+# path (rows too long) or have more than 8 rows and take the two-kernel route.  (1, 14336, 4096)
+# is the decode shape the benchmark times and (1, 9000, 4100) a ragged neighbour: more than 256
+# column blocks AND several groups of loads per wave, the loop the short-K wide cases never enter.
 W8_SHAPES = [(1, 64, 64), (1, 200, 200), (1, 513, 1000), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520),
+             (1, 14336, 4096), (1, 9000, 4100), (2, 14336, 4096),
              (2, 3000, 700), (3, 65, 33), (4, 9000, 300), (4, 4100, 8000), (8, 128, 4096), (8, 8300, 2000),
              (7, 5000, 4100), (2, 2500, 20003), (16, 300, 500)]
 
@@ -70,6 +73,7 @@ def test_w8a8_dynamic_device(sess, oracle, M, N, K, f16):
 
 
 W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520), (2, 65, 20003),
+             (1, 14336, 4096), (1, 9000, 4100),
              (3, 2500, 1000), (4, 9000, 300), (8, 128, 512), (8, 8200, 2000), (5, 4100, 5000), (12, 200, 300)]
 
 
