@@ -82,6 +82,21 @@ int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* workspace,
                                  const float* input_device, const int32_t* expert_ids_device,
                                  const float* route_weights_device, float* output_device);
 
+/* No counterpart in the reference.  rk_npu_f16i8f16_run_dynamic_device without a workspace
+ * and without any allocation, for callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  The scratch the kernels need (the
+ * quantized rows, their scales, K-split partial tiles) lies in a static device array of
+ * 12 MiB that each GPU the library runs on holds until the process ends; a shape needing more
+ * (roughly align128(M) * align256(K) + 4 * align128(M) + the partial tiles, e.g. M = 2048
+ * with K = 4096 fits, M = 4096 with K = 4096 does not) is rejected with RK_NPU_ERR_NOMEM
+ * before any device work.  Device pointers in and out, work enqueued on the stream of the
+ * context the weights belong to, nothing waited for; results are bit-identical to
+ * rk_npu_f16i8f16_run_dynamic_device.  All calls on one GPU share the one array: calls
+ * through the same context are ordered on its stream, calls that overlap on one GPU through
+ * different contexts race. */
+int rk_npu_f16i8f16_run_dynamic_noalloc_device(const rk_npu_f16i8f16_weights* weights, int M,
+                                               const uint16_t* A_device, uint16_t* C_device);
+
 /* Profiling hooks: launch only the GEMV / GEMM stage of an operator on the
  * activations its workspace quantized during the previous run, so that the
  * dominant kernel can be timed by itself with stream events.  `weights` is a

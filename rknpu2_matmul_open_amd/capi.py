@@ -385,6 +385,7 @@ _PROTOTYPES = {
     "rk_npu_hip_capture_end": (P, [P]),
     "rk_npu_hip_graph_launch": (C.c_int, [P, P]),
     "rk_npu_hip_graph_free": (None, [P]),
+    "rk_npu_f16i8f16_run_dynamic_noalloc_device": (C.c_int, [P, C.c_int, P, P]),
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)

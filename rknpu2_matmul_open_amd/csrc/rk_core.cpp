@@ -216,6 +216,11 @@ rk_npu_ctx* rk_npu_open(const char* dev) {
         return nullptr;
     }
     ctx->id = g_next_ctx_id.fetch_add(1);
+    // (rkh_open made `device` current; a failed lookup only disables the no-allocation entry point)
+    if (rkh_static_scratch(device, &ctx->scratch, &ctx->scratch_bytes)) {
+        ctx->scratch = nullptr;
+        ctx->scratch_bytes = 0;
+    }
     return ctx;
 }
 

@@ -221,6 +221,9 @@ int rkh_capture_end(void* stream, void** graph_exec);
 int rkh_graph_launch(void* graph_exec, void* stream);
 void rkh_graph_destroy(void* graph_exec);
 
+/* ---- static scratch: address and size of the file-scope device array on `device` ---- */
+int rkh_static_scratch(int device, void** ptr, size_t* bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,10 @@ struct rk_npu_ctx {
     int cu_count = 0;
     int clock_khz = 0;
     char arch[64] = {0};
+    // This device's copy of the library's static scratch array (looked up at open; null when
+    // the lookup failed): memory for the entry point that allocates nothing.
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
     struct DomainMemory {
         std::atomic<uint64_t> live_bytes{0}, peak_bytes{0}, creates{0}, destroys{0};
     } memory[RK_NPU_IOMMU_DOMAIN_COUNT];

@@ -23,6 +23,7 @@
 #include <float.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <mutex>
 #include <type_traits>
 
 #include "rk_hip_shim.h"
@@ -2489,6 +2490,13 @@ __global__ __launch_bounds__(512) void mfma_i8_probe_kernel(const v4i* __restric
     if (x == 0x5bd1e995 && sink) atomicAdd(sink, 1);
 }
 
+// ------------------------------------------------- static device scratch
+// Scratch memory for the entry point that allocates nothing: one array per
+// device, held from the moment the code object is loaded until the process
+// ends.  Host code never uses the array's name as an address: the per-device
+// address is looked up once with hipGetSymbolAddress and kept.
+constexpr size_t STATIC_SCRATCH_BYTES = size_t(12) << 20;
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
 
 // ------------------------------------------------------------- launchers
 // Workgroups of the 256-column grid below which the K-split variant is used.  Measured on a 32-expert
@@ -3031,5 +3039,24 @@ void rkh_graph_destroy(void* graph_exec) {
     if (graph_exec) (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
 }
 
+// ---- the static scratch array of `device` ----
+int rkh_static_scratch(int device, void** ptr, size_t* bytes) {
+    static void* address[64] = {};
+    static std::mutex guard;
+    *ptr = nullptr;
+    *bytes = 0;
+    if (device < 0 || device >= 64) return RKH_ERR_RUNTIME;
+    std::lock_guard<std::mutex> lock(guard);
+    if (!address[device]) {
+        RKH_CHECK(hipSetDevice(device));
+        void* p = nullptr;
+        RKH_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return RKH_ERR_RUNTIME;
+        address[device] = p;
+    }
+    *ptr = address[device];
+    *bytes = STATIC_SCRATCH_BYTES;
+    return RKH_OK;
+}
 
 } // extern "C"

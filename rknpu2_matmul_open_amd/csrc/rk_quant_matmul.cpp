@@ -386,6 +386,56 @@ int rk_npu_f16i8f16_run_dynamic_device(rk_npu_matmul_workspace* ws,
                       A, C);
 }
 
+// The f16i8f16 dynamic run without a workspace and without any allocation: the
+// quantized rows, their scales and the K-split partial tiles live in this
+// device's copy of the library's static scratch array instead of workspace
+// buffers (same kernels, same launch plan as rk_npu_f16i8f16_run_dynamic_device).
+// Layout of the scratch for one call, every part on a 256-byte boundary:
+//   [row scales: align128(M) floats][tiled int8 rows][K-split partial tiles]
+// Every call on a device shares that array; calls through one context are
+// ordered on its stream, calls through different contexts of the same device
+// race.  The array keeps the previous call's contents: the padding rows / k of
+// the tiled rows are cleared first (a kernel, not a memset: the call may be
+// recorded by a stream capture) whenever this call's shape has padding.
+int rk_npu_f16i8f16_run_dynamic_noalloc_device(const rk_npu_f16i8f16_weights* weights, int M,
+                                               const uint16_t* A, uint16_t* C) {
+    const Weights* w = reinterpret_cast<const Weights*>(weights);
+    if (!w || !A || !C || M < 1 || !w->w_scale) return RK_NPU_ERR_PARAM;
+    rk_npu_ctx* ctx = w->owner.ctx;
+    if (!ctx->scratch) return RK_NPU_ERR_NOMEM;
+    auto round256 = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t scale_bytes = round256((size_t)rkh_align_up(M, RKH_ROW_ALIGN) * sizeof(float));
+    const size_t tiled_bytes = round256(rkh_tiled_i8_bytes(M, w->K, RKH_ROW_ALIGN));
+    const size_t split_bytes = round256(splitk_scratch_bytes(M, w->N, w->K, false));
+    if (scale_bytes + tiled_bytes + split_bytes > ctx->scratch_bytes) return RK_NPU_ERR_NOMEM;
+    uint8_t* base = static_cast<uint8_t*>(ctx->scratch);
+    rkh_quant_args q{};
+    q.src = A;
+    q.in_dtype = RKH_F16;
+    q.mode = RKH_Q_W8_DYNAMIC;
+    q.M = M;
+    q.K = w->K;
+    q.scale = reinterpret_cast<float*>(base);
+    q.dst = base + scale_bytes;
+    rkh_gemm_args g{};
+    g.A = q.dst;
+    g.W = w->tiled.as<>();
+    g.M = M;
+    g.N = w->N;
+    g.K = w->K;
+    g.a_scale = q.scale;
+    g.w_scale = w->w_scale.as<float>();
+    g.epilogue = RKH_EPI_F16;
+    g.C = C;
+    g.ldc = w->N;
+    g.splitk_acc = split_bytes ? reinterpret_cast<int32_t*>(base + scale_bytes + tiled_bytes) : nullptr;
+    std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    int rc = RKH_OK;
+    if (M % RKH_ROW_ALIGN || w->K % RKH_K_ALIGN) rc = rkh_fill32(ctx->stream, q.dst, 0u, tiled_bytes / 4);
+    if (!rc) rc = rkh_quant_gemm(ctx->stream, &q, &g);
+    return map_error(rc);
+}
+
 /* ---- f32i8f32 ---- */
 rk_npu_f32i8f32_weights* rk_npu_f32i8f32_weights_create(rk_npu_iommu_domain* domain,
                                                         const rk_npu_matmul_weight_config* config,
