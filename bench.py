@@ -1,17 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one pass of the hot path over one batch of seeded synthetic input,
 with inputs and weights already resident in HBM: per-token quantization +
 GEMV / GEMM with the fused dequant epilogue (+ SwiGLU / re-quantize / Down for
 the FFN, + route / combine for the MoE layer), enqueued through the
 device-pointer entry points of the C ABI and timed with HIP events on the
-context's stream.  The default workload is BASELINE config 1 (w8a8 decode GEMV,
-M=1, K=4096, N=14336), reported as weight GB/s; the line also carries the
-int8 TOPS of config 2 (w4a8 prefill GEMM, M=2048) because the headline metric
-names both.
+context's stream (the stream the kernels are launched on).
+
+The headline workload is BASELINE config 1 (w8a8 decode GEMV, M=1, K=4096,
+N=14336), reported as weight GB/s.  The same line carries, under "also", every
+other BASELINE configuration (0, 2, 3, 4) and the int4 decode GEMV, each with
+its own roofline block (bound, dominant kernel, algorithmic bytes / operations,
+fraction of the datasheet peak), a per-kernel breakdown from stream events, and
+under "practical" what a read-only stream and a pure-MFMA loop reach on the box
+at hand -- the ceilings the fractions should be read against.
 
 Prints ONE JSON line.
 """
@@ -28,9 +33,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate
 C1_COPIES = 8                # copies of the decode matrix the timed loop cycles through (8 x 58.7 MB)
 FFN_COPIES = 4               # copies of the FFN weights (4 x 88 MB)
-INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate
+MOE_COPIES = 2               # copies of the expert bank (2 x 201 MB)
 METRIC = "int8 TOPS @M=2048 and GEMV HBM GB/s @M=1 (w8a8/w4a8), % of roofline"
 
 
@@ -48,6 +54,27 @@ def _traffic(kernel_key):
             return json.load(f).get(kernel_key)
     except (OSError, ValueError):
         return None
+
+
+def _hbm(kernel, algo_bytes, us, traffic_key=None, **extra):
+    r = {"bound": "hbm", "kernel": kernel, "achieved": algo_bytes / us / 1e3, "peak": HBM_PEAK_GBS,
+         "unit": "GB/s", "frac": algo_bytes / us / 1e3 / HBM_PEAK_GBS, "time_us": us,
+         "algorithmic_bytes": algo_bytes, "traffic": _traffic(traffic_key) if traffic_key else None}
+    r.update(extra)
+    return r
+
+
+def _mfma(kernel, ops_count, us, traffic_key=None, **extra):
+    r = {"bound": "mfma", "kernel": kernel, "achieved": ops_count / us / 1e6, "peak": INT8_PEAK_TOPS,
+         "unit": "TOP/s", "frac": ops_count / us / 1e6 / INT8_PEAK_TOPS, "time_us": us,
+         "algorithmic_ops": ops_count, "traffic": _traffic(traffic_key) if traffic_key else None}
+    r.update(extra)
+    return r
+
+
+def _kernels(sess, ops, step, calls=20):
+    """Per-kernel times of one step from stream events between the kernels."""
+    return [{"kernel": k, "us": round(us, 3)} for k, us in ops.profile_kernels(sess, step, calls)]
 
 
 def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
@@ -90,11 +117,13 @@ def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
     # quantized) is timed as well for reference.
     sess.spin_up(step)
     step_us = sess.time_us(step, steps, warmup)
-    kernel_us = step_us
     for o in copies:  # every copy's workspace holds quantized activations for the plain GEMV
         o.run_device(dA, dC)
     gemv_only_us = sess.time_us(gemv_only, max(steps, 50), warmup)
     same_matrix_us = sess.time_us(step_same_matrix, steps, warmup)
+    # the same eight launches recorded once and replayed as a graph: what the step costs when
+    # the host's per-launch submission is out of the picture
+    graph_us = graph_step_us(sess, step, C1_COPIES, max(steps // C1_COPIES, 5))
     step_same_matrix()
     got = sess.from_device(dC, (M, N), np.uint16)
     weight_bytes = K * N
@@ -108,13 +137,9 @@ def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
         "config": {"workload": "c1: w8a8 decode GEMV M=1 K=4096 N=14336, fp16 in/out, seeds 2/3",
                    "value_is": "int8 weight bytes (58720256) / step time; step = one fused quantize+GEMV kernel; "
                                "the loop cycles through %d copies of the matrix so that every step reads HBM" % C1_COPIES},
-        "roofline": {"bound": "hbm", "kernel": "gemv_wide8_kernel<1> (fused per-token quantize + GEMV)",
-                     "achieved": algo_bytes / kernel_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": algo_bytes / kernel_us / 1e3 / HBM_PEAK_GBS,
-                     "kernel_us": kernel_us, "algorithmic_bytes": algo_bytes,
-                     "gemv_without_quantize_us": gemv_only_us,
-                     "same_matrix_every_step_us": same_matrix_us,
-                     "traffic": _traffic("gemv_c1")},
+        "roofline": _hbm("gemv_wide8_kernel<1> (fused per-token quantize + GEMV)", algo_bytes, step_us, "gemv_c1",
+                         kernel_us=step_us, gemv_without_quantize_us=gemv_only_us,
+                         same_matrix_every_step_us=same_matrix_us, replayed_from_graph_us=graph_us),
     }
     if cpu_baseline:
         from oracle import binding as orc
@@ -137,7 +162,26 @@ def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
     return out
 
 
-def bench_c2(sess, ops, capi, workloads, steps, warmup):
+def graph_step_us(sess, step, steps_in_graph, replays):
+    """Average time of one step when `steps_in_graph` of them are captured once and replayed."""
+    lib = sess.lib
+    for _ in range(steps_in_graph):
+        step()
+    if sess.sync():
+        raise RuntimeError("sync")
+    if lib.rk_npu_hip_capture_begin(sess.ctx):
+        raise RuntimeError("capture_begin")
+    for _ in range(steps_in_graph):
+        step()
+    g = lib.rk_npu_hip_capture_end(sess.ctx)
+    if not g:
+        raise RuntimeError("capture_end")
+    us = sess.time_us(lambda: lib.rk_npu_hip_graph_launch(sess.ctx, g), replays, 3) / steps_in_graph
+    lib.rk_npu_hip_graph_free(g)
+    return us
+
+
+def bench_c2(sess, ops, capi, workloads, steps, warmup, want_mfma_probe=True):
     """w4a8 prefill GEMM, M=2048, K=4096, N=4096."""
     c = workloads.CONFIGS[2]()
     M, K, N = c["M"], c["K"], c["N"]
@@ -163,15 +207,60 @@ def bench_c2(sess, ops, capi, workloads, steps, warmup):
     ops_count = 2.0 * M * K * N
     out = {"workload": "c2: w4a8 prefill GEMM M=2048 K=4096 N=4096, fp16 in/out, seeds 4/5",
            "tops": ops_count / step_us / 1e6, "ms_per_step": step_us / 1e3,
-           "roofline": {"bound": "mfma", "kernel": "gemm_wk_kernel<int4,f16> (128x256 tile, waves split K)",
-                        "achieved": ops_count / kernel_us / 1e6, "peak": INT8_PEAK_TOPS,
-                        "unit": "TOP/s", "frac": ops_count / kernel_us / 1e6 / INT8_PEAK_TOPS,
-                        "kernel_us": kernel_us, "traffic": _traffic("gemm_c2")}}
+           "step_frac_of_int8_peak": ops_count / step_us / 1e6 / INT8_PEAK_TOPS,
+           "roofline": _mfma("gemm_wk_kernel<int4,f16> (128x256 tile, waves split K)", ops_count, kernel_us,
+                             "gemm_c2", kernel_us=kernel_us),
+           "kernels": _kernels(sess, ops, step)}
+    if want_mfma_probe:
+        # the pure-MFMA loop on operands with this workload's bit patterns: int4 codes carried as
+        # 16 * code (weights, first operand) and the int8 codes of the quantized rows (second)
+        q, _ = ws.read_quantized()
+        wbytes = (c["B"].T.reshape(-1)[:16384].astype(np.int16) * 16).astype(np.int8)
+        abytes = q.reshape(-1)[:16384]
+        operands = np.concatenate([wbytes[:8192], abytes[:8192], wbytes[8192:], abytes[8192:]])
+        out["roofline"]["practical_peak"] = mfma_probe(sess, operands)
+        out["roofline"]["frac_of_practical_peak"] = out["roofline"]["achieved"] / out["roofline"]["practical_peak"]
     sess.free_device(dA)
     sess.free_device(dC)
     ws.close()
     w.close()
     return out
+
+
+def mfma_probe(sess, operands_i8, iterations=2000):
+    """TOP/s of the library's pure int8 MFMA loop on the given 32 KiB of operands."""
+    lib = sess.lib
+    d = sess.to_device(np.ascontiguousarray(operands_i8, np.int8))
+    count = C.c_double(0)
+
+    def run():
+        if lib.rk_npu_hip_probe_mfma_i8(sess.ctx, d, iterations, C.byref(count)):
+            raise RuntimeError("probe_mfma")
+
+    sess.spin_up(run, 0.02)
+    us = sess.time_us(run, 20, 3)
+    sess.free_device(d)
+    return count.value / us / 1e6
+
+
+def read_probe(sess, bytes_per_launch, span, footprint=C1_COPIES * 58720256, iters=200):
+    """GB/s of the library's read-only stream, `bytes_per_launch` per launch, rotating over
+    `footprint` bytes so that no launch finds its data in the memory-side cache."""
+    lib = sess.lib
+    pieces = max(footprint // bytes_per_launch, 1)
+    buf = sess.empty_device(pieces * bytes_per_launch)
+    base = buf if isinstance(buf, int) else buf.value
+    turn = [0]
+
+    def run():
+        at = base + (turn[0] % pieces) * bytes_per_launch
+        turn[0] += 1
+        if lib.rk_npu_hip_probe_stream_read(sess.ctx, C.c_void_p(at), bytes_per_launch, span):
+            raise RuntimeError("probe_stream_read")
+
+    us = sess.time_us(run, iters, 20)
+    sess.free_device(buf)
+    return {"GBps": bytes_per_launch / us / 1e3, "us_per_launch": us, "bytes_per_launch": bytes_per_launch}
 
 
 def bench_c1w4(sess, ops, capi, workloads, steps, warmup):
@@ -200,10 +289,8 @@ def bench_c1w4(sess, ops, capi, workloads, steps, warmup):
     algo_bytes = weight_bytes + K * 2 + N * 2 + N * 4
     out = {"workload": "w4a8 decode GEMV M=1 K=4096 N=14336 (int4 weights, 29360128 B), fp16 in/out, seeds 2/3",
            "weight_GBps": weight_bytes / step_us / 1e3, "ms_per_step": step_us / 1e3,
-           "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1,true,1,32> (fused per-token quantize + int4 GEMV)",
-                        "achieved": algo_bytes / step_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": algo_bytes / step_us / 1e3 / HBM_PEAK_GBS, "kernel_us": step_us,
-                        "algorithmic_bytes": algo_bytes, "traffic": None}}
+           "roofline": _hbm("gemv_kernel<1,true,1,32> (fused per-token quantize + int4 GEMV)", algo_bytes, step_us,
+                            "gemv_c1w4", kernel_us=step_us)}
     sess.free_device(dA)
     sess.free_device(dC)
     ws.close()
@@ -237,10 +324,8 @@ def bench_c2w8(sess, ops, capi, workloads, steps, warmup):
     ops_count = 2.0 * M * K * N
     out = {"workload": "w8a8 prefill GEMM M=2048 K=4096 N=4096, fp16 in/out, seeds 4/5",
            "tops": ops_count / step_us / 1e6, "ms_per_step": step_us / 1e3,
-           "roofline": {"bound": "mfma", "kernel": "gemm_wk_kernel<int8,f16> (128x256 tile, waves split K)",
-                        "achieved": ops_count / kernel_us / 1e6, "peak": INT8_PEAK_TOPS,
-                        "unit": "TOP/s", "frac": ops_count / kernel_us / 1e6 / INT8_PEAK_TOPS,
-                        "kernel_us": kernel_us, "traffic": None}}
+           "roofline": _mfma("gemm_wk_kernel<int8,f16> (128x256 tile, waves split K)", ops_count, kernel_us,
+                             kernel_us=kernel_us)}
     sess.free_device(dA)
     sess.free_device(dC)
     op.close()
@@ -270,10 +355,18 @@ def bench_c3(sess, ops, capi, workloads, steps, warmup):
     sess.spin_up(step)
     step_us = sess.time_us(step, steps, warmup)
     ops_count = 2.0 * M * H * 2 * I + 2.0 * M * I * H
-    weight_bytes = (H * 2 * I + I * H) / 2
-    out = {"workload": "c3: fused w4a8 FFN M=128 H=4096 I=14336, seeds 6-9",
+    weight_bytes = (H * 2 * I + I * H) // 2
+    # weights once + x in + fp32 middle written and read back (it is an output of the call and
+    # the input of the re-quantization) + out + both scale vectors
+    algo_bytes = weight_bytes + M * H * 4 + 2 * M * I * 4 + M * H * 4 + (2 * I + H) * 4
+    out = {"workload": "c3: fused w4a8 FFN M=128 H=4096 I=14336 (fp32 in / middle / out), seeds 6-9; the loop cycles "
+                       "through %d copies of the 88 MB of weights" % FFN_COPIES,
            "tops": ops_count / step_us / 1e6, "weight_GBps": weight_bytes / step_us / 1e3,
-           "ms_per_step": step_us / 1e3}
+           "ms_per_step": step_us / 1e3,
+           "roofline": _hbm("whole step; dominant: gemm_wk_kernel<int4,SwiGLU> (gate/up, 58.7 MB of weights)",
+                            algo_bytes, step_us, "ffn_c3", frac_of_int8_peak=ops_count / step_us / 1e6 / INT8_PEAK_TOPS,
+                            algorithmic_ops=ops_count),
+           "kernels": _kernels(sess, ops, step)}
     for d in (dA, dmid, dC):
         sess.free_device(d)
     for o in [gws, dws] + gws_ + dws_:
@@ -284,12 +377,17 @@ def bench_c3(sess, ops, capi, workloads, steps, warmup):
 def bench_c4(sess, ops, capi, workloads, steps, warmup):
     """w8a8 MoE layer, 256 tokens, hidden 2048, 32 experts, top-4, intermediate 1024."""
     c = workloads.CONFIGS[4]()
-    moe = ops.MoeW8(sess, c["H"], c["I"], c["E"], 0, c["top_k"], 256, c["experts"])
+    # the loop alternates between MOE_COPIES banks (403 MB) so that the experts come from HBM
+    banks = [ops.MoeW8(sess, c["H"], c["I"], c["E"], 0, c["top_k"], 256, c["experts"]) for _ in range(MOE_COPIES)]
+    moe = banks[0]
     dx, dids, drt = sess.to_device(c["x"]), sess.to_device(c["ids"]), sess.to_device(c["routes"])
     dout = sess.empty_device(c["T"] * c["H"] * 4)
+    turn = [0]
 
     def step():
-        rc = sess.lib.rk_npu_moe_w8_run_f32_device(moe.ws, moe.w, c["T"], dx, dids, drt, dout)
+        bank = banks[turn[0] % MOE_COPIES]
+        turn[0] += 1
+        rc = sess.lib.rk_npu_moe_w8_run_f32_device(moe.ws, bank.w, c["T"], dx, dids, drt, dout)
         if rc:
             raise RuntimeError("moe rc=%d" % rc)
 
@@ -298,12 +396,20 @@ def bench_c4(sess, ops, capi, workloads, steps, warmup):
     assignments = int((c["routes"] != 0).sum())
     ops_count = assignments * (2.0 * c["H"] * 2 * c["I"] + 2.0 * c["I"] * c["H"])
     weight_bytes = c["E"] * 3 * c["H"] * c["I"]
-    out = {"workload": "c4: w8a8 MoE T=256 H=2048 E=32 top-4 I=1024, seeds 10-14",
+    # every expert's weights once + fp32 tokens in + fp32 result out + routing table + scales
+    algo_bytes = (weight_bytes + 2 * c["T"] * c["H"] * 4 + 2 * c["T"] * c["top_k"] * 4 +
+                  c["E"] * (2 * c["I"] + c["H"]) * 4)
+    out = {"workload": "c4: w8a8 MoE T=256 H=2048 E=32 top-4 I=1024 (fp32 in / out), seeds 10-14; the loop "
+                       "alternates between %d copies of the 201 MB expert bank" % MOE_COPIES,
            "tops": ops_count / step_us / 1e6, "weight_GBps": weight_bytes / step_us / 1e3,
-           "ms_per_step": step_us / 1e3}
+           "ms_per_step": step_us / 1e3,
+           "roofline": _hbm("whole step; dominant: gemm_stream_kernel<SwiGLU> (grouped gate/up, 134 MB of expert weights)",
+                            algo_bytes, step_us, "moe_c4", algorithmic_ops=ops_count),
+           "kernels": _kernels(sess, ops, step)}
     for d in (dx, dids, drt, dout):
         sess.free_device(d)
-    moe.close()
+    for b in banks:
+        b.close()
     return out
 
 
@@ -313,10 +419,22 @@ def bench_c0(sess, ops, capi, workloads, steps, warmup):
     op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
     dA = sess.to_device(c["A"])
     dC = sess.empty_device(M * N * 2)
-    sess.spin_up(lambda: op.run_device(dA, dC))
-    step_us = sess.time_us(lambda: op.run_device(dA, dC), steps, warmup)
-    out = {"workload": "c0: w8a8 GEMM M=64 K=2048 N=2048", "tops": 2.0 * M * K * N / step_us / 1e6,
-           "weight_GBps": K * N / step_us / 1e3, "ms_per_step": step_us / 1e3}
+
+    def step():
+        rc = op.run_device(dA, dC)
+        if rc:
+            raise RuntimeError("run_device rc=%d" % rc)
+
+    sess.spin_up(step)
+    step_us = sess.time_us(step, steps, warmup)
+    ops_count = 2.0 * M * K * N
+    algo_bytes = K * N + M * K * 2 + M * N * 2 + N * 4 + M * 4
+    out = {"workload": "c0: w8a8 GEMM M=64 K=2048 N=2048, fp16 in/out, seeds 0/1 (4.7 MB and 0.54 GOP: bound by launch "
+                       "latency; the weights stay in the memory-side cache)",
+           "tops": ops_count / step_us / 1e6, "weight_GBps": K * N / step_us / 1e3, "ms_per_step": step_us / 1e3,
+           "roofline": _hbm("whole step; dominant: gemm_stream_kernel<KS=4> (64-column tiles, K split over the waves)",
+                            algo_bytes, step_us, algorithmic_ops=ops_count),
+           "kernels": _kernels(sess, ops, step)}
     sess.free_device(dA)
     sess.free_device(dC)
     op.close()
@@ -335,15 +453,33 @@ def bench_copy(sess, steps):
             "GBps_read_plus_write": 2 * nbytes / us / 1e3}
 
 
+def practical_ceilings(sess):
+    """What the box at hand gives with no arithmetic in the way (see include/rk_npu_hip.h):
+    read-only streams in the decode GEMV's access order at the footprints of the HBM-bound
+    configurations, and the pure int8 MFMA loop on random int8 operands."""
+    rng = np.random.default_rng(0)
+    return {
+        "hbm_read_58MB_per_launch": read_probe(sess, 58720256, 131072),
+        "hbm_read_29MB_per_launch": read_probe(sess, 29360128, 65536),
+        "hbm_read_470MB_per_launch": read_probe(sess, C1_COPIES * 58720256, 131072, iters=20),
+        "mfma_int8_random_operands_TOPS": mfma_probe(sess, rng.integers(-127, 128, 32768).astype(np.int8)),
+        "mfma_int8_zero_operands_TOPS": mfma_probe(sess, np.zeros(32768, np.int8)),
+        "note": "read-only stream (16 B per lane, 8 loads per wave in flight, one workgroup per 128 / 64 KiB span, "
+                "rotating over 470 MB) and pure v_mfma_i32_32x32x32_i8 loop (8 waves per CU, operands in registers); "
+                "launch gaps included, as in every figure of this line",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c1", choices=["c1", "all"],
-                    help="c1: headline line (+ c2 TOPS); all: also time configs 0, 3 and 4")
+    ap.add_argument("--workload", default="all", choices=["c1", "all"],
+                    help="all: the headline line with every BASELINE configuration under \"also\" (default); "
+                         "c1: config 1, config 2 and the int4 GEMV only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default=None, choices=["c0", "c1", "c1w4", "c2", "c2w8", "c3", "c4", "copy"],
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c1w4", "c2", "c2w8", "c3", "c4", "copy", "probes"],
                     help="profiling aid: run one configuration's loop only")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -360,6 +496,10 @@ def main():
         print(json.dumps(bench_copy(sess, min(args.steps, 10))))
         sess.close()
         return
+    if args.only == "probes":
+        print(json.dumps(practical_ceilings(sess)))
+        sess.close()
+        return
     if args.only:
         fn = {"c0": bench_c0, "c1w4": bench_c1w4, "c2": bench_c2, "c2w8": bench_c2w8, "c3": bench_c3, "c4": bench_c4}.get(args.only)
         res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)
@@ -371,16 +511,27 @@ def main():
     # GPU measurements first, back to back; the CPU baseline (about 10 s during
     # which the device idles and clocks down) runs last, inside bench_c1.
     log("config 2 (prefill GEMM)")
-    r2 = bench_c2(sess, ops, capi, workloads, args.steps, args.warmup)
-    also = {"c2": r2}
+    also = {"c2": bench_c2(sess, ops, capi, workloads, args.steps, args.warmup)}
     log("w4a8 decode GEMV")
     also["c1w4"] = bench_c1w4(sess, ops, capi, workloads, args.steps, args.warmup)
     if args.workload == "all":
-        for name, fn in (("c2w8", bench_c2w8), ("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
+        for name, fn in (("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
             log("config %s" % name)
             also[name] = fn(sess, ops, capi, workloads, args.steps, args.warmup)
+    log("practical ceilings (read-only stream, pure MFMA loop)")
+    practical = practical_ceilings(sess)
     log("config 1 (decode GEMV)")
     r1 = bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, not args.no_cpu_baseline)
+    r1["roofline"]["practical_peak"] = practical["hbm_read_58MB_per_launch"]["GBps"]
+    r1["roofline"]["frac_of_practical_peak"] = r1["roofline"]["achieved"] / r1["roofline"]["practical_peak"]
+    w4 = also["c1w4"]["roofline"]
+    w4["practical_peak"] = practical["hbm_read_29MB_per_launch"]["GBps"]
+    w4["frac_of_practical_peak"] = w4["achieved"] / w4["practical_peak"]
+    for name in ("c3", "c4"):
+        if name in also:
+            r = also[name]["roofline"]
+            r["practical_peak"] = practical["hbm_read_470MB_per_launch"]["GBps"]
+            r["frac_of_practical_peak"] = r["achieved"] / r["practical_peak"]
     line = {
         "metric": METRIC, "value": r1["value"], "unit": r1["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": r1["ms_per_step"],
@@ -388,6 +539,7 @@ def main():
         "data": "synthetic (seeded numpy PCG64; weights N(0,0.02) quantized per channel, activations fp16 N(0,1))",
         "config": r1["config"], "roofline": r1["roofline"],
         "device": {"arch": arch, "compute_units": cus, "clock_mhz": khz // 1000},
+        "practical": practical,
         "also": also,
     }
     if "cpu_baseline" in r1:

@@ -124,15 +124,28 @@ int rk_npu_w4a8_run_i32(rk_npu_w4a8_workspace* workspace, const rk_npu_w4a8_weig
 /* Measurement probes: what the memory system and the matrix pipes of the box at hand give,
  * to put beside the datasheet peaks.  Each call enqueues ONE kernel on the context's stream
  * (time it with the events above):
- *   - a read-only pass over [src_device, src_device + bytes), 16 bytes per lane, every wave
- *     slot of the chip issuing loads;
+ *   - a read-only pass over [src_device, src_device + bytes) in the decode GEMV's access
+ *     order: one workgroup of eight waves per `span` bytes (a multiple of 1024; 131072 is the
+ *     column block of a K = 4096 int8 matrix), 1 KiB pieces interleaved over the waves, 16
+ *     bytes per lane, eight loads per wave in flight;
  *   - a pure int8 MFMA loop (v_mfma_i32_32x32x32_i8, eight waves per compute unit, four
  *     independent accumulators per wave, operands in registers, no memory traffic) on the
  *     32 KiB at operands_device -- the clock the chip sustains depends on the operands' bit
  *     patterns, so pass data like the workload's; *ops receives the operation count
  *     (2 * 32 * 32 * 32 per MFMA). */
-int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes);
+int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes, size_t span);
 int rk_npu_hip_probe_mfma_i8(rk_npu_ctx* ctx, const void* operands_device, int iterations, double* ops);
+
+/* Per-kernel profile of the *_device calls: between profile_begin and profile_end a stream
+ * event is recorded in front of every kernel the library launches on this context's stream.
+ * profile_end waits for the stream and returns the number of kernels seen (or a negative
+ * RK_NPU_ERR_*): us[i] is the time from the event in front of kernel i to the event in front
+ * of kernel i + 1 (the last one: to the end of the work), i.e. the kernel plus the launch
+ * gap behind it; names receives the kernels' names, one per line, as many as fit.  One
+ * context at a time (RK_NPU_ERR_BUSY otherwise).  The events between the kernels cost a
+ * little themselves: time whole steps without the profile. */
+int rk_npu_hip_profile_begin(rk_npu_ctx* ctx);
+int rk_npu_hip_profile_end(rk_npu_ctx* ctx, char* names, size_t names_bytes, double* us, int capacity);
 
 /* Stream capture: the *_device calls made between capture_begin and capture_end on this
  * context (from the calling thread) are recorded instead of executed -- they only launch

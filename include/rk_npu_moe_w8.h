@@ -122,9 +122,11 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
  * Expert tensors are passed exactly as for the W8 factories (one int8_t per
  * weight, the same scale vectors); an INT4 expert's codes must lie in [-8, 7].
  * On the RK3588 these formats select the NPU's int4 mode, K-sliced INT16
- * partials and their certificates; here an INT4 code is an int8 value, the
- * int8 MFMA path accumulates it in int32 without any intermediate narrowing,
- * and results are bit-identical to the W8 path given the same codes.  What is
+ * partials and their certificates; here INT4 experts are held and streamed as
+ * packed nibbles (half the bytes of a W8 expert, as
+ * rk_npu_moe_w8_weights_device_bytes reports), unpacked in registers to int8
+ * MFMA operands and accumulated in int32 without any intermediate narrowing,
+ * so results are bit-identical to the W8 path given the same codes.  What is
  * kept from the reference is the contract: geometry (hidden and intermediate
  * multiples of 64, hidden <= 8128), code range validation, native_input = 0,
  * and that weights only bind to a workspace made by the factory of the same
@@ -144,9 +146,12 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
  *
  * Packed record of one INT4 expert, rk_npu_moe_quant_expert_blob_bytes() bytes
  * (0 for W8 handles): {u32 magic "RKHM", u32 RK_NPU_MOE_QUANT_BLOB_VERSION,
- * u32 hidden, u32 intermediate}, the gate/up image and the down image in this
- * library's execution layout, 2*intermediate gate/up scales, hidden down
- * scales.  Records are native to this library (not interchangeable with the
+ * u32 hidden, u32 intermediate}, the gate/up image (align256(2*intermediate) *
+ * align256(hidden) / 2 bytes) and the down image (align256(hidden) *
+ * align256(intermediate) / 2 bytes) in this library's execution layout -- 1 KiB
+ * tiles of 32 columns x 64 k, two codes per byte, gate/up column blocks
+ * interleaved --, 2*intermediate gate/up scales, hidden down scales (fp32,
+ * little endian).  Records are native to this library (not interchangeable with the
  * RK3588 build's) and identical between the all-INT4 and the mixed bank of one
  * geometry.  export / import accept a larger buffer than the record, reject a
  * shorter one, a W8 handle, the shared int8 expert, an out-of-range slot, a

@@ -379,8 +379,10 @@ _PROTOTYPES = {
     "rk_npu_w4a8_workspace_read_quantized": (C.c_int, [P, P, P]),
     "rk_npu_w4a8_run_i32": (C.c_int, [P, P, P, P]),
     "rk_npu_hip_fail_alloc_after": (None, [C.c_int]),
-    "rk_npu_hip_probe_stream_read": (C.c_int, [P, P, C.c_size_t]),
+    "rk_npu_hip_probe_stream_read": (C.c_int, [P, P, C.c_size_t, C.c_size_t]),
     "rk_npu_hip_probe_mfma_i8": (C.c_int, [P, P, C.c_int, C.POINTER(C.c_double)]),
+    "rk_npu_hip_profile_begin": (C.c_int, [P]),
+    "rk_npu_hip_profile_end": (C.c_int, [P, C.c_char_p, C.c_size_t, C.POINTER(C.c_double), C.c_int]),
     "rk_npu_hip_capture_begin": (C.c_int, [P]),
     "rk_npu_hip_capture_end": (P, [P]),
     "rk_npu_hip_graph_launch": (C.c_int, [P, P]),

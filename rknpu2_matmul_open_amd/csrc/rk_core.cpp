@@ -360,11 +360,10 @@ int rk_npu_hip_event_elapsed_us(rk_npu_hip_event* start, rk_npu_hip_event* stop,
 void rk_npu_hip_fail_alloc_after(int n) { rkh_fail_malloc_after(n); }
 
 /* ---- measurement probes ---- */
-int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes) {
-    if (!ctx || !src_device || bytes < 16) return RK_NPU_ERR_PARAM;
+int rk_npu_hip_probe_stream_read(rk_npu_ctx* ctx, const void* src_device, size_t bytes, size_t span) {
+    if (!ctx || !src_device || bytes < 16 || span < 1024 || span % 1024) return RK_NPU_ERR_PARAM;
     std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-    // eight workgroups of 512 lanes per compute unit: every wave slot of the chip issues loads
-    return rkhost::map_error(rkh_probe_stream_read(ctx->stream, src_device, bytes, ctx->cu_count * 8, nullptr));
+    return rkhost::map_error(rkh_probe_stream_read(ctx->stream, src_device, bytes, span, nullptr));
 }
 int rk_npu_hip_probe_mfma_i8(rk_npu_ctx* ctx, const void* operands_device, int iterations, double* ops) {
     if (!ctx || !operands_device || iterations < 1) return RK_NPU_ERR_PARAM;
@@ -372,6 +371,78 @@ int rk_npu_hip_probe_mfma_i8(rk_npu_ctx* ctx, const void* operands_device, int i
     if (ops) *ops = (double)workgroups * 8.0 * iterations * 4.0 * 2.0 * 32 * 32 * 32;
     std::lock_guard<std::mutex> submit(ctx->submit_mutex);
     return rkhost::map_error(rkh_probe_mfma_i8(ctx->stream, operands_device, workgroups, iterations, nullptr));
+}
+
+/* ---- per-kernel profile ---- */
+namespace {
+std::mutex g_profile_owner_mutex;
+rk_npu_ctx* g_profile_owner = nullptr; // the marker is process-wide: one context profiles at a time
+
+void profile_marker(void* user, void* stream, const char* kernel) {
+    rk_npu_ctx* ctx = static_cast<rk_npu_ctx*>(user);
+    if (stream != ctx->stream) return;
+    std::lock_guard<std::mutex> lock(ctx->profile_mutex);
+    if (!ctx->profiling) return;
+    void* event = nullptr;
+    if (rkh_event_create(&event)) return;
+    rkh_event_record(event, stream);
+    ctx->profile_marks.push_back({kernel, event});
+}
+} // namespace
+
+int rk_npu_hip_profile_begin(rk_npu_ctx* ctx) {
+    if (!ctx) return RK_NPU_ERR_PARAM;
+    std::lock_guard<std::mutex> owner(g_profile_owner_mutex);
+    if (g_profile_owner) return RK_NPU_ERR_BUSY;
+    g_profile_owner = ctx;
+    {
+        std::lock_guard<std::mutex> lock(ctx->profile_mutex);
+        ctx->profiling = true;
+    }
+    rkh_set_marker(profile_marker, ctx);
+    return RK_NPU_OK;
+}
+
+int rk_npu_hip_profile_end(rk_npu_ctx* ctx, char* names, size_t names_bytes, double* us, int capacity) {
+    if (!ctx || capacity < 0 || (capacity > 0 && !us)) return RK_NPU_ERR_PARAM;
+    {
+        std::lock_guard<std::mutex> owner(g_profile_owner_mutex);
+        if (g_profile_owner != ctx) return RK_NPU_ERR_PARAM;
+        rkh_set_marker(nullptr, nullptr);
+        g_profile_owner = nullptr;
+    }
+    std::vector<rk_npu_ctx::ProfileMark> marks;
+    {
+        std::lock_guard<std::mutex> lock(ctx->profile_mutex);
+        ctx->profiling = false;
+        marks.swap(ctx->profile_marks);
+    }
+    void* last = nullptr;
+    int rc = rkh_event_create(&last);
+    if (!rc) rc = rkh_event_record(last, ctx->stream);
+    if (!rc) rc = rkh_sync(ctx->stream);
+    int count = 0;
+    size_t used = 0;
+    if (names && names_bytes) names[0] = 0;
+    for (size_t i = 0; i < marks.size() && !rc; ++i) {
+        if (count >= capacity) break;
+        void* next = i + 1 < marks.size() ? marks[i + 1].event : last;
+        double span = 0.0;
+        rc = rkh_event_elapsed_us(marks[i].event, next, &span);
+        us[count++] = span;
+        if (names) { // newline-separated kernel names, as many as fit
+            const size_t len = std::strlen(marks[i].kernel);
+            if (used + len + 2 <= names_bytes) {
+                std::memcpy(names + used, marks[i].kernel, len);
+                names[used + len] = '\n';
+                used += len + 1;
+                names[used] = 0;
+            }
+        }
+    }
+    for (auto& m : marks) rkh_event_destroy(m.event);
+    rkh_event_destroy(last);
+    return rc ? RK_NPU_ERR_SUBMIT : count;
 }
 
 /* ---- stream capture ---- */

@@ -160,6 +160,13 @@ typedef struct rkh_gemm_args {
     int max_blocks;
     size_t w_expert_stride;  /* bytes between experts in W                        */
     size_t ws_expert_stride; /* floats between experts in w_scale                 */
+    /* Grouped mode, expert formats: experts below int4_experts are tiled int4 images in W4
+     * (expert e at e * w4_expert_stride), the others tiled int8 images in W (expert e at
+     * (e - int4_experts) * w_expert_stride; W may be NULL when there is none).  A bank that
+     * holds both formats takes one launch per format; w_int4 is not used in grouped mode. */
+    const uint8_t* W4;
+    int int4_experts;
+    size_t w4_expert_stride;
 } rkh_gemm_args;
 int rkh_gemm(void* stream, const rkh_gemm_args* args);
 /* quantize + GEMM as one request: for decode-sized M the quantization is fused
@@ -209,11 +216,19 @@ int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args);
 
 
 /* ---- measurement probes (practical ceilings beside the datasheet peaks) ---- */
-/* One read-only pass over [src, src + bytes) with `workgroups` workgroups of 512 lanes. */
-int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, int workgroups, void* sink);
+/* One read-only pass over [src, src + bytes): a workgroup of 512 lanes per `span` bytes
+ * (a multiple of 1024), pieces of 1 KiB interleaved over its eight waves. */
+int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, size_t span, void* sink);
 /* `workgroups` x 8 waves x `iterations` x 4 int8 MFMAs (32x32x32) on operands read once from
  * `operands` (32 KiB: 4 x 512 lanes x 16 bytes). */
 int rkh_probe_mfma_i8(void* stream, const void* operands, int workgroups, int iterations, void* sink);
+
+/* ---- stage marker ----
+ * While a marker is set, it is called with the kernel's name right before every kernel this
+ * shim launches (on the launching thread, with the stream of the launch).  Process-wide;
+ * NULL switches it off.  For per-kernel timing of multi-kernel steps with stream events. */
+typedef void (*rkh_marker_fn)(void* user, void* stream, const char* kernel);
+void rkh_set_marker(rkh_marker_fn fn, void* user);
 
 /* ---- stream capture ---- */
 int rkh_capture_begin(void* stream);

@@ -34,6 +34,15 @@ struct rk_npu_ctx {
     // Device work of one context is issued on one stream; submissions from
     // different workspaces are serialised here so stream order == call order.
     std::mutex submit_mutex;
+    // Per-kernel profile (rk_npu_hip_profile_begin / _end): one stream event in front of every
+    // kernel launched on this context's stream while it is on.
+    struct ProfileMark {
+        const char* kernel;
+        void* event;
+    };
+    std::mutex profile_mutex;
+    bool profiling = false;
+    std::vector<ProfileMark> profile_marks;
     // Rejected-input flags of workspaces used through the *_device entry
     // points since the last rk_npu_hip_sync().
     std::mutex pending_mutex;

@@ -41,6 +41,15 @@ namespace {
                                                                : RKH_ERR_RUNTIME; \
     } while (0)
 
+// Stage marker (see rkh_set_marker): told the name of every kernel launched through this
+// file just before the launch, so that a caller can put stream events between the kernels
+// of a multi-kernel step.  Null unless a caller is profiling.
+rkh_marker_fn g_marker = nullptr;
+void* g_marker_user = nullptr;
+inline void mark(hipStream_t stream, const char* kernel) {
+    if (g_marker) g_marker(g_marker_user, stream, kernel);
+}
+
 // Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(<N-1>{}).
 template <int N, int I = 0, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -232,12 +241,19 @@ __device__ __forceinline__ size_t tiled_chunk_offset(int row, int c, int KB) {
     return ((size_t)(row >> 5) * KB + kb) * 1024 + (size_t)((row & 31) + 32 * half) * 16;
 }
 
-// 16 quantized codes into the tiled matrix.  A plain store on purpose: the next
-// kernel reads these tiles, and with streaming (non-temporal) stores it found
-// them in HBM instead of the memory-side cache -- the quantization got 1 us
-// shorter and the GEMM behind it 1.5 us longer.
+// 16 quantized codes into the tiled matrix, as a write-through store (system scope, but not
+// streaming).  The next kernel reads these tiles.  A plain store leaves the line dirty in this
+// die's L2 until the write-back at the end of the kernel, which the launch then waits for
+// (2048 x 4096 codes: 8.8 us with plain stores, 8.0 us written through); a streaming
+// (non-temporal) store also bypasses the memory-side cache, and the GEMM behind it then
+// fetches the tiles from HBM (the quantization got 1 us shorter and the GEMM 1.5 us longer).
+// (The instruction is inline assembly because the cache policy cannot be spelled otherwise;
+// the compiler therefore does not know that it is a 16-byte store, after which a vector
+// instruction may not overwrite the data registers for two wait states -- the s_nop keeps
+// that distance, without it the next instruction occasionally changed the first dword.)
 __device__ __forceinline__ void store_codes(uint8_t* dst, uint4 codes) {
-    *reinterpret_cast<uint4*>(dst) = codes;
+    const v4i v = {(int)codes.x, (int)codes.y, (int)codes.z, (int)codes.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
 }
 
 // int8 code of v * inv as the low byte of the result.
@@ -542,8 +558,7 @@ __global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
 #pragma unroll
         for (int i = 0; i < Q8_CACHE; ++i) {
             const int c = cl + CSTEP * i;
-            if (c < nchunks)
-                store_codes(a.dst + tiled_chunk_offset(m, c, KB), quantize16<false>(v[i], inv));
+            if (c < nchunks) store_codes(a.dst + tiled_chunk_offset(m, c, KB), quantize16<false>(v[i], inv));
         }
     } else {
         for (int c = cl; c < nchunks; c += CSTEP) {
@@ -2008,10 +2023,13 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // KS waves share a column pair, taking 1/KS of K each; their accumulators are
 // added through LDS before the first of them runs the epilogue -- KS times as
 // many workgroups.
-// W4 (dense int4 weights only): a step is one 64-deep super-tile -- two
-// activation tiles and 1 KiB of packed weights per column block, unpacked in
-// registers into the two operands (every code times 16, undone by one shift of
-// the accumulators, so K may not exceed 2^17).
+// W4 (int4 weights, dense or an expert bank's int4 images): a step is one
+// 64-deep super-tile -- two activation tiles and 1 KiB of packed weights per
+// column block, unpacked in registers into the two operands (every code times
+// 16, undone by one shift of the accumulators, so K may not exceed 2^17).  A
+// bank may hold int4 and int8 experts (routed INT4, shared int8): each format
+// has its launch over the same grid, and a workgroup whose row block belongs to
+// an expert of the other format exits at once.
 template <int EPI, int KS, bool W4>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
     constexpr int TN = 2, WAVES = 4;
@@ -2036,7 +2054,11 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     const int live_blocks = g.blk_expert ? g.num_blocks[0] : mblocks;
     if (mblk >= live_blocks) return;
     const int e = g.blk_expert ? g.blk_expert[mblk] : 0;
-    const uint8_t* Wb = g.W + (size_t)e * g.w_expert_stride;
+    // grouped: this launch serves the experts held in its own format (int4 images come first in a bank)
+    if (g.blk_expert && (e < g.int4_experts) != W4) return;
+    const uint8_t* Wb = !g.blk_expert ? g.W
+                        : W4          ? g.W4 + (size_t)e * g.w4_expert_stride
+                                      : g.W + (size_t)(e - g.int4_experts) * g.w_expert_stride;
     const float* w_scale = g.w_scale ? g.w_scale + (size_t)e * g.ws_expert_stride : nullptr;
 
     // this wave's column blocks and k-tiles [kt0, kt0 + kts)
@@ -2434,29 +2456,27 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a
 // on, to put beside the datasheet peaks: a read-only stream over a footprint and
 // a pure-MFMA loop with operands in registers.
 //
-// Read-only stream: every step of the grid reads one slab of adjacent 1 KiB
-// pieces (16 bytes per lane), workgroup after workgroup, so that the whole grid
-// sweeps memory front to back -- the access order that gave the highest rate of
-// those tried.  The xor of everything read is written only if it equals a value
-// it never takes, which keeps the loads alive.
-__global__ __launch_bounds__(512) void stream_read_probe_kernel(const uint4* __restrict__ src, size_t chunks,
-                                                                uint32_t* sink) {
-    const size_t stride = (size_t)gridDim.x * 512;
+// Read-only stream in the access order of the decode GEMV: every workgroup (eight waves)
+// owns one contiguous span, its waves take the span's 1 KiB pieces in turn (16 bytes per
+// lane), eight loads per wave in flight.  The xor of everything read is written only if it
+// equals a value it is most unlikely to take, which keeps the loads alive.
+__global__ __launch_bounds__(512) void stream_read_probe_kernel(const uint8_t* __restrict__ src, size_t span,
+                                                                size_t bytes, uint32_t* sink) {
+    const size_t begin = (size_t)blockIdx.x * span;
+    const size_t end = begin + span < bytes ? begin + span : bytes;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t x = 0;
-    size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
-    for (; i + 3 * stride < chunks; i += 4 * stride) { // four loads in flight per lane
-        const v4i a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i));
-        const v4i b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + stride));
-        const v4i c = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + 2 * stride));
-        const v4i d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + 3 * stride));
-        x ^= (uint32_t)(a.x ^ a.y ^ a.z ^ a.w) ^ (uint32_t)(b.x ^ b.y ^ b.z ^ b.w) ^
-             (uint32_t)(c.x ^ c.y ^ c.z ^ c.w) ^ (uint32_t)(d.x ^ d.y ^ d.z ^ d.w);
+    for (size_t at = begin + (size_t)wave * 1024; at < end; at += 8 * 8 * 1024) {
+        v4i got[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t off = at + (size_t)u * 8 * 1024 + (size_t)lane * 16;
+            got[u] = off + 16 <= end ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + off)) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x ^= (uint32_t)(got[u].x ^ got[u].y ^ got[u].z ^ got[u].w);
     }
-    for (; i < chunks; i += stride) {
-        const v4i a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i));
-        x ^= (uint32_t)(a.x ^ a.y ^ a.z ^ a.w);
-    }
-    if (x == 0x9e3779b9u && sink) atomicAdd(sink, 1u); // (a value chosen to be improbable, not impossible: the sink is scratch)
+    if (x == 0x9e3779b9u && sink) atomicAdd(sink, 1u);
 }
 
 // Pure int8 MFMA: every wave keeps four independent 32x32 accumulators busy with
@@ -2512,22 +2532,27 @@ constexpr long DENSE_KS4_BELOW = 128; // dense use of the same kernel: every row
 // call, a handful for a decode step) the tile shrinks to 64 columns and the
 // waves split K instead.
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
-    if (g.w_int4 && (g.blk_expert || g.K > 131072)) return RKH_ERR_RUNTIME;
-    const int mblocks = g.blk_expert ? g.max_blocks : (g.M + 31) / 32;
+    const bool grouped = g.blk_expert != nullptr;
+    const bool any_int4 = grouped ? g.int4_experts > 0 : g.w_int4 != 0;
+    const bool any_int8 = grouped ? g.W != nullptr : !g.w_int4;
+    if (any_int4 && g.K > 131072) return RKH_ERR_RUNTIME; // (int4 codes ride as 16 * code in an int32 sum)
+    if (grouped && any_int4 && !g.W4) return RKH_ERR_RUNTIME;
+    const int mblocks = grouped ? g.max_blocks : (g.M + 31) / 32;
     const long wide = (long)mblocks * ((g.N + 255) / 256);
-    const int ks = wide < (g.blk_expert ? GROUPED_KS4_BELOW : DENSE_KS4_BELOW) ? 4 : 1;
+    const int ks = wide < (grouped ? GROUPED_KS4_BELOW : DENSE_KS4_BELOW) ? 4 : 1;
     const int cols = 256 / ks;
     const int nblocks = (g.N + cols - 1) / cols;
     const dim3 grid(mblocks * nblocks), block(256);
+    mark(st, ks == 4 ? "gemm_stream_kernel<KS=4>" : "gemm_stream_kernel");
 #define RK_LAUNCH(EPI)                                                                                         \
     do {                                                                                                       \
-        if (g.w_int4 && ks == 4)                                                                               \
+        if (any_int4 && ks == 4)                                                                               \
             hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true>), grid, block, 0, st, g, mblocks, nblocks);   \
-        else if (g.w_int4)                                                                                     \
+        else if (any_int4)                                                                                     \
             hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true>), grid, block, 0, st, g, mblocks, nblocks);   \
-        else if (ks == 4)                                                                                      \
+        if (any_int8 && ks == 4)                                                                               \
             hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, false>), grid, block, 0, st, g, mblocks, nblocks);  \
-        else                                                                                                   \
+        else if (any_int8)                                                                                     \
             hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false>), grid, block, 0, st, g, mblocks, nblocks);  \
     } while (0)
     switch (g.epilogue) {
@@ -2559,6 +2584,7 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
     const int per = (ksteps_total + ksplit - 1) / ksplit;
     ksplit = (ksteps_total + per - 1) / per; // no empty part
     const dim3 grid(mblocks * nblocks * ksplit), block(512);
+    mark(st, "gemm_wk_kernel");
 #define RK_WK(W4, EPI)                                                                              \
     do {                                                                                            \
         /* the LDS opt-in is per function and per device: once for each device this process uses */ \
@@ -2573,6 +2599,7 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
         }                                                                                           \
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, \
                            nblocks, ksplit, per);                                                   \
+        if (ksplit > 1) mark(st, "gemm_wk_reduce_kernel");                                          \
         if (ksplit > 1)                                                                             \
             hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>),                                \
                                dim3(mblocks * nblocks * (TM == 1 ? 4 : 8)), dim3(64), 0, st, g,     \
@@ -2610,12 +2637,14 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
     if (MR == 1 && !g.w_int4 && cw == 32) { // (see gemv_wide8_kernel)
+        mark(st, qt ? "gemv_wide8_kernel (fused quantize)" : "gemv_wide8_kernel");
         if (qt == 0) hipLaunchKernelGGL((gemv_wide8_kernel<0>), grid, block, 0, st, g, q);
         else if (qt == 1) hipLaunchKernelGGL((gemv_wide8_kernel<1>), grid, block, 0, st, g, q);
         else hipLaunchKernelGGL((gemv_wide8_kernel<2>), grid, block, 0, st, g, q);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
+    mark(st, qt ? "gemv_kernel (fused quantize)" : "gemv_kernel");
 #define RK_GEMV(W4, QT)                                                                        \
     do {                                                                                       \
         if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, g, q);        \
@@ -2637,6 +2666,7 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
     const dim3 grid(g.interleave_F / 32), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+    mark(st, qt ? "gemv_swiglu_kernel (fused quantize)" : "gemv_swiglu_kernel");
 #define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, g, q)
     if (g.w_int4) {
         if (qt == 0) RK_SWI(true, 0); else if (qt == 1) RK_SWI(true, 1); else RK_SWI(true, 2);
@@ -2684,6 +2714,15 @@ bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu 
 
 int g_fail_malloc_after = 0;
 
+// RK_NPU_HIP_EXP: bit mask of code paths under evaluation (tuning aid, read once).
+int exp_flags() {
+    static const int flags = [] {
+        const char* v = getenv("RK_NPU_HIP_EXP");
+        return v ? atoi(v) : 0;
+    }();
+    return flags;
+}
+
 } // namespace
 
 // =================================================================== C ABI
@@ -2722,6 +2761,11 @@ void rkh_close(int device, void* stream) {
 }
 
 void rkh_fail_malloc_after(int n) { g_fail_malloc_after = n; }
+
+void rkh_set_marker(rkh_marker_fn fn, void* user) {
+    g_marker_user = user;
+    g_marker = fn;
+}
 
 int rkh_malloc(int device, void** ptr, size_t bytes) {
     *ptr = nullptr;
@@ -2764,6 +2808,7 @@ int rkh_d2d(void* stream, void* dst, const void* src, size_t bytes) {
 }
 int rkh_fill32(void* stream, void* dst, uint32_t value, size_t words) {
     if (!words) return RKH_OK;
+    mark((hipStream_t)stream, "fill32_kernel");
     const int blocks = (int)((words + 255) / 256 < 4096 ? (words + 255) / 256 : 4096);
     hipLaunchKernelGGL(fill32_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                        static_cast<uint32_t*>(dst), value, words);
@@ -2838,6 +2883,7 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
         const bool rows4 = args->M < 8 * 2 * 256; // 8 rows would give fewer than two workgroups per compute unit
         const dim3 grid(rows4 ? (args->M + 3) / 4 : (args->M + 7) / 8);
         const hipStream_t st = (hipStream_t)stream;
+        mark(st, "quant_rows8_kernel");
         if (args->in_dtype == RKH_F16) {
             if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 4>), grid, block, 0, st, *args);
             else hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 8>), grid, block, 0, st, *args);
@@ -2850,6 +2896,7 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     }
     const bool reuse = mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE;
     if (reuse && args->in_dtype == RKH_F32 && args->M >= 64 && (args->K + 15) / 16 <= 64 * QR_CACHE) {
+        mark((hipStream_t)stream, "requant_rows_wave_kernel");
         hipLaunchKernelGGL(requant_rows_wave_kernel, dim3((args->M + 3) / 4), block, 0, (hipStream_t)stream, *args);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
@@ -2862,6 +2909,7 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
         while (split < 8 && args->M * split < 512 && row_chunks / (split * 2) >= 128) split *= 2;
     }
     const dim3 grid(args->M * split);
+    mark((hipStream_t)stream, "quant_rows_kernel");
     switch (args->in_dtype) {
     case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args, split); break;
     case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args, split); break;
@@ -2982,6 +3030,7 @@ int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args) {
         (long)args->rows * args->top_k > ROUTE_MAX_ASSIGNMENTS)
         return RKH_ERR_RUNTIME;
     const dim3 grid(args->rows), block(256);
+    mark((hipStream_t)stream, "moe_scatter_kernel");
     if (args->in_dtype == RKH_F32)
         hipLaunchKernelGGL(moe_scatter_kernel<float>, grid, block, 0, (hipStream_t)stream, *args);
     else if (args->in_dtype == RKH_I8)
@@ -2994,15 +3043,18 @@ int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args) {
 
 int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args) {
     const dim3 grid((args->H / 4 + 255) / 256, args->rows);
+    mark((hipStream_t)stream, "moe_combine_kernel");
     hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, (hipStream_t)stream, *args);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
 
-int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, int workgroups, void* sink) {
-    if (!src || bytes < 16 || workgroups < 1) return RKH_ERR_RUNTIME;
-    hipLaunchKernelGGL(stream_read_probe_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream,
-                       static_cast<const uint4*>(src), bytes / 16, static_cast<uint32_t*>(sink));
+int rkh_probe_stream_read(void* stream, const void* src, size_t bytes, size_t span, void* sink) {
+    if (!src || bytes < 16 || span < 1024 || span % 1024) return RKH_ERR_RUNTIME;
+    const size_t workgroups = (bytes + span - 1) / span;
+    if (workgroups > 0x7fffffffu) return RKH_ERR_RUNTIME;
+    hipLaunchKernelGGL(stream_read_probe_kernel, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream,
+                       static_cast<const uint8_t*>(src), span, bytes, static_cast<uint32_t*>(sink));
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }

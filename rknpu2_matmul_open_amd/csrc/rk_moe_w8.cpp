@@ -40,11 +40,12 @@ bool valid(const rk_npu_moe_w8_config& c) {
            (c.native_input == 0 || c.native_input == 1) && c.timeout_ms >= 1 &&
            c.timeout_ms <= 60000 && c.middle == RK_NPU_MOE_MIDDLE_CPU;
 }
-// Expert formats (reference src/rk_npu_moe_w8.cpp:366-387).  W4 experts hold
+// Expert formats (reference src/rk_npu_moe_w8.cpp:366-387).  W4 experts arrive as
 // signed INT4 codes in the same int8 arrays; the arithmetic is that of the W8
 // path with codes restricted to [-8, 7] (the reference's own test runs one body
-// against both), so they execute on the same kernels and are kept as int8 on
-// the device.
+// against both).  On the device they are packed two codes per byte (tiled int4,
+// half the bytes to hold and to stream) and run on the int4 variant of the
+// grouped kernel, whose integer sums equal the int8 path's exactly.
 enum Mode { kW8 = 0, kW4 = 1, kRoutedW4SharedW8 = 2 };
 bool expert_is_w4(int mode, int expert, int routed) {
     return mode == kW4 || (mode == kRoutedW4SharedW8 && expert < routed);
@@ -70,14 +71,20 @@ struct rk_npu_moe_w8_weights {
     rk_npu_moe_w8_weight_config config{};
     int mode = kW8;
     int count = 0;              // routed + shared
-    size_t gate_stride = 0;     // bytes between experts in gate_up
+    int count4 = 0;             // leading experts held as int4 images (all of them, the routed ones, or none)
+    size_t gate_stride = 0;     // bytes between int8 experts in gate_up
     size_t down_stride = 0;
-    DeviceBuffer gate_up;       // count x tiled int8 [align256(2I) x align256(H)], gate/up interleaved
-    DeviceBuffer down;          // count x tiled int8 [align256(H) x align256(I)]
+    size_t gate_stride4 = 0;    // bytes between int4 experts in gate_up4
+    size_t down_stride4 = 0;
+    DeviceBuffer gate_up;       // (count - count4) x tiled int8 [align256(2I) x align256(H)], gate/up interleaved
+    DeviceBuffer down;          // (count - count4) x tiled int8 [align256(H) x align256(I)]
+    DeviceBuffer gate_up4;      // count4 x tiled int4, same geometry
+    DeviceBuffer down4;
     DeviceBuffer gate_scales;   // count x [2I]
     DeviceBuffer down_scales;   // count x [H]
     uint64_t bytes() const {
-        return gate_up.bytes() + down.bytes() + gate_scales.bytes() + down_scales.bytes();
+        return gate_up.bytes() + down.bytes() + gate_up4.bytes() + down4.bytes() + gate_scales.bytes() +
+               down_scales.bytes();
     }
 };
 
@@ -162,7 +169,10 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
 
     rkh_gemm_args g{};
     g.A = ws->a_tiled.as<>();
-    g.W = w->gate_up.as<>();
+    g.W = w->gate_up ? w->gate_up.as<>() : nullptr;
+    g.W4 = w->gate_up4 ? w->gate_up4.as<>() : nullptr;
+    g.int4_experts = w->count4;
+    g.w4_expert_stride = w->gate_stride4;
     g.M = ws->sorted_rows;
     g.N = 2 * I;
     g.K = H;
@@ -199,7 +209,10 @@ int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
 
     rkh_gemm_args d{};
     d.A = ws->h_tiled.as<>();
-    d.W = w->down.as<>();
+    d.W = w->down ? w->down.as<>() : nullptr;
+    d.W4 = w->down4 ? w->down4.as<>() : nullptr;
+    d.int4_experts = w->count4;
+    d.w4_expert_stride = w->down_stride4;
     d.M = ws->sorted_rows;
     d.N = H;
     d.K = I;
@@ -373,14 +386,21 @@ void rk_npu_moe_w8_config_init(rk_npu_moe_w8_config* c, int hidden, int intermed
 
 namespace {
 
-// Packs one expert into slot e of the bank (the context's submit mutex is held).
+// Packs one expert into slot e of the bank (the context's submit mutex is held): slots below
+// count4 take int4 images (the codes were range-checked on the host), the others int8 images.
 int pack_expert(rk_npu_moe_w8_weights* w, DeviceBuffer& raw, int e, const rk_npu_moe_w8_expert& x) {
     const int H = w->config.hidden, I = w->config.intermediate;
     void* stream = w->owner.ctx->stream;
+    const bool int4 = e < w->count4;
+    const int e8 = e - w->count4;
     int rc = rkh_h2d(stream, raw.as<>(), x.gate_up, (size_t)H * 2 * I);
-    if (!rc) rc = rkh_pack_w8(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e);
+    if (!rc)
+        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up4.as<>() + w->gate_stride4 * e, nullptr)
+                  : rkh_pack_w8(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e8);
     if (!rc) rc = rkh_h2d(stream, raw.as<>(), x.down, (size_t)I * H);
-    if (!rc) rc = rkh_pack_w8(stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e);
+    if (!rc)
+        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), I, H, 0, w->down4.as<>() + w->down_stride4 * e, nullptr)
+                  : rkh_pack_w8(stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e8);
     if (!rc) rc = rkh_h2d(stream, w->gate_scales.as<float>() + (size_t)e * 2 * I, x.gate_up_scales, (size_t)2 * I * sizeof(float));
     if (!rc) rc = rkh_h2d(stream, w->down_scales.as<float>() + (size_t)e * H, x.down_scales, (size_t)H * sizeof(float));
     // the staging buffer is reused: finish this expert before the next copy lands
@@ -415,14 +435,20 @@ rk_npu_moe_w8_weights* create_weights(rk_npu_iommu_domain* domain, const rk_npu_
     w->config = *config;
     w->mode = mode;
     w->count = count;
+    w->count4 = mode == kW4 ? count : mode == kRoutedW4SharedW8 ? config->routed_experts : 0;
     w->gate_stride = rkh_tiled_i8_bytes(2 * I, H, RKH_COL_ALIGN);
     w->down_stride = rkh_tiled_i8_bytes(H, I, RKH_COL_ALIGN);
+    w->gate_stride4 = rkh_tiled_i4_bytes(2 * I, H, RKH_COL_ALIGN);
+    w->down_stride4 = rkh_tiled_i4_bytes(H, I, RKH_COL_ALIGN);
     rk_npu_ctx* ctx = domain->ctx;
     std::lock_guard<std::mutex> lock(ctx->submit_mutex);
     DeviceBuffer raw;
     const bool zero = experts == nullptr;
-    if (w->gate_up.alloc(w->owner, w->gate_stride * count, zero) ||
-        w->down.alloc(w->owner, w->down_stride * count, zero) ||
+    const int count8 = count - w->count4;
+    if ((count8 && (w->gate_up.alloc(w->owner, w->gate_stride * count8, zero) ||
+                    w->down.alloc(w->owner, w->down_stride * count8, zero))) ||
+        (w->count4 && (w->gate_up4.alloc(w->owner, w->gate_stride4 * w->count4, zero) ||
+                       w->down4.alloc(w->owner, w->down_stride4 * w->count4, zero))) ||
         w->gate_scales.alloc(w->owner, (size_t)count * 2 * I * sizeof(float), zero) ||
         w->down_scales.alloc(w->owner, (size_t)count * H * sizeof(float), zero) ||
         raw.alloc(w->owner, (size_t)H * 2 * I, false))
@@ -551,17 +577,19 @@ rk_npu_moe_w8_weights* rk_npu_moe_quant_slots_create(rk_npu_iommu_domain* domain
 
 namespace {
 
-// A packed expert record: header, then the expert's device images exactly as the
-// kernels read them (gate/up and down tiles, gate/up and down scales).  Records
-// are produced by rk_npu_moe_quant_export_expert of this library and are not
-// interchangeable with the reference's (its records hold NPU tile images).
+// A packed INT4 expert record: header, then the expert's device images exactly as
+// the kernels read them (gate/up and down int4 tiles, two codes per byte; gate/up
+// and down scales).  Records are produced by rk_npu_moe_quant_export_expert of
+// this library and are not interchangeable with the reference's (its records
+// hold NPU tile images).  Every byte of an image is two valid codes, so a record
+// cannot smuggle a value outside [-8, 7] into a slot.
 struct RecordHeader {
     uint32_t magic, version, hidden, intermediate;
 };
 constexpr uint32_t kRecordMagic = 0x4d484b52u; // "RKHM"
 
 uint64_t record_bytes(const rk_npu_moe_w8_weights* w) {
-    return sizeof(RecordHeader) + w->gate_stride + w->down_stride +
+    return sizeof(RecordHeader) + w->gate_stride4 + w->down_stride4 +
            ((uint64_t)2 * w->config.intermediate + w->config.hidden) * sizeof(float);
 }
 
@@ -587,10 +615,10 @@ int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights* w, int e, void* 
     std::memcpy(p, &header, sizeof(header));
     p += sizeof(header);
     std::lock_guard<std::mutex> lock(ctx->submit_mutex);
-    int rc = rkh_d2h(ctx->stream, p, w->gate_up.as<>() + w->gate_stride * e, w->gate_stride);
-    p += w->gate_stride;
-    if (!rc) rc = rkh_d2h(ctx->stream, p, w->down.as<>() + w->down_stride * e, w->down_stride);
-    p += w->down_stride;
+    int rc = rkh_d2h(ctx->stream, p, w->gate_up4.as<>() + w->gate_stride4 * e, w->gate_stride4);
+    p += w->gate_stride4;
+    if (!rc) rc = rkh_d2h(ctx->stream, p, w->down4.as<>() + w->down_stride4 * e, w->down_stride4);
+    p += w->down_stride4;
     if (!rc) rc = rkh_d2h(ctx->stream, p, w->gate_scales.as<float>() + (size_t)e * 2 * I, (size_t)2 * I * sizeof(float));
     p += (size_t)2 * I * sizeof(float);
     if (!rc) rc = rkh_d2h(ctx->stream, p, w->down_scales.as<float>() + (size_t)e * H, (size_t)H * sizeof(float));
@@ -617,8 +645,8 @@ int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights* w, int slot, con
     RecordHeader header;
     std::memcpy(&header, p, sizeof(header));
     const uint8_t* gate = p + sizeof(header);
-    const uint8_t* down = gate + w->gate_stride;
-    const uint8_t* gate_scales = down + w->down_stride;
+    const uint8_t* down = gate + w->gate_stride4;
+    const uint8_t* gate_scales = down + w->down_stride4;
     const uint8_t* down_scales = gate_scales + (size_t)2 * I * sizeof(float);
     auto at = Clock::now();
     bool ok = header.magic == kRecordMagic && header.version == RK_NPU_MOE_QUANT_BLOB_VERSION &&
@@ -638,11 +666,11 @@ int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights* w, int slot, con
     if (!rc) rc = rkh_sync(ctx->stream);
     if (timings) timings->copy_us = elapsed_us(at);
     at = Clock::now();
-    if (!rc) rc = rkh_h2d(ctx->stream, w->gate_up.as<>() + w->gate_stride * slot, gate, w->gate_stride);
+    if (!rc) rc = rkh_h2d(ctx->stream, w->gate_up4.as<>() + w->gate_stride4 * slot, gate, w->gate_stride4);
     if (!rc) rc = rkh_sync(ctx->stream);
     if (timings) timings->gate_sync_us = elapsed_us(at);
     at = Clock::now();
-    if (!rc) rc = rkh_h2d(ctx->stream, w->down.as<>() + w->down_stride * slot, down, w->down_stride);
+    if (!rc) rc = rkh_h2d(ctx->stream, w->down4.as<>() + w->down_stride4 * slot, down, w->down_stride4);
     if (!rc) rc = rkh_sync(ctx->stream);
     if (timings) {
         timings->down_sync_us = elapsed_us(at);
@@ -665,10 +693,10 @@ int rk_npu_moe_quant_swap_slots(rk_npu_moe_w8_weights* a, int ai, rk_npu_moe_w8_
     const size_t H = a->config.hidden, I = a->config.intermediate;
     rk_npu_ctx* ctx = a->owner.ctx;
     std::lock_guard<std::mutex> lock(ctx->submit_mutex);
-    int rc = rkh_exchange32(ctx->stream, a->gate_up.as<>() + a->gate_stride * ai, b->gate_up.as<>() + b->gate_stride * bi,
-                            a->gate_stride / 4);
-    if (!rc) rc = rkh_exchange32(ctx->stream, a->down.as<>() + a->down_stride * ai, b->down.as<>() + b->down_stride * bi,
-                                 a->down_stride / 4);
+    int rc = rkh_exchange32(ctx->stream, a->gate_up4.as<>() + a->gate_stride4 * ai, b->gate_up4.as<>() + b->gate_stride4 * bi,
+                            a->gate_stride4 / 4);
+    if (!rc) rc = rkh_exchange32(ctx->stream, a->down4.as<>() + a->down_stride4 * ai, b->down4.as<>() + b->down_stride4 * bi,
+                                 a->down_stride4 / 4);
     if (!rc) rc = rkh_exchange32(ctx->stream, a->gate_scales.as<float>() + ai * 2 * I, b->gate_scales.as<float>() + bi * 2 * I, 2 * I);
     if (!rc) rc = rkh_exchange32(ctx->stream, a->down_scales.as<float>() + ai * H, b->down_scales.as<float>() + bi * H, H);
     return map_error(rc);

@@ -112,6 +112,32 @@ class Session:
         return us.value / iters
 
 
+def profile_kernels(sess, fn, iters, warmup=3):
+    """Average time per kernel of one fn() call, from stream events between the kernels:
+    a list of (kernel name, microseconds) in launch order (kernel plus the launch gap behind it)."""
+    for _ in range(warmup):
+        fn()
+    check(sess.sync(), "sync")
+    lib = sess.lib
+    check(lib.rk_npu_hip_profile_begin(sess.ctx), "profile_begin")
+    for _ in range(iters):
+        fn()
+    cap = 64 * iters
+    us = (C.c_double * cap)()
+    names = C.create_string_buffer(64 * cap)
+    n = lib.rk_npu_hip_profile_end(sess.ctx, names, len(names), us, cap)
+    if n < 0:
+        raise RkError(n, "profile_end")
+    labels = names.value.decode().split("\n")[:-1]
+    per = n // iters
+    if per * iters != n or len(labels) != n:
+        raise RuntimeError("profile: %d kernels over %d calls" % (n, iters))
+    out = []
+    for k in range(per):
+        out.append((labels[k], sum(us[i * per + k] for i in range(iters)) / iters))
+    return out
+
+
 def default_strategy(kind, M, N, K, k_tile=None, n_tile=None):
     """A strategy any caller of the reference would pass: full-K tile up to
     2048, n_tile <= 3072, one core, one CPU."""

@@ -245,11 +245,18 @@ def test_int4_experts_equal_the_int8_path(sess, oracle, flavour, shared):
         assert rc == 0 and rc2 == 0
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
         lib = sess.lib
-        assert lib.rk_npu_moe_quant_expert_blob_bytes(moe.w) > (2 * I * H + H * I)
+        # INT4 experts are held as packed nibbles: a record is header + half a byte per weight
+        # (+ padding to whole tiles) + scales, and the bank takes about half of an int8 bank
+        blob = lib.rk_npu_moe_quant_expert_blob_bytes(moe.w)
+        assert (2 * I * H + H * I) // 2 + (2 * I + H) * 4 < blob
         # handles of another expert format do not bind
         w8 = ops.MoeW8(sess, H, I, E, shared, top_k, 64, experts)
         try:
             assert lib.rk_npu_moe_quant_expert_blob_bytes(w8.w) == 0
+            b4, b8 = lib.rk_npu_moe_w8_weights_device_bytes(moe.w), lib.rk_npu_moe_w8_weights_device_bytes(w8.w)
+            int4_experts = E + shared if flavour == "quant" else E
+            images8 = (b8 - (E + shared) * (2 * I + H) * 4) // (E + shared)   # int8 image bytes per expert
+            assert b8 - b4 == int4_experts * images8 // 2
             assert moe.run_f32(x, ids, routes, weights=w8.w)[0] == capi.RK_NPU_ERR_PARAM
             assert w8.run_f32(x, ids, routes, weights=moe.w)[0] == capi.RK_NPU_ERR_PARAM
         finally:
