@@ -50,6 +50,21 @@ inline void mark(hipStream_t stream, const char* kernel) {
     if (g_marker) g_marker(g_marker_user, stream, kernel);
 }
 
+// Build with -DRK_DEBUG_TS for in-kernel wall-clock stamps (tuning aid, never in the product
+// build): RK_TS(i) stores the 100 MHz real-time counter seen by a workgroup's first wave into slot i
+// of its record (8 slots per workgroup) of the buffer set with rkh_debug_set_ts.
+#ifdef RK_DEBUG_TS
+__device__ unsigned long long* rk_dbg_ts = nullptr;
+#define RK_TS(i)                                                                                  \
+    do {                                                                                          \
+        /* (a wave-uniform branch: every lane of the first wave stores the same word) */         \
+        if (rk_dbg_ts && __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0)                   \
+            rk_dbg_ts[(size_t)blockIdx.x * 8 + (i)] = wall_clock64();                             \
+    } while (0)
+#else
+#define RK_TS(i) do {} while (0)
+#endif
+
 // Compile-time loop: f(std::integral_constant<int, 0>{}) ... f(<N-1>{}).
 template <int N, int I = 0, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -2030,10 +2045,11 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // bank may hold int4 and int8 experts (routed INT4, shared int8): each format
 // has its launch over the same grid, and a workgroup whose row block belongs to
 // an expert of the other format exits at once.
-template <int EPI, int KS, bool W4>
-__global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
-    constexpr int TN = 2, WAVES = 4;
+template <int EPI, int KS, bool W4, bool BAL = false>
+__global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
+    constexpr int TN = 2, WAVES = BAL ? 8 : 4;
     constexpr bool KSPLIT = KS > 1;
+    static_assert(!BAL || !KSPLIT, "the balanced variant does not split K");
     constexpr int CG = WAVES / KS; // column pairs per workgroup
     constexpr int RING = 8; // (16 with K split four ways, a wave's whole share in flight, was measured slower)
     constexpr int AT = W4 ? 2 : 1;   // activation tiles per step
@@ -2048,10 +2064,14 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     // steps over K: k-tiles (a multiple of 8 = RING) or, for int4 weights, super-tiles (a multiple of 4)
     const int KB = (int)rkh_align_up(g.K, RKH_K_ALIGN) / (32 * AT);
 
-    const int logical = xcd_remap(blockIdx.x, mblocks * nblocks);
-    const int mblk = logical % mblocks, nblk = logical / mblocks;
+    [[maybe_unused]] constexpr int TSB = EPI == RKH_EPI_SWIGLU ? 4 : 0; // (debug stamps: the SwiGLU launch keeps its own slots)
+    RK_TS(TSB + 0);
     // dense use (no block -> expert table): one weight matrix, every row block live
     const int live_blocks = g.blk_expert ? g.num_blocks[0] : mblocks;
+
+    // One unit of work of a wave: row block mblk x the column pair that starts at column block
+    // pair_pb0 (BAL) or the wave's pair of column tile nblk (otherwise).
+    auto run_unit = [&](int mblk, int nblk, int pair_pb0) {
     if (mblk >= live_blocks) return;
     const int e = g.blk_expert ? g.blk_expert[mblk] : 0;
     // grouped: this launch serves the experts held in its own format (int4 images come first in a bank)
@@ -2063,16 +2083,49 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
 
     // this wave's column blocks and k-tiles [kt0, kt0 + kts)
     const int cg = wave / KS, kq = wave % KS; // column pair, part of K
-    const int pb0 = (nblk * CG + cg) * TN;
-    const int share = (KB + KS - 1) / KS;
-    const int kts = max(0, min(share, KB - kq * share));
-    const int kt0 = min(kq * share, KB - 1); // (a wave without a share still loads in bounds)
+    const int pb0 = BAL ? pair_pb0 : (nblk * CG + cg) * TN;
+    // K split over waves: wave kq takes the steps kq, kq + KS, ... -- interleaved, so that the
+    // KS waves of a column pair read KS adjacent KiB of each column block at a time (waves that
+    // each walk a private range of memory reached 5.2 TB/s in a read-only test, waves that
+    // interleave 6.4)
+    const int kts = KB > kq ? (KB - kq + KS - 1) / KS : 0;
+    const int kt0 = min(kq, KB - 1); // (a wave without a share still loads in bounds)
     const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * (1024 * AT);
     const uint8_t* wsrc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) wsrc[j] = Wb + ((size_t)(pb0 + j) * KB + kt0) * 1024;
     const unsigned lane_off = lane * 16;
     int left = max(kts, 1) - 1; // how often the sources may still advance
+
+    // The scales of this wave's tile pair are requested now, ahead of every load of the ring
+    // (loads return in issue order, so they are back with the first step), and handed to the
+    // epilogue through the wave's staging area: fetched at the start of the epilogue they cost
+    // it a round trip to memory (an epilogue of 2.8 us instead of 1.4, of a kernel whose loop
+    // takes 7).  Lane l holds the row scale of row l % 32 and the column scale of column l % 32
+    // of column block l / 32 of the pair.
+    const int m0 = mblk * 32;
+    const int m_limit = g.blk_expert ? live_blocks * 32 : g.M;
+    float my_as = 0.0f, my_ws = 0.0f;
+    bool as_ok = false, ws_ok = false;
+    if constexpr (EPI != RKH_EPI_I32) {
+        const int m = m0 + (lane & 31);
+        const int pb = pb0 + (lane >> 5);
+        int n;
+        if constexpr (EPI == RKH_EPI_SWIGLU) { // pb0 is even: the gate block, its up block right behind it
+            const int nl = (pb0 >> 1) * 32 + (lane & 31);
+            n = (lane >> 5 ? g.interleave_F : 0) + nl;
+            ws_ok = nl < g.interleave_F;
+        } else {
+            const bool live = g.interleave_F ? pb < g.N / 32 : pb * 32 < g.N;
+            n = block_first_col(pb, g.interleave_F) + (lane & 31);
+            ws_ok = live && n < g.N;
+        }
+        as_ok = m < m_limit;
+        const float* pa = g.a_scale + (as_ok ? m : 0);
+        const float* pw = w_scale + (ws_ok ? n : 0);
+        asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
+        asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
+    }
 
     v16i acc[TN];
 #pragma unroll
@@ -2090,7 +2143,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
             regs[L] = r;
         });
-        const int step = left > 0 ? 1024 : 0;
+        const int step = left > 0 ? 1024 * KS : 0;
         asrc += step * AT;
 #pragma unroll
         for (int j = 0; j < TN; ++j) wsrc[j] += step;
@@ -2109,6 +2162,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
             constexpr int SLOT = decltype(slot_tag)::value;
             issue(ring[(SLOT + RING - 1) % RING]);
             wait(ring[SLOT]);
+            if (SLOT == 0 && s == 0) RK_TS(TSB + 1);
             // (a K share need not be a multiple of RING: the steps past its end reload the last tile and are skipped)
             if ((!KSPLIT && !W4) || s + SLOT < kts) {
 #pragma unroll
@@ -2132,11 +2186,12 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
     // regards their destination registers as dead: without the uses below it may
     // give one of them to an epilogue value ahead of the wait, and the load then
     // lands on top of that value.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(my_as), "+v"(my_ws)::"memory");
 #pragma unroll
     for (int t = 0; t < RING; ++t)
 #pragma unroll
         for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(ring[t][l]));
+    RK_TS(TSB + 2);
 
     if constexpr (KSPLIT) {
         // the other parts of K hand their accumulators to part 0: [column pair][part - 1][tile][q][lane] x 4 ints
@@ -2170,15 +2225,47 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(rkh_gemm_args g, int m
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[j][r] >>= 4;
     }
-    const int m_limit = g.blk_expert ? live_blocks * 32 : g.M;
     uint8_t* stage_lds = stage_raw + wave * (32 * (32 * 4 + 8));
-    const int m0 = mblk * 32;
+    float as = 0.0f, ws[TN][16];
+    if constexpr (EPI != RKH_EPI_I32) { // scales: lane-wise registers -> the wave's staging area -> per-lane order
+        float* sc = reinterpret_cast<float*>(stage_lds);
+        sc[lane] = ws_ok ? my_ws : 0.0f;
+        if (lane < 32) sc[64 + lane] = as_ok ? my_as : 0.0f;
+        __builtin_amdgcn_wave_barrier();
+        as = sc[64 + (lane & 31)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ws[j][r] = sc[j * 32 + tile_col(r, lane)];
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // (read before the staging below overwrites the area)
+    }
     if constexpr (EPI == RKH_EPI_SWIGLU) {
-        epilogue_swiglu(g, acc[0], acc[1], m0, pb0, lane, g.a_scale, w_scale, m_limit, stage_lds);
+        epilogue_swiglu_scaled(g, acc[0], acc[1], m0, pb0, lane, as, ws[0], ws[1], m_limit, stage_lds);
     } else {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-            epilogue_tile<EPI>(g, acc[j], m0, pb0 + j, lane, g.a_scale, w_scale, m_limit, stage_lds);
+            epilogue_tile_scaled<EPI>(g, acc[j], m0, pb0 + j, lane, as, ws[j], m_limit, stage_lds);
+    }
+    RK_TS(TSB + 3);
+    }; // run_unit
+
+    if constexpr (!BAL) {
+        const int logical = xcd_remap(blockIdx.x, mblocks * nblocks);
+        run_unit(logical % mblocks, logical / mblocks, 0);
+    } else {
+        // Balanced launch: one workgroup of eight waves per compute unit, the units (live row
+        // block, column pair) dealt out in equal contiguous shares -- first to the dies (a
+        // workgroup's die is blockIdx % 8), then to the workgroups of a die -- and a share walked
+        // by its workgroup's waves in turn.  Consecutive units are column pairs of one row block,
+        // so the waves of a workgroup share the activation tiles through the L1, and the row
+        // blocks of one expert meet in one die's L2.
+        const int pairs = (g.N + 63) / 64;
+        const long units = (long)live_blocks * pairs;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = (int)(gridDim.x + 7 - xcd) >> 3;
+        const long die0 = units * xcd / 8, die1 = units * (xcd + 1) / 8;
+        const long first = die0 + (die1 - die0) * slot / slots, last = die0 + (die1 - die0) * (slot + 1) / slots;
+        for (long u = first + wave; u < last; u += WAVES) run_unit((int)(u / pairs), 0, (int)(u % pairs) * TN);
     }
 }
 
@@ -2525,6 +2612,20 @@ static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
 // (Splitting K two ways over 128-column tiles for 4 .. 64 tokens was measured too: 1 - 3 us slower than
 // the wide tile at every size.)
 constexpr long GROUPED_KS4_BELOW = 96;
+constexpr long GROUPED_BALANCED_UNITS_PER_CU = 4; // (row block, column pair) units per compute unit from which the balanced launch is used
+
+// Compute units of the current device (0 if the query fails), looked up once per device.
+int compute_units() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (!cached[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 constexpr long DENSE_KS4_BELOW = 128; // dense use of the same kernel: every row block is live
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
 // 256-column tile); blocks beyond the live count exit at once.  When that grid
@@ -2542,6 +2643,36 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     const int ks = wide < (grouped ? GROUPED_KS4_BELOW : DENSE_KS4_BELOW) ? 4 : 1;
     const int cols = 256 / ks;
     const int nblocks = (g.N + cols - 1) / cols;
+    // Many row blocks (a prefill-sized MoE call): the balanced launch, one workgroup per compute
+    // unit.  With a workgroup per (row block, column tile) the 392 workgroups of a 256-token,
+    // 32-expert, top-4 layer left 136 compute units with two of them and 120 with one, and a
+    // compute unit draws at most 40 - 55 GB/s however many workgroups it holds: the launch
+    // lasted as long as the compute units with two (down projection: last workgroup done after
+    // 17.8 us, 15.4 balanced).  RK_NPU_HIP_GROUPED=balanced|tiles forces the choice (tuning aid).
+    const int cus = compute_units();
+    bool balanced = grouped && cus > 0 && (long)mblocks * ((g.N + 63) / 64) >= GROUPED_BALANCED_UNITS_PER_CU * (long)cus;
+    static const char* forced = getenv("RK_NPU_HIP_GROUPED");
+    if (forced && forced[0] == 'b') balanced = grouped && cus > 0;
+    if (forced && forced[0] == 't') balanced = false;
+    if (balanced) {
+        mark(st, "gemm_stream_kernel<balanced>");
+        const dim3 grid(cus), block(512);
+#define RK_LAUNCH_BAL(EPI)                                                                                          \
+    do {                                                                                                            \
+        if (any_int4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true, true>), grid, block, 0, st, g, mblocks, nblocks);  \
+        if (any_int8) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false, true>), grid, block, 0, st, g, mblocks, nblocks); \
+    } while (0)
+        switch (g.epilogue) {
+        case RKH_EPI_I32: RK_LAUNCH_BAL(RKH_EPI_I32); break;
+        case RKH_EPI_F16: RK_LAUNCH_BAL(RKH_EPI_F16); break;
+        case RKH_EPI_F32: RK_LAUNCH_BAL(RKH_EPI_F32); break;
+        case RKH_EPI_SWIGLU: RK_LAUNCH_BAL(RKH_EPI_SWIGLU); break;
+        default: return RKH_ERR_RUNTIME;
+        }
+#undef RK_LAUNCH_BAL
+        RKH_CHECK(hipGetLastError());
+        return RKH_OK;
+    }
     const dim3 grid(mblocks * nblocks), block(256);
     mark(st, ks == 4 ? "gemm_stream_kernel<KS=4>" : "gemm_stream_kernel");
 #define RK_LAUNCH(EPI)                                                                                         \
@@ -2714,15 +2845,6 @@ bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu 
 
 int g_fail_malloc_after = 0;
 
-// RK_NPU_HIP_EXP: bit mask of code paths under evaluation (tuning aid, read once).
-int exp_flags() {
-    static const int flags = [] {
-        const char* v = getenv("RK_NPU_HIP_EXP");
-        return v ? atoi(v) : 0;
-    }();
-    return flags;
-}
-
 } // namespace
 
 // =================================================================== C ABI
@@ -2761,6 +2883,14 @@ void rkh_close(int device, void* stream) {
 }
 
 void rkh_fail_malloc_after(int n) { g_fail_malloc_after = n; }
+
+#ifdef RK_DEBUG_TS
+int rkh_debug_set_ts(void* device_buffer) {
+    unsigned long long* p = static_cast<unsigned long long*>(device_buffer);
+    RKH_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(rk_dbg_ts), &p, sizeof(p)));
+    return RKH_OK;
+}
+#endif
 
 void rkh_set_marker(rkh_marker_fn fn, void* user) {
     g_marker_user = user;
