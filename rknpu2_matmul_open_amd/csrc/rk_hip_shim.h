@@ -97,9 +97,11 @@ int rkh_event_elapsed_us(void* start, void* stop, double* us); /* waits for stop
  * of dst. */
 int rkh_pack_w8(void* stream, const int8_t* src, int K, int N, int interleave_F, uint8_t* dst);
 /* Same for int4 codes in [-8, 7] (one int8 per code in src).  bad_flag (device
- * int, may be NULL) is OR-ed with 1 if a code is outside [-8, 7]. */
+ * int, may be NULL) is OR-ed with 1 if a code is outside [-8, 7].  colsum (device
+ * int32 [N], zero-filled by the caller, may be NULL) receives sum_k B[k, n] per
+ * logical column: the constant the int4 GEMV kernels add (rkh_gemm_args.w_colsum). */
 int rkh_pack_w4(void* stream, const int8_t* src, int K, int N, int interleave_F, uint8_t* dst,
-                int* bad_flag);
+                int* bad_flag, int32_t* colsum);
 
 /* ---- per-row activation quantization ---- */
 enum rkh_quant_mode {
@@ -147,6 +149,8 @@ typedef struct rkh_gemm_args {
     int interleave_F;     /* 0, or F when the weight columns are gate/up interleaved */
     const float* a_scale; /* [align(M)]                                            */
     const float* w_scale; /* [N] in logical column order                           */
+    const int32_t* w_colsum; /* int4 weights, dense: [N] column sums of the codes (rkh_pack_w4); the
+                              * M <= 8 kernels need them, without them such calls take the MFMA path */
     int epilogue;         /* rkh_epilogue                                          */
     void* C;              /* [M, ldc]                                              */
     int ldc;

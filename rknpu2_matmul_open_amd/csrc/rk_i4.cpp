@@ -58,7 +58,8 @@ int weights_bytes(const rk_npu_i4_weight_config& c, uint64_t* bytes) {
 struct rk_npu_i4i4i32_weights {
     Owner owner;
     rk_npu_i4_weight_config config{};
-    DeviceBuffer tiled; // tiled int4
+    DeviceBuffer tiled;  // tiled int4
+    DeviceBuffer colsum; // [N] int32 column sums of the codes (constant of the decode GEMV's digit split)
 };
 
 struct rk_npu_i4_workspace {
@@ -113,6 +114,7 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
         g.A = ws->a_tiled.as<>();
         g.W = w->tiled.as<>();
         g.w_int4 = 1;
+        g.w_colsum = w->colsum.as<int32_t>();
         g.M = c.M;
         g.N = c.N;
         g.K = c.K;
@@ -202,7 +204,10 @@ rk_npu_i4i4i32_weights* rk_npu_i4i4i32_weights_create(rk_npu_iommu_domain* domai
     if (upload(w->owner, raw, B, (size_t)cfg->K * cfg->N)) return nullptr;
     if (bad.alloc(w->owner, sizeof(int), true)) return nullptr;
     if (w->tiled.alloc(w->owner, rkh_tiled_i4_bytes(cfg->N, cfg->K, RKH_COL_ALIGN), false)) return nullptr;
-    if (rkh_pack_w4(ctx->stream, raw.as<int8_t>(), cfg->K, cfg->N, 0, w->tiled.as<>(), bad.as<int>())) return nullptr;
+    if (w->colsum.alloc(w->owner, (size_t)cfg->N * sizeof(int32_t), true)) return nullptr;
+    if (rkh_pack_w4(ctx->stream, raw.as<int8_t>(), cfg->K, cfg->N, 0, w->tiled.as<>(), bad.as<int>(),
+                    w->colsum.as<int32_t>()))
+        return nullptr;
     int bad_host = 0;
     if (rkh_d2h(ctx->stream, &bad_host, bad.as<>(), sizeof(int)) || rkh_sync(ctx->stream)) return nullptr;
     if (bad_host) return nullptr; // a code outside [-8, 7]

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__
 __global__ __launch_bounds__(256) void pack_w4_kernel(const int8_t* __restrict__ src, int K, int N,
                                                       int KB2, int interleave_F,
                                                       uint8_t* __restrict__ dst, size_t total_chunks,
-                                                      int* bad_flag) {
+                                                      int* bad_flag, int32_t* colsum) {
     const size_t chunk = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (chunk >= total_chunks) return;
     const int lane = (int)(chunk & 63);
@@ -140,6 +140,7 @@ __global__ __launch_bounds__(256) void pack_w4_kernel(const int8_t* __restrict__
     const bool col_ok = interleave_F ? (p < N / 32) : (n < N);
     uint32_t w[4] = {0, 0, 0, 0};
     bool bad = false;
+    int sum = 0; // of this lane's 32 codes: a share of the column sum the GEMV kernels need
     if (col_ok) {
         for (int t = 0; t < 2; ++t) {            // the two 32-k halves of the super-tile
             const int k0 = kb2 * 64 + t * 32 + (lane >> 5) * 16;
@@ -149,6 +150,7 @@ __global__ __launch_bounds__(256) void pack_w4_kernel(const int8_t* __restrict__
                 if (k < K) {
                     code = src[(size_t)k * N + n];
                     if (code < -8 || code > 7) bad = true;
+                    sum += code;
                 }
                 // word = t*2 + j/8 ; within the word: byte (j%8)%4, high nibble when (j%8) >= 4
                 const int k8 = j & 7;
@@ -158,6 +160,7 @@ __global__ __launch_bounds__(256) void pack_w4_kernel(const int8_t* __restrict__
         }
     }
     if (bad && bad_flag) atomicOr(bad_flag, 1);
+    if (colsum && col_ok && sum) atomicAdd(&colsum[n], sum);
     reinterpret_cast<uint4*>(dst)[chunk] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
@@ -628,6 +631,37 @@ __device__ __forceinline__ void store_out(void* C, int epi, size_t index, int ac
     }
 }
 
+// ---- int4 weights in the GEMV kernels: no unpacking --------------------------------
+// An int8 activation code q is split into two signed int4 digits, q = 16 * h + l + 8 with
+// h = q >> 4 and l = (q & 15) - 8 (both in [-8, 7]), so that
+//     sum_k q * w  =  16 * sum_k h * w  +  sum_k l * w  +  8 * sum_k w,
+// and the two digit sums are v_dot8_i32_i4 products against the packed weight words as they
+// lie in memory; the last term is a per-column constant computed at upload.  The staged
+// activations hold, for every 8 consecutive k, one word of h digits and one of l digits in
+// the nibble order of the weight words (byte j: k0 + j low, k0 + 4 + j high).  Unpacking the
+// weights to int8 operands instead took 12 vector instructions per 1 KiB tile and lane on top
+// of 8 dot products, and with every tile of a short K in flight at once that arithmetic, not
+// the stream, was the tail of the kernel.
+__device__ __forceinline__ void split_digits(uint32_t a, uint32_t b, uint32_t& hi, uint32_t& lo) {
+    hi = ((a >> 4) & 0x0F0F0F0Fu) | (b & 0xF0F0F0F0u);
+    lo = ((a & 0x0F0F0F0Fu) | ((b & 0x0F0F0F0Fu) << 4)) ^ 0x88888888u;
+}
+// 16 consecutive int8 codes -> {h, l, h, l} of their two groups of 8
+__device__ __forceinline__ uint4 digits16(uint4 codes) {
+    uint4 r;
+    split_digits(codes.x, codes.y, r.x, r.y);
+    split_digits(codes.z, codes.w, r.z, r.w);
+    return r;
+}
+// Both digit sums of the 16 k a lane holds of one 32-deep half of an int4 super-tile: av = the
+// staged digits {h, l, h, l}, w0 / w1 = the two weight words.
+__device__ __forceinline__ void dot_digits(const v4i& av, int w0, int w1, int& acc_h, int& acc_l) {
+    acc_h = __builtin_amdgcn_sdot8(av.x, w0, acc_h, false);
+    acc_l = __builtin_amdgcn_sdot8(av.y, w0, acc_l, false);
+    acc_h = __builtin_amdgcn_sdot8(av.z, w1, acc_h, false);
+    acc_l = __builtin_amdgcn_sdot8(av.w, w1, acc_l, false);
+}
+
 // ------------------------------------------------------------------ GEMV
 // One workgroup per physical 32-column block; the waves of the group split K
 // (k-tiles interleaved across waves so that neighbouring loads are adjacent in
@@ -687,9 +721,25 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
     const unsigned lane_byte = (unsigned)((col0 + lane % CW) + 32 * half) * 16u;
     // chunk of K staged in LDS at a time (multiple of 64)
     const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
-    int acc[MR], folded[MR];
+    int acc[MR], acc_lo[MR]; // (int4 weights: the sums of the high and of the low activation digits)
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = folded[m] = 0;
+    for (int m = 0; m < MR; ++m) acc[m] = acc_lo[m] = 0;
+
+    // int4 weights: the epilogue's per-column constants (scale, column sum) are requested now.
+    // A matrix of this kind is half the bytes, its stream is over in half the time, and two
+    // dependent round trips to memory at the very end weigh twice as much.  (For int8 weights
+    // the same prefetch was measured and came out 0.1 us slower.)
+    float pre_ws = 1.0f;
+    int pre_cs = 0;
+    if constexpr (W4) {
+        if ((int)threadIdx.x < MR * CW) {
+            const int n = block_first_col(p, g.interleave_F) + col0 + (int)threadIdx.x % CW;
+            if (n < g.N) {
+                pre_ws = g.w_scale ? g.w_scale[n] : 1.0f;
+                pre_cs = g.w_colsum[n];
+            }
+        }
+    }
 
     const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
     const uint8_t* wbase = g.W + (size_t)p * block_bytes;
@@ -780,7 +830,7 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
                 float v[16];
                 RowLoader<T>::unpack(araw[i], v);
                 const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
                 if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
             }
         }
@@ -796,7 +846,7 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
                 const int m = idx / chunks, c = idx - m * chunks;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
             }
         }
         __syncthreads();
@@ -822,27 +872,15 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
                         acc[m] = __builtin_amdgcn_sdot4(av.w, wu.w, acc[m], false);
                     }
                 } else {
-                    // The words pass through an empty asm statement so that their unpacking
-                    // stays here: moved up to where the prefetched group arrived (the compiler
-                    // does that) the sixteen operand words per tile of all eight tiles are live
-                    // across the prologue, more registers than two workgroups per compute unit leave.
-                    int wv[4] = {wu.x, wu.y, wu.z, wu.w};
+                    // (the staged activations of the lane's 16 k of each 32-deep half: digits, see above)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(wv[i]));
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {       // the two 32-k halves
-                        const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
-                        const int hi0 = wv[2 * s] & 0xF0F0F0F0;
-                        const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
-                        const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
+                    for (int s = 0; s < 2; ++s) {
+                        const int w0 = s ? wu.z : wu.x, w1 = s ? wu.w : wu.y;
 #pragma unroll
                         for (int m = 0; m < MR; ++m) {
                             const v4i av = *reinterpret_cast<const v4i*>(
                                 a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
-                            acc[m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[m], false);
-                            acc[m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[m], false);
+                            dot_digits(av, w0, w1, acc[m], acc_lo[m]);
                         }
                     }
                 }
@@ -876,14 +914,8 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
                     acc[0] = __builtin_amdgcn_sdot4(t.a[0].z, wu.z, acc[0], false);
                     acc[0] = __builtin_amdgcn_sdot4(t.a[0].w, wu.w, acc[0], false);
                 } else {
-                    const int wv[4] = {wu.x, wu.y, wu.z, wu.w};
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].x, (wv[2 * s] << 4) & 0xF0F0F0F0, acc[0], false);
-                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].y, wv[2 * s] & 0xF0F0F0F0, acc[0], false);
-                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].z, (wv[2 * s + 1] << 4) & 0xF0F0F0F0, acc[0], false);
-                        acc[0] = __builtin_amdgcn_sdot4(t.a[s].w, wv[2 * s + 1] & 0xF0F0F0F0, acc[0], false);
-                    }
+                    dot_digits(t.a[0], wu.x, wu.y, acc[0], acc_lo[0]);
+                    dot_digits(t.a[1], wu.z, wu.w, acc[0], acc_lo[0]);
                 }
             };
             v4i w[GEMV_UNROLL];
@@ -927,20 +959,11 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
             }
         }
-        if constexpr (W4) {
-            // int4 operands are carried as 16 * code; fold each K chunk's exact
-            // multiple-of-16 partial back so very long K cannot overflow int32.
-#pragma unroll
-            for (int m = 0; m < MR; ++m) {
-                folded[m] += acc[m] >> 4;
-                acc[m] = 0;
-            }
-        }
     }
 
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-        int v = W4 ? folded[m] : acc[m];
+        int v = W4 ? 16 * acc[m] + acc_lo[m] : acc[m];
         v += __shfl_xor(v, 32);
         if (CW <= 16) v += __shfl_xor(v, 16);
         if (CW <= 8) v += __shfl_xor(v, 8);
@@ -955,10 +978,11 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
         const int n = block_first_col(p, g.interleave_F) + col0 + j;
+        if (W4) sum += 8 * pre_cs; // (the constant term of the digit split)
         if (n < g.N)
             store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
                       QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
-                      g.w_scale ? g.w_scale[n] : 1.0f);
+                      W4 ? pre_ws : (g.w_scale ? g.w_scale[n] : 1.0f));
     }
 }
 
@@ -1189,11 +1213,11 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
     const int F = g.interleave_F;
     const int j = blockIdx.x; // 32-column block of the middle
     const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
-    int acc[2][MR], folded[2][MR];
+    int acc[2][MR], acc_lo[2][MR]; // (int4 weights: sums of the high / low activation digits, see split_digits)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int m = 0; m < MR; ++m) acc[b][m] = folded[b][m] = 0;
+        for (int m = 0; m < MR; ++m) acc[b][m] = acc_lo[b][m] = 0;
 
     const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
     const uint8_t* wbase = g.W + (size_t)(2 * j) * block_bytes;    // gate block, the up block right behind it
@@ -1272,7 +1296,7 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
                 float v[16];
                 RowLoader<T>::unpack(araw[i], v);
                 const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
                 if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
             }
         }
@@ -1286,7 +1310,7 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
                 const int m = idx / chunks, c = idx - m * chunks;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
             }
         }
         __syncthreads();
@@ -1310,37 +1334,19 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
                             acc[b][m] = __builtin_amdgcn_sdot4(av.w, w[b][u].w, acc[b][m], false);
                         }
                     } else {
-                        int wv[4] = {w[b][u].x, w[b][u].y, w[b][u].z, w[b][u].w};
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(wv[i])); // (unpack here: see gemv_kernel)
 #pragma unroll
                         for (int s = 0; s < 2; ++s) {
-                            const int lo0 = (wv[2 * s] << 4) & 0xF0F0F0F0;
-                            const int hi0 = wv[2 * s] & 0xF0F0F0F0;
-                            const int lo1 = (wv[2 * s + 1] << 4) & 0xF0F0F0F0;
-                            const int hi1 = wv[2 * s + 1] & 0xF0F0F0F0;
+                            const int w0 = s ? w[b][u].z : w[b][u].x, w1 = s ? w[b][u].w : w[b][u].y;
 #pragma unroll
                             for (int m = 0; m < MR; ++m) {
                                 const v4i av = *reinterpret_cast<const v4i*>(
                                     a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
-                                acc[b][m] = __builtin_amdgcn_sdot4(av.x, lo0, acc[b][m], false);
-                                acc[b][m] = __builtin_amdgcn_sdot4(av.y, hi0, acc[b][m], false);
-                                acc[b][m] = __builtin_amdgcn_sdot4(av.z, lo1, acc[b][m], false);
-                                acc[b][m] = __builtin_amdgcn_sdot4(av.w, hi1, acc[b][m], false);
+                                dot_digits(av, w0, w1, acc[b][m], acc_lo[b][m]);
                             }
                         }
                     }
                 }
             }
-        }
-        if constexpr (W4) { // (codes are carried times 16: fold every chunk's exact multiple of 16 back)
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-#pragma unroll
-                for (int m = 0; m < MR; ++m) {
-                    folded[b][m] += acc[b][m] >> 4;
-                    acc[b][m] = 0;
-                }
         }
     }
 
@@ -1348,7 +1354,7 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
     for (int b = 0; b < 2; ++b)
 #pragma unroll
         for (int m = 0; m < MR; ++m) {
-            int v = W4 ? folded[b][m] : acc[b][m];
+            int v = W4 ? 16 * acc[b][m] + acc_lo[b][m] : acc[b][m];
             v += __shfl_xor(v, 32);
             if (lane < 32) red[b][wave][m][lane] = v;
         }
@@ -1366,6 +1372,10 @@ void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
         }
         uint32_t bits = 0;
         if (live) {
+            if (W4) { // (the constant term of the digit split)
+                gate += 8 * g.w_colsum[n];
+                up += 8 * g.w_colsum[F + n];
+            }
             const float as = QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f);
             const float gf = dequant(gate, as, g.w_scale ? g.w_scale[n] : 1.0f);
             const float uf = dequant(up, as, g.w_scale ? g.w_scale[F + n] : 1.0f);
@@ -2833,6 +2843,7 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 // The decode path can quantize inside the GEMV when the rows fit the kernel's
 // LDS staging and per-thread register cache.
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
+    if (g.w_int4 && !g.w_colsum) return false;
     if (g.blk_expert || g.M > 8 || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
@@ -2994,12 +3005,12 @@ int rkh_pack_w8(void* stream, const int8_t* src, int K, int N, int interleave_F,
 }
 
 int rkh_pack_w4(void* stream, const int8_t* src, int K, int N, int interleave_F, uint8_t* dst,
-                int* bad_flag) {
+                int* bad_flag, int32_t* colsum) {
     const int KB2 = (int)(rkh_align_up(K, RKH_K_ALIGN) / 64);
     const size_t pblocks = (size_t)(rkh_align_up(N, RKH_COL_ALIGN) / 32);
     const size_t chunks = pblocks * KB2 * 64;
     hipLaunchKernelGGL(pack_w4_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, src, K, N, KB2, interleave_F, dst, chunks, bad_flag);
+                       (hipStream_t)stream, src, K, N, KB2, interleave_F, dst, chunks, bad_flag, colsum);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
@@ -3119,8 +3130,9 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     const rkh_gemm_args& g = *args;
     hipStream_t st = (hipStream_t)stream;
     const bool grouped = g.blk_expert != nullptr;
-    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU) return dispatch_gemv(st, g, nullptr);
-    if (gemv_swiglu_applies(g)) return dispatch_gemv_swiglu(st, g, nullptr);
+    const bool gemv_ok = !g.w_int4 || g.w_colsum; // (the int4 GEMV kernels need the column sums)
+    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU && gemv_ok) return dispatch_gemv(st, g, nullptr);
+    if (gemv_swiglu_applies(g) && gemv_ok) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
     const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);

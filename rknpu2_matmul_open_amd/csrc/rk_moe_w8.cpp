@@ -395,11 +395,11 @@ int pack_expert(rk_npu_moe_w8_weights* w, DeviceBuffer& raw, int e, const rk_npu
     const int e8 = e - w->count4;
     int rc = rkh_h2d(stream, raw.as<>(), x.gate_up, (size_t)H * 2 * I);
     if (!rc)
-        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up4.as<>() + w->gate_stride4 * e, nullptr)
+        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up4.as<>() + w->gate_stride4 * e, nullptr, nullptr)
                   : rkh_pack_w8(stream, raw.as<int8_t>(), H, 2 * I, I, w->gate_up.as<>() + w->gate_stride * e8);
     if (!rc) rc = rkh_h2d(stream, raw.as<>(), x.down, (size_t)I * H);
     if (!rc)
-        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), I, H, 0, w->down4.as<>() + w->down_stride4 * e, nullptr)
+        rc = int4 ? rkh_pack_w4(stream, raw.as<int8_t>(), I, H, 0, w->down4.as<>() + w->down_stride4 * e, nullptr, nullptr)
                   : rkh_pack_w8(stream, raw.as<int8_t>(), I, H, 0, w->down.as<>() + w->down_stride * e8);
     if (!rc) rc = rkh_h2d(stream, w->gate_scales.as<float>() + (size_t)e * 2 * I, x.gate_up_scales, (size_t)2 * I * sizeof(float));
     if (!rc) rc = rkh_h2d(stream, w->down_scales.as<float>() + (size_t)e * H, x.down_scales, (size_t)H * sizeof(float));

@@ -221,6 +221,7 @@ struct rk_npu_w4a8_weights {
     int interleave_F = 0;  // N/2 when N % 64 == 0 (gate/up column blocks interleaved)
     DeviceBuffer tiled;    // tiled int4
     DeviceBuffer w_scale;  // [N]
+    DeviceBuffer colsum;   // [N] int32: sum over k of the codes of a column (decode GEMV constant)
 };
 
 struct rk_npu_w4a8_workspace {
@@ -316,6 +317,7 @@ rkh_gemm_args gemm_args(rk_npu_w4a8_workspace* ws, const rk_npu_w4a8_weights* w,
     g.interleave_F = w->interleave_F;
     g.a_scale = ws->a_scale.as<float>();
     g.w_scale = w->w_scale.as<float>();
+    g.w_colsum = w->colsum.as<int32_t>();
     g.C = dC;
     g.splitk_acc = ws->splitk ? ws->splitk.as<int32_t>() : nullptr;
     switch (out) {
@@ -486,8 +488,9 @@ rk_npu_w4a8_weights* w4a8_create_weights(rk_npu_iommu_domain* domain, const rk_n
     if (upload(w->owner, raw, B, (size_t)cfg.K * cfg.N)) return nullptr;
     if (bad.alloc(w->owner, sizeof(int), true)) return nullptr;
     if (w->tiled.alloc(w->owner, rkh_tiled_i4_bytes(cfg.N, cfg.K, RKH_COL_ALIGN), false)) return nullptr;
+    if (w->colsum.alloc(w->owner, (size_t)cfg.N * sizeof(int32_t), true)) return nullptr;
     if (rkh_pack_w4(ctx->stream, raw.as<int8_t>(), cfg.K, cfg.N, w->interleave_F, w->tiled.as<>(),
-                    bad.as<int>()))
+                    bad.as<int>(), w->colsum.as<int32_t>()))
         return nullptr;
     if (upload(w->owner, w->w_scale, w_scale, (size_t)cfg.N * sizeof(float))) return nullptr;
     int bad_host = 0;
