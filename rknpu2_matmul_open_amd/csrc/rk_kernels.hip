@@ -725,22 +725,6 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[m] = acc_lo[m] = 0;
 
-    // int4 weights: the epilogue's per-column constants (scale, column sum) are requested now.
-    // A matrix of this kind is half the bytes, its stream is over in half the time, and two
-    // dependent round trips to memory at the very end weigh twice as much.  (For int8 weights
-    // the same prefetch was measured and came out 0.1 us slower.)
-    float pre_ws = 1.0f;
-    int pre_cs = 0;
-    if constexpr (W4) {
-        if ((int)threadIdx.x < MR * CW) {
-            const int n = block_first_col(p, g.interleave_F) + col0 + (int)threadIdx.x % CW;
-            if (n < g.N) {
-                pre_ws = g.w_scale ? g.w_scale[n] : 1.0f;
-                pre_cs = g.w_colsum[n];
-            }
-        }
-    }
-
     const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
     const uint8_t* wbase = g.W + (size_t)p * block_bytes;
     // Weight loads go through a buffer descriptor over this column block: a load whose offset
@@ -978,11 +962,11 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
         const int n = block_first_col(p, g.interleave_F) + col0 + j;
-        if (W4) sum += 8 * pre_cs; // (the constant term of the digit split)
+        if (W4 && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
         if (n < g.N)
             store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
                       QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
-                      W4 ? pre_ws : (g.w_scale ? g.w_scale[n] : 1.0f));
+                      g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
 
