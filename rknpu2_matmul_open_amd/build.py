@@ -20,6 +20,9 @@ SOURCES = ["rk_kernels.hip", "rk_core.cpp", "rk_quant_matmul.cpp", "rk_autotune.
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # leading scalar kernel arguments arrive in registers at wave start (14 dwords is what the
+    # hardware's user registers hold beside the argument pointer)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall", "-Wno-unused-function",
     "-I" + CSRC, "-I" + os.path.join(ROOT, "include"),
 ]

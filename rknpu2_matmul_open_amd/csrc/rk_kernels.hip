@@ -309,6 +309,35 @@ __device__ __forceinline__ uint4 quantize16(const float* v, float inv) {
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// ---- leading scalar arguments
+// The first 14 dwords of a kernel's scalar arguments arrive in registers when a wave starts
+// (kernel-argument preload, switched on by the build's -amdgpu-kernarg-preload-count);
+// a structure passed by value is fetched from memory by every wave, one more round trip ahead
+// of its first data load.  The hot kernels therefore repeat, ahead of their argument
+// structure, the fields their first loads depend on, and copy them back over the structure.
+#define RK_QUANT_HEAD_PARAMS                                                                          \
+    const void* h_src, const int* h_active, const uint32_t* h_row_max, int h_M, int h_K, int h_mode, int h_parts
+#define RK_QUANT_HEAD(a) (a).src, (a).active_blocks, (a).row_max_bits, (a).M, (a).K, (a).mode, (a).row_max_parts
+#define RK_QUANT_HEAD_APPLY(a)                                                                        \
+    do {                                                                                              \
+        (a).src = h_src; (a).active_blocks = h_active; (a).row_max_bits = h_row_max;                  \
+        (a).M = h_M; (a).K = h_K; (a).mode = h_mode; (a).row_max_parts = h_parts;                     \
+    } while (0)
+#define RK_GEMM_HEAD_PARAMS                                                                           \
+    const uint8_t* h_A, const uint8_t* h_W, const uint8_t* h_W4, const int* h_blk_expert, const int* h_num_blocks, \
+        int h_M, int h_K, int h_int4_experts
+#define RK_GEMM_HEAD(g) (g).A, (g).W, (g).W4, (g).blk_expert, (g).num_blocks, (g).M, (g).K, (g).int4_experts
+#define RK_GEMM_HEAD_APPLY(g)                                                                         \
+    do {                                                                                              \
+        (g).A = h_A; (g).W = h_W; (g).W4 = h_W4; (g).blk_expert = h_blk_expert;                       \
+        (g).num_blocks = h_num_blocks; (g).M = h_M; (g).K = h_K; (g).int4_experts = h_int4_experts;   \
+    } while (0)
+#define RK_SCATTER_HEAD(a) (a).ids, (a).routes, (a).src, (a).rows, (a).top_k, (a).experts, (a).shared, (a).K
+#define RK_GEMV_HEAD_PARAMS const uint8_t* h_W, const void* h_src, int h_M, int h_K
+#define RK_GEMV_HEAD(g, q) (g).W, (q).src, (g).M, (g).K
+#define RK_GEMV_HEAD_APPLY(g, q)                                                                      \
+    do { (g).W = h_W; (q).src = h_src; (g).M = h_M; (g).K = h_K; } while (0)
+
 constexpr int QR_CACHE = 4; // 16-element chunks kept in registers per thread
 
 // `split` workgroups share a row (blockIdx.x = row * split + part), each taking a
@@ -316,7 +345,8 @@ constexpr int QR_CACHE = 4; // 16-element chunks kept in registers per thread
 // row for its maximum are launched with split > 1: re-quantization finds the
 // maximum in the partial maxima the GEMM left behind, which every part reads.
 template <typename T>
-__global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int split) {
+__global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, int split, rkh_quant_args a) {
+    RK_QUANT_HEAD_APPLY(a);
     __shared__ float wave_max[4];
     __shared__ int wave_bad[4];
     const int m = blockIdx.x / split, part = blockIdx.x - m * split, t = threadIdx.x;
@@ -450,7 +480,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(rkh_quant_args a, int s
 // the partial maxima the SwiGLU epilogue left behind, so a row needs no
 // workgroup-wide reduction; with a workgroup per row three of its four waves
 // had nothing to do.  Rows of up to 64 * QR_CACHE chunks.
-__global__ __launch_bounds__(256) void requant_rows_wave_kernel(rkh_quant_args a) {
+__global__ __launch_bounds__(256) void requant_rows_wave_kernel(RK_QUANT_HEAD_PARAMS, rkh_quant_args a) {
+    RK_QUANT_HEAD_APPLY(a);
     const int lane = lane_id(), m = blockIdx.x * 4 + wave_id();
     if (m >= a.M || (a.active_blocks && m >= a.active_blocks[0] * 32)) return;
     const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
@@ -503,7 +534,8 @@ __global__ __launch_bounds__(256) void requant_rows_wave_kernel(rkh_quant_args a
 constexpr int Q8_CACHE = 8;
 
 template <typename T, int ROWS>
-__global__ __launch_bounds__(256) void quant_rows8_kernel(rkh_quant_args a) {
+__global__ __launch_bounds__(256) void quant_rows8_kernel(RK_QUANT_HEAD_PARAMS, rkh_quant_args a) {
+    RK_QUANT_HEAD_APPLY(a);
     static_assert(ROWS == 8 || ROWS == 4, "rows per workgroup");
     constexpr int CPW = 64 / ROWS;    // chunk columns per wave instruction
     constexpr int CSTEP = 4 * CPW;    // chunk columns per workgroup pass
@@ -697,7 +729,8 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 // and the cross-lane reduction takes two or three xor-shuffles instead of one.
 template <int MR, bool W4, int QT, int CW>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
-void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
+void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
+    RK_GEMV_HEAD_APPLY(g, q);
     static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
     constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
     // (padding for the single-row variants of narrow matrices: their look-ahead of GEMV_UNROLL loads per wave, and
@@ -987,7 +1020,8 @@ void gemv_kernel(rkh_gemm_args g, rkh_quant_args q) {
 // faster on gemv_kernel (7.8 against 8.3 us) and stay there.
 template <int QT>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
-void gemv_wide8_kernel(rkh_gemm_args g, rkh_quant_args q) {
+void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
+    RK_GEMV_HEAD_APPLY(g, q);
     constexpr int MR = 1;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
@@ -1185,7 +1219,8 @@ constexpr int GEMV_SWIGLU_UNROLL = 4; // load instructions per wave and block in
 // rows q.src itself (same prologue: rows requested first, then the first group of weights).
 template <int MR, bool W4, int QT>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
-void gemv_swiglu_kernel(rkh_gemm_args g, rkh_quant_args q) {
+void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
+    RK_GEMV_HEAD_APPLY(g, q);
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[2][GEMV_WAVES][MR][32];
     __shared__ uint32_t row_max[MR];
@@ -1617,8 +1652,9 @@ __device__ __forceinline__ void wk_tile_coords(int tile, int mblocks, int nblock
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm" // m0 is set and clobbered on purpose below
 template <int TM, bool W4, int EPI>
-__global__ __launch_bounds__(512) void gemm_wk_kernel(rkh_gemm_args g, int mblocks, int nblocks, int ksplit,
-                                                      int ksteps_per_part) {
+__global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int mblocks, int nblocks, int ksplit,
+                                                      int ksteps_per_part, rkh_gemm_args g) {
+    RK_GEMM_HEAD_APPLY(g);
     constexpr int TN = 2, KTS = 8 / TM, KTW = KTS / 2; // k-tiles per sub-step: all / this wave's
     constexpr int NSW = (TM == 4 || (TM == 2 && W4)) ? 8 : 4;
     constexpr int NBUF = WK_NBUF, G = WK_G, D = WK_D, BM = 32 * TM, BUF = WK_BUF;
@@ -2040,7 +2076,9 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // has its launch over the same grid, and a workgroup whose row block belongs to
 // an expert of the other format exits at once.
 template <int EPI, int KS, bool W4, bool BAL = false>
-__global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(rkh_gemm_args g, int mblocks, int nblocks) {
+__global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HEAD_PARAMS, int mblocks, int nblocks,
+                                                                      rkh_gemm_args g) {
+    RK_GEMM_HEAD_APPLY(g);
     constexpr int TN = 2, WAVES = BAL ? 8 : 4;
     constexpr bool KSPLIT = KS > 1;
     static_assert(!BAL || !KSPLIT, "the balanced variant does not split K");
@@ -2286,7 +2324,12 @@ constexpr int ROUTE_MAX_TOPK = 8;
 constexpr int ROUTE_MAX_ASSIGNMENTS = 2048; // rows * top_k
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a) {
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const int32_t* h_ids, const float* h_routes, const void* h_src,
+                                                          int h_rows, int h_top_k, int h_experts, int h_shared, int h_K,
+                                                          rkh_moe_scatter_args a) {
+    // (leading scalar arguments: see RK_GEMM_HEAD_PARAMS)
+    a.ids = h_ids; a.routes = h_routes; a.src = h_src;
+    a.rows = h_rows; a.top_k = h_top_k; a.experts = h_experts; a.shared = h_shared; a.K = h_K;
     __shared__ int bins[4][ROUTE_MAX_EXPERTS];   // live assignments per expert, per wave
     __shared__ int start[ROUTE_MAX_EXPERTS + 1]; // first sorted row of each bucket
     __shared__ int own_key[ROUTE_MAX_TOPK], own_rank[ROUTE_MAX_TOPK], own_wave[ROUTE_MAX_TOPK];
@@ -2512,7 +2555,10 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(rkh_moe_scatter_args a
 
 // out[t, n] = sum over slots, in slot order, of fma(Y[dest, n], w, out); the
 // shared expert is the last slot with coefficient 1.
-__global__ __launch_bounds__(256) void moe_combine_kernel(rkh_moe_combine_args a) {
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* h_Y, const int* h_dest_rows, const float* h_routes,
+                                                          float* h_out, int h_rows, int h_top_k, int h_shared, int h_H) {
+    // (every field as a leading scalar argument: see RK_GEMM_HEAD_PARAMS)
+    const rkh_moe_combine_args a = {h_Y, h_dest_rows, h_routes, h_rows, h_top_k, h_shared, h_H, h_out};
     const int tkn = blockIdx.y;
     const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (n >= a.H) return;
@@ -2653,8 +2699,8 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
         const dim3 grid(cus), block(512);
 #define RK_LAUNCH_BAL(EPI)                                                                                          \
     do {                                                                                                            \
-        if (any_int4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true, true>), grid, block, 0, st, g, mblocks, nblocks);  \
-        if (any_int8) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false, true>), grid, block, 0, st, g, mblocks, nblocks); \
+        if (any_int4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);  \
+        if (any_int8) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); \
     } while (0)
         switch (g.epilogue) {
         case RKH_EPI_I32: RK_LAUNCH_BAL(RKH_EPI_I32); break;
@@ -2672,13 +2718,13 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
 #define RK_LAUNCH(EPI)                                                                                         \
     do {                                                                                                       \
         if (any_int4 && ks == 4)                                                                               \
-            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true>), grid, block, 0, st, g, mblocks, nblocks);   \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);   \
         else if (any_int4)                                                                                     \
-            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true>), grid, block, 0, st, g, mblocks, nblocks);   \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);   \
         if (any_int8 && ks == 4)                                                                               \
-            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, false>), grid, block, 0, st, g, mblocks, nblocks);  \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, false>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);  \
         else if (any_int8)                                                                                     \
-            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false>), grid, block, 0, st, g, mblocks, nblocks);  \
+            hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);  \
     } while (0)
     switch (g.epilogue) {
     case RKH_EPI_I32: RK_LAUNCH(RKH_EPI_I32); break;
@@ -2722,8 +2768,8 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
                                           hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES)); \
             opted_in[dev] = true;                                                                   \
         }                                                                                           \
-        hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st, g, mblocks, \
-                           nblocks, ksplit, per);                                                   \
+        hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st,           \
+                           RK_GEMM_HEAD(g), mblocks, nblocks, ksplit, per, g);                      \
         if (ksplit > 1) mark(st, "gemm_wk_reduce_kernel");                                          \
         if (ksplit > 1)                                                                             \
             hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>),                                \
@@ -2763,18 +2809,18 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
     if (MR == 1 && !g.w_int4 && cw == 32) { // (see gemv_wide8_kernel)
         mark(st, qt ? "gemv_wide8_kernel (fused quantize)" : "gemv_wide8_kernel");
-        if (qt == 0) hipLaunchKernelGGL((gemv_wide8_kernel<0>), grid, block, 0, st, g, q);
-        else if (qt == 1) hipLaunchKernelGGL((gemv_wide8_kernel<1>), grid, block, 0, st, g, q);
-        else hipLaunchKernelGGL((gemv_wide8_kernel<2>), grid, block, 0, st, g, q);
+        if (qt == 0) hipLaunchKernelGGL((gemv_wide8_kernel<0>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else if (qt == 1) hipLaunchKernelGGL((gemv_wide8_kernel<1>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else hipLaunchKernelGGL((gemv_wide8_kernel<2>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
     mark(st, qt ? "gemv_kernel (fused quantize)" : "gemv_kernel");
 #define RK_GEMV(W4, QT)                                                                        \
     do {                                                                                       \
-        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, g, q);        \
-        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, g, q); \
-        else hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, g, q);               \
+        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
+        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q); \
+        else hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
     } while (0)
     if (g.w_int4) {
         if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
@@ -2792,7 +2838,7 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
     mark(st, qt ? "gemv_swiglu_kernel (fused quantize)" : "gemv_swiglu_kernel");
-#define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, g, q)
+#define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q)
     if (g.w_int4) {
         if (qt == 0) RK_SWI(true, 0); else if (qt == 1) RK_SWI(true, 1); else RK_SWI(true, 2);
     } else {
@@ -3010,11 +3056,11 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
         const hipStream_t st = (hipStream_t)stream;
         mark(st, "quant_rows8_kernel");
         if (args->in_dtype == RKH_F16) {
-            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 4>), grid, block, 0, st, *args);
-            else hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 8>), grid, block, 0, st, *args);
+            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 4>), grid, block, 0, st, RK_QUANT_HEAD(*args), *args);
+            else hipLaunchKernelGGL((quant_rows8_kernel<uint16_t, 8>), grid, block, 0, st, RK_QUANT_HEAD(*args), *args);
         } else {
-            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<float, 4>), grid, block, 0, st, *args);
-            else hipLaunchKernelGGL((quant_rows8_kernel<float, 8>), grid, block, 0, st, *args);
+            if (rows4) hipLaunchKernelGGL((quant_rows8_kernel<float, 4>), grid, block, 0, st, RK_QUANT_HEAD(*args), *args);
+            else hipLaunchKernelGGL((quant_rows8_kernel<float, 8>), grid, block, 0, st, RK_QUANT_HEAD(*args), *args);
         }
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
@@ -3022,7 +3068,8 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     const bool reuse = mode == RKH_Q_REUSE_BITS || mode == RKH_Q_REUSE_BITS_MOE;
     if (reuse && args->in_dtype == RKH_F32 && args->M >= 64 && (args->K + 15) / 16 <= 64 * QR_CACHE) {
         mark((hipStream_t)stream, "requant_rows_wave_kernel");
-        hipLaunchKernelGGL(requant_rows_wave_kernel, dim3((args->M + 3) / 4), block, 0, (hipStream_t)stream, *args);
+        hipLaunchKernelGGL(requant_rows_wave_kernel, dim3((args->M + 3) / 4), block, 0, (hipStream_t)stream,
+                           RK_QUANT_HEAD(*args), *args);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
@@ -3036,9 +3083,9 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     const dim3 grid(args->M * split);
     mark((hipStream_t)stream, "quant_rows_kernel");
     switch (args->in_dtype) {
-    case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *args, split); break;
-    case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, *args, split); break;
-    case RKH_I8: hipLaunchKernelGGL(quant_rows_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args, split); break;
+    case RKH_F16: hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, RK_QUANT_HEAD(*args), split, *args); break;
+    case RKH_F32: hipLaunchKernelGGL(quant_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, RK_QUANT_HEAD(*args), split, *args); break;
+    case RKH_I8: hipLaunchKernelGGL(quant_rows_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, RK_QUANT_HEAD(*args), split, *args); break;
     default: return RKH_ERR_RUNTIME;
     }
     RKH_CHECK(hipGetLastError());
@@ -3158,9 +3205,9 @@ int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args) {
     const dim3 grid(args->rows), block(256);
     mark((hipStream_t)stream, "moe_scatter_kernel");
     if (args->in_dtype == RKH_F32)
-        hipLaunchKernelGGL(moe_scatter_kernel<float>, grid, block, 0, (hipStream_t)stream, *args);
+        hipLaunchKernelGGL(moe_scatter_kernel<float>, grid, block, 0, (hipStream_t)stream, RK_SCATTER_HEAD(*args), *args);
     else if (args->in_dtype == RKH_I8)
-        hipLaunchKernelGGL(moe_scatter_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, *args);
+        hipLaunchKernelGGL(moe_scatter_kernel<int8_t>, grid, block, 0, (hipStream_t)stream, RK_SCATTER_HEAD(*args), *args);
     else
         return RKH_ERR_RUNTIME;
     RKH_CHECK(hipGetLastError());
@@ -3170,7 +3217,8 @@ int rkh_moe_scatter(void* stream, const rkh_moe_scatter_args* args) {
 int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args) {
     const dim3 grid((args->H / 4 + 255) / 256, args->rows);
     mark((hipStream_t)stream, "moe_combine_kernel");
-    hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, (hipStream_t)stream, *args);
+    hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, (hipStream_t)stream, args->Y, args->dest_rows,
+                       args->routes, args->out, args->rows, args->top_k, args->shared, args->H);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
