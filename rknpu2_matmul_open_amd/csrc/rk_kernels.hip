@@ -1018,10 +1018,16 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 // gemv_kernel's exact waits (11.4 with an explicit wait for the whole group in
 // front of the prologue or of the K loop).  Int4 matrices of the same shape are
 // faster on gemv_kernel (7.8 against 8.3 us) and stay there.
+// Tried on this kernel and slower, same box, 10.6 us as it stands: a second group of tiles
+// requested before the prologue (11.0 us; all 16 loads of a wave requested at the start: 12.2),
+// the wave index read into a scalar register (10.85: the branches around the loads become
+// scalar and the compiler counts the loads exactly again), the column scales of the epilogue
+// fetched with the first loads (10.7).
 template <int QT>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     RK_GEMV_HEAD_APPLY(g, q);
+    RK_TS(0);
     constexpr int MR = 1;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
     __shared__ int red[GEMV_WAVES][MR][32];
@@ -1040,17 +1046,25 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 
     const uint8_t* wbase = g.W + (size_t)p * KB * 1024;
 
-    // Fused path: put the first batch of weight loads in flight before the
-    // quantization prologue so that its latency hides behind them.
-    // The activation rows are requested FIRST: loads return in issue order, so
-    // behind the weight loads they would arrive with the last of those, and the
-    // prologue (and with it the second batch of weight loads) would start only
-    // then.  Fetched first they are back after one L2 round trip and the whole
-    // quantization runs under the weight loads' latency.
+    // Fused path: the first group of weight loads goes out ahead of everything else, then the
+    // activation rows.  This kernel waits for all of its loads wherever it needs one (see
+    // above), so the order of the requests does not change what the prologue waits for, and
+    // the weight requests are a dozen instructions from the kernel's entry instead of behind
+    // the row loader's code (in-kernel time stamps: 2.4 us from a wave's start until its weight
+    // requests were out; 4096 x 14336: 10.6 us against 10.9 us with the rows requested first).
     v4i wpre[GEMV_UNROLL];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
     typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
     if constexpr (QT != 0) {
+        const int tiles = Kp >> 5;
+#pragma unroll
+        for (int u = 0; u < GEMV_UNROLL; ++u) {
+            const int tt = wave + u * GEMV_WAVES;
+            wpre[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                       wbase + (size_t)tt * 1024 + lane * 16))
+                                 : v4i{0, 0, 0, 0};
+        }
+        __builtin_amdgcn_sched_barrier(0);
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
 #pragma unroll
         for (int i = 0; i < GEMV_QCHUNKS; ++i) {
@@ -1062,15 +1076,7 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        const int tiles = Kp >> 5;
-#pragma unroll
-        for (int u = 0; u < GEMV_UNROLL; ++u) {
-            const int tt = wave + u * GEMV_WAVES;
-            wpre[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                       wbase + (size_t)tt * 1024 + lane * 16))
-                                 : v4i{0, 0, 0, 0};
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        RK_TS(4);
     }
     if constexpr (QT != 0) {
         using T = QT_T;
@@ -1078,6 +1084,7 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
         if (t < MR) row_max[t] = 0u;
         __syncthreads();
+        RK_TS(5);
         // (the rows stay in registers as fetched and are converted once per pass:
         // holding them as floats across the barriers costs the int4 variants their
         // second workgroup per compute unit)
@@ -1126,6 +1133,7 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
         }
         // a_scale of the epilogue comes from LDS in this path
+        RK_TS(1);
     }
 
     for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
@@ -1180,6 +1188,7 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         }
     }
 
+    RK_TS(2);
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         int v = acc[m];
@@ -1191,6 +1200,7 @@ void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     if ((int)threadIdx.x < MR * 32) {
         const int m = (int)threadIdx.x >> 5, j = (int)threadIdx.x & 31;
         if (m >= g.M) return;
+        RK_TS(3);
         int sum = 0;
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
@@ -2272,6 +2282,10 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
         __builtin_amdgcn_wave_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // (read before the staging below overwrites the area)
     }
+    // (The epilogue is bound by its vector ALU work -- some 800 instructions of a wave for the
+    // SwiGLU pair, 4 cycles each, two waves per SIMD: 4.3 us measured at the end of a unit whose
+    // loop takes 14 us, 1.9 us for the plain fp32 tile pair.  A dry pass through the same code
+    // while the first loads were in flight, to have it in the instruction cache, changed nothing.)
     if constexpr (EPI == RKH_EPI_SWIGLU) {
         epilogue_swiglu_scaled(g, acc[0], acc[1], m0, pb0, lane, as, ws[0], ws[1], m_limit, stage_lds);
     } else {
