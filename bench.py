@@ -137,7 +137,7 @@ def bench_c1(sess, ops, capi, workloads, steps, warmup, cpu_baseline):
         "config": {"workload": "c1: w8a8 decode GEMV M=1 K=4096 N=14336, fp16 in/out, seeds 2/3",
                    "value_is": "int8 weight bytes (58720256) / step time; step = one fused quantize+GEMV kernel; "
                                "the loop cycles through %d copies of the matrix so that every step reads HBM" % C1_COPIES},
-        "roofline": _hbm("gemv_wide8_kernel<1> (fused per-token quantize + GEMV)", algo_bytes, step_us, "gemv_c1",
+        "roofline": _hbm("gemv_kernel<1,false,1,32,burst> (fused per-token quantize + GEMV)", algo_bytes, step_us, "gemv_c1",
                          kernel_us=step_us, gemv_without_quantize_us=gemv_only_us,
                          same_matrix_every_step_us=same_matrix_us, replayed_from_graph_us=graph_us),
     }

@@ -6,7 +6,7 @@
 //   quant_rows_kernel                   per-token absmax + int8 codes, workgroup per row (HBM, small)
 //   quant_rows8_kernel                  the same for many rows, 8 / 4 rows per workgroup (HBM)
 //   requant_rows_wave_kernel            re-quantize short fp32 rows, wave per row        (HBM, small)
-//   gemv_kernel / gemv_wide8_kernel     M <= 8 decode path: dot4, no MFMA, optional fused
+//   gemv_kernel                         M <= 8 decode path: dot4, no MFMA, optional fused
 //                                       per-token quantization                           (HBM)
 //   gemv_swiglu_kernel                  gate/up + SwiGLU of one or two rows              (HBM)
 //   gemm_wk_kernel                      int8 MFMA 32x32x32, (32..128) x 256 tiles, activations
@@ -727,11 +727,32 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 // then covers the workgroup's part of 32 / CW consecutive k-tiles (pieces of
 // 16 * CW bytes): lane = column % CW + CW * k-half + 2 * CW * (tile of the group),
 // and the cross-lane reduction takes two or three xor-shuffles instead of one.
-template <int MR, bool W4, int QT, int CW>
+//
+// BURST (one int8 row of a wide matrix, more than 256 column blocks -- the decode shape of the
+// benchmark): the loads past the end of K are skipped by branches instead of being sent through
+// the bounds-checked descriptor.  With the branches the compiler no longer counts the
+// outstanding loads exactly and waits for ALL of a wave's loads wherever it needs one of them --
+// so every wave of a workgroup has its whole group of tiles before the quantization prologue
+// starts, passes the prologue's barriers with nothing outstanding, uses the group at once and
+// asks for the next group in one burst together with the other seven waves.  For a matrix that
+// is bound by memory throughput that is the faster order, measured on one box for 4096 x 14336:
+// 11.05 us against 11.5 us with exact waits (11.4 with an explicit wait for the whole group in
+// front of the prologue or of the K loop).  Int4 matrices of the same shape are faster with
+// exact waits (7.8 against 8.3 us).  Since the prologue waits for everything anyway, the weight
+// tiles are requested ahead of the activation rows, a dozen instructions from the kernel's
+// entry instead of behind the row loader's code (in-kernel time stamps: 2.4 us from a wave's
+// start until its weight requests were out; 10.9 -> 10.6 us).  Tried on this variant and slower,
+// same box, against 10.6 us: a second group of tiles requested before the prologue (11.0 us; all
+// 16 loads of a wave requested at the start: 12.2), the wave index read into a scalar register
+// (10.85: the branches around the loads become scalar and the compiler counts the loads exactly
+// again), the column scales of the epilogue fetched with the first loads (10.7).
+template <int MR, bool W4, int QT, int CW, bool BURST = false>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     RK_GEMV_HEAD_APPLY(g, q);
+    RK_TS(0);
     static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
+    static_assert(!BURST || (MR == 1 && !W4 && CW == 32), "the burst variant serves one int8 row, whole column blocks");
     constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
     // (padding for the single-row variants of narrow matrices: their look-ahead of GEMV_UNROLL loads per wave, and
     // one more step for the activations, runs up to that many load instructions past the end
@@ -767,8 +788,14 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     const __amdgpu_buffer_rsrc_t wrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)block_bytes, 0x00020000);
     auto load_tile = [&](int unit, int units, int first_tile) -> v4i { // `unit` counts this wave's load instructions
-        const unsigned off = unit < units ? (unsigned)(first_tile + unit * TPL + sub) * 1024u + lane_byte : 0xFFFFFFF0u;
-        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+        if constexpr (BURST) {
+            return unit < units ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                      wbase + (size_t)(first_tile + unit) * 1024 + lane * 16))
+                                : v4i{0, 0, 0, 0};
+        } else {
+            const unsigned off = unit < units ? (unsigned)(first_tile + unit * TPL + sub) * 1024u + lane_byte : 0xFFFFFFF0u;
+            return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+        }
     };
 
     // Fused path: put the first batch of weight loads in flight before the
@@ -777,11 +804,17 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // behind the weight loads they would arrive with the last of those, and the
     // prologue (and with it the second batch of weight loads) would start only
     // then.  Fetched first they are back after one L2 round trip and the whole
-    // quantization runs under the weight loads' latency.
+    // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
     v4i wpre[GEMV_UNROLL];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
     typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
     if constexpr (QT != 0) {
+        const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
+        if constexpr (BURST) {
+#pragma unroll
+            for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
 #pragma unroll
         for (int i = 0; i < GEMV_QCHUNKS; ++i) {
@@ -793,10 +826,12 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
+        if constexpr (!BURST) {
 #pragma unroll
-        for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        RK_TS(4);
     }
     if constexpr (QT != 0) {
         using T = QT_T;
@@ -1002,216 +1037,6 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                       g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
-
-
-// ---- single-row int8 GEMV of a wide matrix (more than 256 column blocks) ----
-// The same workgroup layout as gemv_kernel<1, false, QT, 32>, but with the
-// loads past the end of K skipped by branches instead of being sent through a
-// bounds-checked descriptor.  With the branches the compiler no longer counts
-// the outstanding loads exactly and waits for ALL of a wave's loads wherever it
-// needs one of them -- so every wave of a workgroup has its whole group of tiles
-// before the quantization prologue starts, passes the prologue's barriers with
-// nothing outstanding, uses the group at once and asks for the next group in
-// one burst together with the other seven waves.  For a matrix that is bound
-// by memory throughput that is the faster order, measured on one box for
-// 4096 x 14336 (the decode shape of the benchmark): 11.05 us against 11.5 us for
-// gemv_kernel's exact waits (11.4 with an explicit wait for the whole group in
-// front of the prologue or of the K loop).  Int4 matrices of the same shape are
-// faster on gemv_kernel (7.8 against 8.3 us) and stay there.
-// Tried on this kernel and slower, same box, 10.6 us as it stands: a second group of tiles
-// requested before the prologue (11.0 us; all 16 loads of a wave requested at the start: 12.2),
-// the wave index read into a scalar register (10.85: the branches around the loads become
-// scalar and the compiler counts the loads exactly again), the column scales of the epilogue
-// fetched with the first loads (10.7).
-template <int QT>
-__global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
-void gemv_wide8_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
-    RK_GEMV_HEAD_APPLY(g, q);
-    RK_TS(0);
-    constexpr int MR = 1;
-    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
-    __shared__ int red[GEMV_WAVES][MR][32];
-    __shared__ uint32_t row_max[MR];
-    __shared__ float row_scale[MR];
-    const int lane = lane_id(), wave = wave_id();
-    const int half = lane >> 5;
-    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
-    const int KB = Kp / 32;
-    const int p = blockIdx.x;
-    // chunk of K staged in LDS at a time (multiple of 64)
-    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
-    int acc[MR];
-#pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = 0;
-
-    const uint8_t* wbase = g.W + (size_t)p * KB * 1024;
-
-    // Fused path: the first group of weight loads goes out ahead of everything else, then the
-    // activation rows.  This kernel waits for all of its loads wherever it needs one (see
-    // above), so the order of the requests does not change what the prologue waits for, and
-    // the weight requests are a dozen instructions from the kernel's entry instead of behind
-    // the row loader's code (in-kernel time stamps: 2.4 us from a wave's start until its weight
-    // requests were out; 4096 x 14336: 10.6 us against 10.9 us with the rows requested first).
-    v4i wpre[GEMV_UNROLL];
-    using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
-    typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
-    if constexpr (QT != 0) {
-        const int tiles = Kp >> 5;
-#pragma unroll
-        for (int u = 0; u < GEMV_UNROLL; ++u) {
-            const int tt = wave + u * GEMV_WAVES;
-            wpre[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                       wbase + (size_t)tt * 1024 + lane * 16))
-                                 : v4i{0, 0, 0, 0};
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = (int)threadIdx.x + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                const QT_T* row = static_cast<const QT_T*>(q.src) + (size_t)m * K;
-                araw[i] = RowLoader<QT_T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        RK_TS(4);
-    }
-    if constexpr (QT != 0) {
-        using T = QT_T;
-        const int t = threadIdx.x;
-        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
-        if (t < MR) row_max[t] = 0u;
-        __syncthreads();
-        RK_TS(5);
-        // (the rows stay in registers as fetched and are converted once per pass:
-        // holding them as floats across the barriers costs the int4 variants their
-        // second workgroup per compute unit)
-        bool bad = false;
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                float mx = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    mx = fmaxf(mx, fabsf(v[j]));
-                    bad |= not_finite(v[j]);
-                }
-                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
-            }
-        }
-        __syncthreads();
-        if (t < g.M) {
-            const float mx = __uint_as_float(row_max[t]);
-            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
-                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
-            row_scale[t] = sc;
-            if (p == 0 && q.scale) q.scale[t] = sc;
-        }
-        if (p == 0 && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
-        // zero the K padding of the staged rows
-        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) {
-            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
-            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = packed;
-                if (p == 0 && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
-            }
-        }
-        // a_scale of the epilogue comes from LDS in this path
-        RK_TS(1);
-    }
-
-    for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
-        const int kc = min(kc_max, Kp - kc0);
-        // stage activations: row-major [MR][kc] in LDS from the tiled buffer
-        const int chunks = kc >> 4;
-        if (kc0) __syncthreads();
-        if constexpr (QT == 0) {
-            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
-                const int m = idx / chunks, c = idx - m * chunks;
-                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
-            }
-        }
-        __syncthreads();
-
-        // One group = GEMV_UNROLL tiles per wave.
-        const int tiles = kc >> 5, tile0 = kc0 >> 5;
-        auto fetch = [&](v4i* w, int tb) {
-#pragma unroll
-            for (int u = 0; u < GEMV_UNROLL; ++u) {
-                const int tt = tb + u * GEMV_WAVES;
-                w[u] = tt < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
-                                        wbase + (size_t)(tile0 + tt) * 1024 + lane * 16))
-                                  : v4i{0, 0, 0, 0};
-            }
-        };
-        auto consume = [&](const v4i* w, int tb) {
-#pragma unroll
-            for (int u = 0; u < GEMV_UNROLL; ++u) {
-                const int tt = tb + u * GEMV_WAVES;
-                if (tt >= tiles) continue;
-#pragma unroll
-                for (int m = 0; m < MR; ++m) {
-                    const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
-                    acc[m] = __builtin_amdgcn_sdot4(av.x, w[u].x, acc[m], false);
-                    acc[m] = __builtin_amdgcn_sdot4(av.y, w[u].y, acc[m], false);
-                    acc[m] = __builtin_amdgcn_sdot4(av.z, w[u].z, acc[m], false);
-                    acc[m] = __builtin_amdgcn_sdot4(av.w, w[u].w, acc[m], false);
-                }
-            }
-        };
-        int tb = wave;
-        if constexpr (QT != 0) { // the group fetched ahead of the prologue (the fused path has a single K chunk)
-            consume(wpre, tb);
-            tb += GEMV_WAVES * GEMV_UNROLL;
-        }
-        for (; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
-            v4i w[GEMV_UNROLL];
-            fetch(w, tb);
-            consume(w, tb);
-        }
-    }
-
-    RK_TS(2);
-#pragma unroll
-    for (int m = 0; m < MR; ++m) {
-        int v = acc[m];
-        v += __shfl_xor(v, 32);
-        if (lane < 32) red[wave][m][lane] = v;
-    }
-    __syncthreads();
-    static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
-    if ((int)threadIdx.x < MR * 32) {
-        const int m = (int)threadIdx.x >> 5, j = (int)threadIdx.x & 31;
-        if (m >= g.M) return;
-        RK_TS(3);
-        int sum = 0;
-#pragma unroll
-        for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
-        const int n = block_first_col(p, g.interleave_F) + j;
-        if (n < g.N)
-            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
-                      QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
-                      g.w_scale ? g.w_scale[n] : 1.0f);
-    }
-}
-
 
 
 // ---- gate/up GEMV with the SwiGLU epilogue (one or two rows, quantized rows in g.A) ----
@@ -2821,11 +2646,11 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
-    if (MR == 1 && !g.w_int4 && cw == 32) { // (see gemv_wide8_kernel)
-        mark(st, qt ? "gemv_wide8_kernel (fused quantize)" : "gemv_wide8_kernel");
-        if (qt == 0) hipLaunchKernelGGL((gemv_wide8_kernel<0>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
-        else if (qt == 1) hipLaunchKernelGGL((gemv_wide8_kernel<1>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
-        else hipLaunchKernelGGL((gemv_wide8_kernel<2>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+    if (MR == 1 && !g.w_int4 && cw == 32) { // (the burst variant, see gemv_kernel)
+        mark(st, qt ? "gemv_kernel<burst> (fused quantize)" : "gemv_kernel<burst>");
+        if (qt == 0) hipLaunchKernelGGL((gemv_kernel<1, false, 0, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else if (qt == 1) hipLaunchKernelGGL((gemv_kernel<1, false, 1, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else hipLaunchKernelGGL((gemv_kernel<1, false, 2, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
