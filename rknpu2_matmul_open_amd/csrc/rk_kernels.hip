@@ -839,6 +839,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
         if (t < MR) row_max[t] = 0u;
         __syncthreads();
+        RK_TS(5);
         // (the rows stay in registers as fetched and are converted once per pass:
         // holding them as floats across the barriers costs the int4 variants their
         // second workgroup per compute unit)
@@ -887,6 +888,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
         }
         // a_scale of the epilogue comes from LDS in this path
+        RK_TS(1);
     }
 
     for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
@@ -1013,6 +1015,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         }
     }
 
+    RK_TS(2);
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         int v = W4 ? 16 * acc[m] + acc_lo[m] : acc[m];
@@ -1026,6 +1029,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     if ((int)threadIdx.x < MR * CW) {
         const int m = (int)threadIdx.x / CW, j = (int)threadIdx.x % CW;
         if (m >= g.M) return;
+        RK_TS(3);
         int sum = 0;
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
