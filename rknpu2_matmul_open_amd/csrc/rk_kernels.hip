@@ -1865,18 +1865,16 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
+                    // int4 weights ride as 16 * code: a part's sum is an exact multiple of 16 that fits
+                    // int32 (a part spans at most 2^17 k), but the sum of the parts times 16 need not --
+                    // so the factor comes off each part before it is added
+                    constexpr int SH = W4 ? 4 : 0;
                     const v4i got = *reinterpret_cast<const v4i*>(src + j * 1024 + (q * 64 + lane) * 4);
-                    sum[j][q * 4] += got.x;
-                    sum[j][q * 4 + 1] += got.y;
-                    sum[j][q * 4 + 2] += got.z;
-                    sum[j][q * 4 + 3] += got.w;
+                    sum[j][q * 4] += got.x >> SH;
+                    sum[j][q * 4 + 1] += got.y >> SH;
+                    sum[j][q * 4 + 2] += got.z >> SH;
+                    sum[j][q * 4 + 3] += got.w >> SH;
                 }
-        }
-        if constexpr (W4) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sum[j][r] >>= 4;
         }
         const int m0 = mblk * BM + (keep0 + ii) * 32;
         if constexpr (EPI == RKH_EPI_SWIGLU) {

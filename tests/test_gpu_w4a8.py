@@ -70,6 +70,36 @@ def test_w4a8_f32_and_f16_bit_exact(sess, oracle, M, N, K):
         w.close()
 
 
+@pytest.mark.parametrize("M", [1, 2, 9, 200])
+def test_w4a8_k_beyond_one_part_of_the_times16_range(sess, oracle, M):
+    """K > 2^17: the MFMA kernels carry int4 codes as 16 * code, so one K part may not span more
+    than 2^17 k before an extreme int32 sum could wrap; longer K is split into parts (M > 8), and
+    the decode kernels (M <= 8) multiply the nibbles as they are.  Extreme codes and activations
+    make every wrong split show: |sum| = 127 * 8 * K = 1.35e8, times 16 = 2.16e9 > 2^31."""
+    N, K = 96, 131072 + 2048 + 64
+    rng = np.random.default_rng(M + 4242)
+    B = np.full((K, N), -8, np.int8)
+    B[:, 1::2] = 7
+    B[:, 2::5] = _codes(rng, (K, len(range(2, N, 5))))
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.001
+    A = (rng.standard_normal((M, K)) * 2).astype(np.float32)
+    A[0] = 127.0                                        # q = 127 everywhere
+    if M > 1:
+        A[M - 1] = -127.0
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        want = oracle.w4a8(A, B, ws)
+        assert int(np.abs(want["acc"].astype(np.int64)).max()) * 16 > 2**31   # the case is what it claims
+        rc, acc = wsp.run_i32(w, A)
+        assert rc == 0 and np.array_equal(acc, want["acc"])
+        rc, got = wsp.run_f32(w, A)
+        assert rc == 0 and np.array_equal(_bits32(got), _bits32(want["C"]))
+    finally:
+        wsp.close()
+        w.close()
+
+
 def test_w4a8_extremes_and_tiny_scale(sess, oracle):
     M, N, K = 4, 64, 2048
     B = np.full((K, N), -8, np.int8)
