@@ -148,7 +148,11 @@ def test_single_expert_no_shared_and_empty_routes(sess, oracle):
 
 @pytest.mark.parametrize("T,H,E,top_k,I,shared", [(7, 64, 4, 2, 32, 0), (33, 128, 8, 3, 96, 1),
                                                    (100, 96, 40, 8, 64, 0), (256, 256, 16, 4, 160, 1),
-                                                   (19, 160, 5, 1, 544, 0)])
+                                                   (19, 160, 5, 1, 544, 0),
+                                                   # the envelope: every assignment slot in use (256 x 8 =
+                                                   # 2048) over a thousand experts + the shared one (most
+                                                   # buckets hold one or two rows); the widest middle
+                                                   (256, 64, 1000, 8, 32, 1), (5, 64, 2, 1, 8192, 0)])
 def test_random_moe_bit_exact(sess, oracle, T, H, E, top_k, I, shared):
     c = workloads.moe_case(T, H, E, top_k, I, seeds=(T, H, E, top_k, I))
     experts = c["experts"]
@@ -162,6 +166,56 @@ def test_random_moe_bit_exact(sess, oracle, T, H, E, top_k, I, shared):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
         assert sess.lib.rk_npu_moe_w8_weights_device_bytes(moe.w) >= (E + shared) * 3 * H * I
         assert sess.lib.rk_npu_moe_w8_workspace_device_bytes(moe.ws) > 0
+    finally:
+        moe.close()
+
+
+def test_moe_extreme_codes_and_magnitudes(sess, oracle):
+    """All-extreme operands: every expert code +-127, tokens at +-3e38 / denormal / all-equal
+    magnitudes, so that the int32 sums (127 * 127 * K), the scales at both ends of the fp32 range
+    and the saturating SiLU branch (|gate| far beyond 80) are exercised together."""
+    T, H, E, top_k, I = 12, 256, 3, 2, 96
+    rng = np.random.default_rng(99)
+    experts = []
+    for e in range(E):
+        g = np.where(rng.random((H, 2 * I)) < 0.5, -127, 127).astype(np.int8)
+        d = np.where(rng.random((I, H)) < 0.5, -127, 127).astype(np.int8)
+        if e == 0:
+            g[:] = 127
+            d[:] = -127
+        gs = (rng.random(2 * I).astype(np.float32) + 0.5) * np.float32([1e-3, 1.0, 30.0][e])
+        ds = (rng.random(H).astype(np.float32) + 0.5) * np.float32([1e-3, 1.0, 1e-6][e])
+        experts.append((g, gs, d, ds))
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    x[0] = 3.0e38
+    x[1] = -3.0e38
+    x[2] = np.where(rng.random(H) < 0.5, -1.0, 1.0)           # every |q| = 127
+    x[3] = 1e-30
+    x[4] = 0.0
+    x[5, :] = 0.0
+    x[5, 7] = -2.5e-36                                         # a scale close to the smallest accepted
+    ids = np.stack([rng.permutation(E)[:top_k] for _ in range(T)]).astype(np.int32)
+    routes = (rng.random((T, top_k), dtype=np.float32) + np.float32(0.1))
+    routes[2, 0] = 0.0                                         # a dropped route
+    moe = ops.MoeW8(sess, H, I, E, 0, top_k, 32, experts)
+    try:
+        rc, got = moe.run_f32(x, ids, routes)
+        rc2, want = oracle.moe_w8(experts, H, I, E, 0, top_k, ids, routes, input_f32=x)
+        assert rc == rc2
+        if rc == 0:
+            # A middle that overflows has no defined result in the reference (its scalar path casts
+            # NaN to int, its NEON path saturates): such rows only have to be non-finite on both
+            # sides, and must not disturb the other tokens of the batch.
+            finite = np.isfinite(want).all(axis=1)
+            assert not finite[0] and not finite[1] and finite[2:].all()
+            assert not np.isfinite(got[~finite]).all(axis=1).any()
+            assert np.array_equal(got[finite].view(np.uint32), want[finite].view(np.uint32))
+        # the same call without the overflowing tokens
+        keep = [2, 3, 4, 5, 6, 7, 8, 9, 10, 11]
+        rc, got = moe.run_f32(x[keep], ids[keep], routes[keep])
+        rc2, want = oracle.moe_w8(experts, H, I, E, 0, top_k, ids[keep], routes[keep], input_f32=x[keep])
+        assert rc == 0 and rc2 == 0
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     finally:
         moe.close()
 
