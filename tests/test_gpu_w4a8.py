@@ -36,7 +36,9 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           (650, 6900, 1000), (641, 6912, 200),
           # decode GEMV variants: 16 columns per workgroup (one row: rolling load window; several rows),
           # 32 columns per workgroup on a wide matrix, K staged in several chunks
-          (1, 4096, 4096), (3, 2500, 1000), (1, 9000, 520), (8, 8200, 5000)]
+          (1, 4096, 4096), (3, 2500, 1000), (1, 9000, 520), (8, 8200, 5000),
+          # degenerate and lopsided: single k / column, far more rows than columns, very wide matrices
+          (1, 1, 1), (2500, 3, 2), (1, 70001, 64), (9, 70001, 40), (300, 30000, 70)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

@@ -21,6 +21,9 @@ def _rand_i8(rng, shape, lo=-127, hi=127):
 I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96), (17, 40, 33),
               (33, 130, 70), (64, 256, 256), (65, 257, 129), (128, 512, 384), (300, 48, 33),
               (200, 1000, 520),
+              # degenerate and lopsided: single k / column / row, far more rows than anything else,
+              # a very wide matrix for one row, for a row block and for many rows
+              (1, 1, 1), (5000, 3, 1), (2, 1, 5000), (4100, 40, 70), (1, 70001, 64), (9, 70001, 40), (300, 40000, 33),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
               (100, 8448, 160), (128, 96, 3000),
               # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
@@ -67,6 +70,7 @@ def test_i8i8i32_extremes_wrap(sess, oracle):
 F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64, 128),
               (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024),
               (650, 7000, 1100),  # large-tile kernel
+              (1, 1, 1), (3000, 2, 3), (1, 70001, 48), (2100, 4100, 130),  # degenerate / lopsided
               # decode GEMV variants: 16 columns per workgroup with the rolling load window (one row),
               # with several rows, with K staged in several chunks; wide matrices with one / several rows
               (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300)]
