@@ -319,6 +319,33 @@ def test_int4_experts_equal_the_int8_path(sess, oracle, flavour, shared):
         moe.close()
 
 
+@pytest.mark.parametrize("flavour", ["quant", "w4"])
+def test_int4_experts_at_prefill_size_take_the_balanced_launch(sess, oracle, flavour):
+    """256 tokens, top-4 of 16 experts + the shared one, hidden 1024, intermediate 1024: the grouped
+    gate/up GEMM has about 50 row blocks x 32 column pairs, enough units for the balanced launch
+    (one workgroup per compute unit), here over packed int4 images; with "w4" the shared expert is
+    int8, so the bank holds both formats and every grouped GEMM is one launch per format."""
+    T, H, E, top_k, I = 256, 1024, 16, 4, 1024
+    rng = np.random.default_rng(2024)
+    experts = []
+    for e in range(E + 1):
+        lo, hi = (-8, 7) if (flavour == "quant" or e < E) else (-127, 127)
+        experts.append((rng.integers(lo, hi + 1, (H, 2 * I)).astype(np.int8),
+                        (rng.random(2 * I).astype(np.float32) + 0.5) * np.float32(0.02),
+                        rng.integers(lo, hi + 1, (I, H)).astype(np.int8),
+                        (rng.random(H).astype(np.float32) + 0.5) * np.float32(0.02)))
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    ids, routes = _routes(rng, T, E, top_k)
+    moe = ops.MoeW8(sess, H, I, E, 1, top_k, 256, experts, flavour=flavour)
+    try:
+        rc, got = moe.run_f32(x, ids, routes)
+        rc2, want = oracle.moe_w8(experts, H, I, E, 1, top_k, ids, routes, input_f32=x)
+        assert rc == 0 and rc2 == 0
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    finally:
+        moe.close()
+
+
 def test_int4_factories_validate_codes_geometry_and_layout(sess):
     lib = sess.lib
     H, I, E = 128, 64, 3
