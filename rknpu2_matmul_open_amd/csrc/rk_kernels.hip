@@ -2531,9 +2531,11 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     // lasted as long as the compute units with two (down projection: last workgroup done after
     // 17.8 us, 15.4 balanced).  RK_NPU_HIP_GROUPED=balanced|tiles forces the choice (tuning aid).
     const int cus = compute_units();
-    bool balanced = grouped && cus > 0 && (long)mblocks * ((g.N + 63) / 64) >= GROUPED_BALANCED_UNITS_PER_CU * (long)cus;
+    const bool moe_epilogue = g.epilogue == RKH_EPI_F32 || g.epilogue == RKH_EPI_SWIGLU;
+    bool balanced = grouped && moe_epilogue && cus > 0 &&
+                    (long)mblocks * ((g.N + 63) / 64) >= GROUPED_BALANCED_UNITS_PER_CU * (long)cus;
     static const char* forced = getenv("RK_NPU_HIP_GROUPED");
-    if (forced && forced[0] == 'b') balanced = grouped && cus > 0;
+    if (forced && forced[0] == 'b') balanced = grouped && moe_epilogue && cus > 0;
     if (forced && forced[0] == 't') balanced = false;
     if (balanced) {
         mark(st, "gemm_stream_kernel<balanced>");
@@ -2543,9 +2545,7 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
         if (any_int4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, true, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);  \
         if (any_int8) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 1, false, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); \
     } while (0)
-        switch (g.epilogue) {
-        case RKH_EPI_I32: RK_LAUNCH_BAL(RKH_EPI_I32); break;
-        case RKH_EPI_F16: RK_LAUNCH_BAL(RKH_EPI_F16); break;
+        switch (g.epilogue) { // (grouped GEMMs are the MoE layer's: gate/up + SwiGLU and the fp32 down projection)
         case RKH_EPI_F32: RK_LAUNCH_BAL(RKH_EPI_F32); break;
         case RKH_EPI_SWIGLU: RK_LAUNCH_BAL(RKH_EPI_SWIGLU); break;
         default: return RKH_ERR_RUNTIME;
@@ -2617,16 +2617,14 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
                                dim3(mblocks * nblocks * (TM == 1 ? 4 : 8)), dim3(64), 0, st, g,     \
                                mblocks, nblocks, ksplit);                                           \
     } while (0)
-#define RK_WK_EPI(W4)                                           \
-    switch (g.epilogue) {                                       \
-    case RKH_EPI_I32: RK_WK(W4, RKH_EPI_I32); break;            \
-    case RKH_EPI_F16: RK_WK(W4, RKH_EPI_F16); break;            \
-    case RKH_EPI_F32: RK_WK(W4, RKH_EPI_F32); break;            \
-    case RKH_EPI_SWIGLU: RK_WK(W4, RKH_EPI_SWIGLU); break;      \
-    default: return RKH_ERR_RUNTIME;                            \
+    // (a dense SwiGLU GEMM exists for int4 weights only: the w4a8 FFN; the MoE layer's is grouped)
+    switch (g.epilogue) {
+    case RKH_EPI_I32: if (g.w_int4) RK_WK(true, RKH_EPI_I32); else RK_WK(false, RKH_EPI_I32); break;
+    case RKH_EPI_F16: if (g.w_int4) RK_WK(true, RKH_EPI_F16); else RK_WK(false, RKH_EPI_F16); break;
+    case RKH_EPI_F32: if (g.w_int4) RK_WK(true, RKH_EPI_F32); else RK_WK(false, RKH_EPI_F32); break;
+    case RKH_EPI_SWIGLU: if (g.w_int4) RK_WK(true, RKH_EPI_SWIGLU); else return RKH_ERR_RUNTIME; break;
+    default: return RKH_ERR_RUNTIME;
     }
-    if (g.w_int4) { RK_WK_EPI(true) } else { RK_WK_EPI(false) }
-#undef RK_WK_EPI
 #undef RK_WK
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
@@ -2661,7 +2659,8 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     do {                                                                                       \
         if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
         else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q); \
-        else hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
+        else if constexpr (!(MR == 1 && !W4)) /* (one int8 row, 32 columns: the burst variant above) */   \
+            hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
     } while (0)
     if (g.w_int4) {
         if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
@@ -2680,11 +2679,10 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
     mark(st, qt ? "gemv_swiglu_kernel (fused quantize)" : "gemv_swiglu_kernel");
 #define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q)
-    if (g.w_int4) {
-        if (qt == 0) RK_SWI(true, 0); else if (qt == 1) RK_SWI(true, 1); else RK_SWI(true, 2);
-    } else {
-        if (qt == 0) RK_SWI(false, 0); else if (qt == 1) RK_SWI(false, 1); else RK_SWI(false, 2);
-    }
+    // (dense SwiGLU exists for int4 weights only, with rows as fp32 or already quantized:
+    // the w4a8 interface has no other call, and gemv_swiglu_applies lets nothing else through)
+    if (!g.w_int4 || qt == 1) return RKH_ERR_RUNTIME;
+    if (qt == 0) RK_SWI(true, 0); else RK_SWI(true, 2);
 #undef RK_SWI
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
@@ -2695,7 +2693,7 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
 // Measured for 4096 -> 2 x 14336 int4 against 14.9 us on the MFMA kernel: 12.8 us for one row,
 // 13.8 for two, 15.1 for four, 20.1 for eight -- so from three rows on the MFMA kernel keeps it.
 bool gemv_swiglu_applies(const rkh_gemm_args& g) {
-    return !g.blk_expert && g.M <= 2 && g.epilogue == RKH_EPI_SWIGLU && g.interleave_F >= 32 &&
+    return !g.blk_expert && g.w_int4 && g.M <= 2 && g.epilogue == RKH_EPI_SWIGLU && g.interleave_F >= 32 &&
            g.interleave_F % 32 == 0 && g.N == 2 * g.interleave_F && g.K <= (1 << 24);
 }
 

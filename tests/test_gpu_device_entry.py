@@ -37,7 +37,8 @@ def _special_rows(A, as_f16):
 W8_SHAPES = [(1, 64, 64), (1, 200, 200), (1, 513, 1000), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520),
              (1, 14336, 4096), (1, 9000, 4100), (2, 14336, 4096),
              (2, 3000, 700), (3, 65, 33), (4, 9000, 300), (4, 4100, 8000), (8, 128, 4096), (8, 8300, 2000),
-             (7, 5000, 4100), (2, 2500, 20003), (16, 300, 500)]
+             (7, 5000, 4100), (2, 2500, 20003), (16, 300, 500),
+             (2, 1000, 300), (7, 4100, 300)]   # two rows, 8 columns per workgroup; five to eight rows, 16 columns
 
 
 @pytest.mark.parametrize("M,N,K", W8_SHAPES)
@@ -74,7 +75,9 @@ def test_w8a8_dynamic_device(sess, oracle, M, N, K, f16):
 
 W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520), (2, 65, 20003),
              (1, 14336, 4096), (1, 9000, 4100),
-             (3, 2500, 1000), (4, 9000, 300), (8, 128, 512), (8, 8200, 2000), (5, 4100, 5000), (12, 200, 300)]
+             (3, 2500, 1000), (4, 9000, 300), (8, 128, 512), (8, 8200, 2000), (5, 4100, 5000), (12, 200, 300),
+             # two rows at every column width of the kernel; four rows, 8 columns; six rows, 16 columns
+             (2, 4096, 512), (2, 9000, 300), (2, 1000, 200), (4, 1000, 300), (6, 4100, 300)]
 
 
 @pytest.mark.parametrize("M,N,K", W4_SHAPES)

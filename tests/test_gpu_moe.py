@@ -321,11 +321,12 @@ def test_int4_experts_equal_the_int8_path(sess, oracle, flavour, shared):
 
 @pytest.mark.parametrize("flavour", ["quant", "w4"])
 def test_int4_experts_at_prefill_size_take_the_balanced_launch(sess, oracle, flavour):
-    """256 tokens, top-4 of 16 experts + the shared one, hidden 1024, intermediate 1024: the grouped
-    gate/up GEMM has about 50 row blocks x 32 column pairs, enough units for the balanced launch
-    (one workgroup per compute unit), here over packed int4 images; with "w4" the shared expert is
-    int8, so the bank holds both formats and every grouped GEMM is one launch per format."""
-    T, H, E, top_k, I = 256, 1024, 16, 4, 1024
+    """256 tokens, top-8 of 16 experts + the shared one, hidden 1024, intermediate 1024: the grouped
+    GEMMs have about 75 row blocks x 32 (gate/up) and x 16 (down) column pairs, enough units for the
+    balanced launch (one workgroup per compute unit) of both, here over packed int4 images; with "w4"
+    the shared expert is int8, so the bank holds both formats and every grouped GEMM is one launch
+    per format."""
+    T, H, E, top_k, I = 256, 1024, 16, 8, 1024
     rng = np.random.default_rng(2024)
     experts = []
     for e in range(E + 1):

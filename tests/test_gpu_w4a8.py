@@ -38,7 +38,10 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           # 32 columns per workgroup on a wide matrix, K staged in several chunks
           (1, 4096, 4096), (3, 2500, 1000), (1, 9000, 520), (8, 8200, 5000),
           # degenerate and lopsided: single k / column, far more rows than columns, very wide matrices
-          (1, 1, 1), (2500, 3, 2), (1, 70001, 64), (9, 70001, 40), (300, 30000, 70)]
+          (1, 1, 1), (2500, 3, 2), (1, 70001, 64), (9, 70001, 40), (300, 30000, 70),
+          # 64-row tiles of the large-tile kernel; K split over workgroups + reduce launch; two / three rows
+          # on a wide matrix
+          (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -187,7 +190,8 @@ SWIGLU_SHAPES = [(1, 64, 64), (1, 4160, 1000), (2, 192, 20003),  # one / two row
                  (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
                  (128, 1024, 512),
                  (20, 32896, 128), (32, 2048, 700),  # weight-streaming kernel: wide grid / K split inside the workgroup
-                 (650, 6912, 520), (641, 7040, 300)]  # large-tile kernel (F a multiple of 64 / only of 32)
+                 (650, 6912, 520), (641, 7040, 300),  # large-tile kernel (F a multiple of 64 / only of 32)
+                 (40, 128, 4100)]  # two 32-row tiles: K split over workgroups, SwiGLU in the reduce launch
 
 
 @pytest.mark.parametrize("M,N,K", SWIGLU_SHAPES)

@@ -24,6 +24,8 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               # degenerate and lopsided: single k / column / row, far more rows than anything else,
               # a very wide matrix for one row, for a row block and for many rows
               (1, 1, 1), (5000, 3, 1), (2, 1, 5000), (4100, 40, 70), (1, 70001, 64), (9, 70001, 40), (300, 40000, 33),
+              # 64-row tiles of the large-tile kernel (too few 128-row tiles); K split over workgroups + reduce launch
+              (300, 8448, 200), (130, 96, 4100),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
               (100, 8448, 160), (128, 96, 3000),
               # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
@@ -73,7 +75,11 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               (1, 1, 1), (3000, 2, 3), (1, 70001, 48), (2100, 4100, 130),  # degenerate / lopsided
               # decode GEMV variants: 16 columns per workgroup with the rolling load window (one row),
               # with several rows, with K staged in several chunks; wide matrices with one / several rows
-              (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300)]
+              (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300),
+              (2, 9000, 300), (4, 4100, 300),   # two rows on a wide matrix; four rows, 16 columns per workgroup
+              # weight-streaming kernel on a wide grid; 64-row tiles of the large-tile kernel;
+              # eight rows per quantization workgroup (M >= 4096)
+              (100, 8448, 160), (300, 8448, 200), (4200, 64, 100)]
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
@@ -97,7 +103,10 @@ def test_f16i8f16_dynamic_bit_exact(sess, oracle, M, N, K):
         op.close()
 
 
-@pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203)])  # second: many-row quantization path
+# second: many-row quantization path; then 128- and 64-row tiles of the large-tile kernel, K split over
+# workgroups + reduce launch, eight rows per quantization workgroup
+@pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203), (650, 7000, 300), (300, 8448, 200), (261, 96, 3000),
+                                   (4200, 64, 100)])
 def test_f32i8f32_dynamic_and_static(sess, oracle, M, N, K):
     rng = np.random.default_rng(5)
     A = rng.standard_normal((M, K)).astype(np.float32) * 3
