@@ -106,7 +106,9 @@ def test_f16i8f16_dynamic_bit_exact(sess, oracle, M, N, K):
 # second: many-row quantization path; then 128- and 64-row tiles of the large-tile kernel, K split over
 # workgroups + reduce launch, eight rows per quantization workgroup
 @pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203), (650, 7000, 300), (300, 8448, 200), (261, 96, 3000),
-                                   (4200, 64, 100)])
+                                   (4200, 64, 100),
+                                   # an input / an output of more than 64 MiB: beyond the pinned staging mirrors
+                                   (4200, 64, 4100), (4200, 4100, 64)])
 def test_f32i8f32_dynamic_and_static(sess, oracle, M, N, K):
     rng = np.random.default_rng(5)
     A = rng.standard_normal((M, K)).astype(np.float32) * 3
