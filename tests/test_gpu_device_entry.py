@@ -199,3 +199,93 @@ def test_w4a8_ffn_device_nonfinite_middle_is_rejected(sess):
             sess.free_device(d)
         for o in (gws, dws, gw, dw):
             o.close()
+
+
+# ---- device pointers that are only element-aligned -------------------------------------------
+# The device entry points take any pointer into device memory.  Rows that do not start on a
+# 16-byte boundary take the element-wise loaders and outputs the element-wise stores; nothing
+# in the interface asks for more than the element's own alignment.
+
+def _offset_copy(sess, array, elems):
+    """Device copy of `array` that starts `elems` elements into an allocation -> (base, pointer)."""
+    a = np.ascontiguousarray(array)
+    base = sess.empty_device(a.nbytes + 64)
+    p = base + elems * a.itemsize
+    assert sess.lib.rk_npu_hip_upload(sess.ctx, p, capi.ptr(a), a.nbytes) == 0
+    return base, p
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 9000, 520), (1, 2100, 1000), (4, 300, 200), (40, 300, 260), (300, 520, 200)])
+@pytest.mark.parametrize("f16", [True, False])
+def test_w8a8_device_pointers_with_element_alignment_only(sess, oracle, M, N, K, f16):
+    c = workloads.w8a8_case(M, K, N, seed_w=M + N + 2, seed_a=K + 13)
+    if f16:
+        A, kind, out_dtype = c["A"], capi.F16I8F16_DYNAMIC, np.uint16
+    else:
+        A = oracle.half_to_float(c["A"]).astype(np.float32).reshape(M, K) * 2.0
+        kind, out_dtype = capi.F32I8F32_DYNAMIC, np.float32
+    size = np.dtype(out_dtype).itemsize
+    op = ops.W8A8Linear(sess, kind, M, c["B"], c["w_scale"])
+    baseA, dA = _offset_copy(sess, A, 1)
+    baseC = sess.empty_device(M * N * size + 64)
+    dC = baseC + 3 * size
+    try:
+        assert op.run_device(dA, dC) == 0
+        assert sess.sync() == 0
+        got = sess.from_device(dC, (M, N), out_dtype)
+        want = oracle.w8a8(A, c["B"], c["w_scale"])["C"]
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    finally:
+        sess.free_device(baseA)
+        sess.free_device(baseC)
+        op.close()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 9000, 520), (2, 300, 200), (40, 300, 260), (300, 520, 200)])
+def test_w4a8_device_pointers_with_element_alignment_only(sess, oracle, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    B = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 0.02
+    A = (rng.standard_normal((M, K)) * 2).astype(np.float32)
+    A16 = A.astype(np.float16).view(np.uint16)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    baseA, dA = _offset_copy(sess, A, 1)
+    baseA16, dA16 = _offset_copy(sess, A16, 3)
+    baseC, baseC16 = sess.empty_device(M * N * 4 + 64), sess.empty_device(M * N * 2 + 64)
+    dC, dC16 = baseC + 4, baseC16 + 2
+    try:
+        assert sess.lib.rk_npu_w4a8_run_f32_device(wsp.h, w.h, dA, dC) == 0
+        assert sess.lib.rk_npu_w4a8_run_f16_device(wsp.h, w.h, dA16, dC16) == 0
+        assert sess.sync() == 0
+        assert np.array_equal(_bits32(sess.from_device(dC, (M, N), np.float32)), _bits32(oracle.w4a8(A, B, ws)["C"]))
+        assert np.array_equal(sess.from_device(dC16, (M, N), np.uint16), oracle.w4a8(A16, B, ws)["C"])
+    finally:
+        for d in (baseA, baseA16, baseC, baseC16):
+            sess.free_device(d)
+        wsp.close()
+        w.close()
+
+
+@pytest.mark.parametrize("T", [3, 70])
+def test_moe_device_pointers_with_element_alignment_only(sess, oracle, T):
+    H, E, top_k, I = 128, 6, 2, 64
+    c = workloads.moe_case(T, H, E, top_k, I)
+    moe = ops.MoeW8(sess, H, I, E, 0, top_k, 128, c["experts"])
+    x = np.ascontiguousarray(c["x"], np.float32)
+    ids, routes = np.ascontiguousarray(c["ids"], np.int32), np.ascontiguousarray(c["routes"], np.float32)
+    bx, dx = _offset_copy(sess, x, 1)
+    bi, dids = _offset_copy(sess, ids, 1)
+    br, drt = _offset_copy(sess, routes, 3)
+    bo = sess.empty_device(T * H * 4 + 64)
+    dout = bo + 4
+    try:
+        assert sess.lib.rk_npu_moe_w8_run_f32_device(moe.ws, moe.w, T, dx, dids, drt, dout) == 0
+        assert sess.sync() == 0
+        rc, want = oracle.moe_w8(c["experts"], H, I, E, 0, top_k, ids, routes, input_f32=x)
+        got = sess.from_device(dout, (T, H), np.float32)
+        assert rc == 0 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    finally:
+        for d in (bx, bi, br, bo):
+            sess.free_device(d)
+        moe.close()
