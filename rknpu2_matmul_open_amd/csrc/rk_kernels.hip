@@ -1435,8 +1435,8 @@ __device__ __forceinline__ void epilogue_swiglu(const rkh_gemm_args& g, const v1
 // fragment reads and eight MFMAs.
 //
 // Activations: every wave copies its 1 KiB share of a sub-step global -> LDS
-// directly (no registers), WK_D sub-steps ahead, into a ring of WK_NBUF
-// buffers.  Weights: global -> registers, NSW-1 sub-steps ahead (8 bytes per
+// directly (no registers), D sub-steps ahead (WK_D; 8 for the 128-row tile), into
+// a ring of WK_NBUF buffers.  Weights: global -> registers, NSW-1 sub-steps ahead (8 bytes per
 // lane and k-tile pair for int4, 16 per k-tile for int8).  The fragments of
 // the NEXT sub-step are read and, for int4, its operands unpacked in the
 // shadow of this sub-step's MFMAs.
@@ -1491,12 +1491,24 @@ __device__ __forceinline__ void wk_tile_coords(int tile, int mblocks, int nblock
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm" // m0 is set and clobbered on purpose below
 template <int TM, bool W4, int EPI>
-__global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int mblocks, int nblocks, int ksplit,
-                                                      int ksteps_per_part, rkh_gemm_args g) {
-    RK_GEMM_HEAD_APPLY(g);
+__global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const uint8_t* h_W, int h_M, int h_K,
+                                                      int mblocks, int nblocks, int ksplit, int ksteps_per_part,
+                                                      rkh_gemm_args g) {
+    // (leading scalar arguments, see RK_GEMM_HEAD_PARAMS: everything the tile coordinates and the
+    // prologue's loads depend on, ten dwords, arrives in registers)
+    g.A = h_A; g.W = h_W; g.M = h_M; g.K = h_K;
+    RK_TS(0);
     constexpr int TN = 2, KTS = 8 / TM, KTW = KTS / 2; // k-tiles per sub-step: all / this wave's
-    constexpr int NSW = (TM == 4 || (TM == 2 && W4)) ? 8 : 4;
-    constexpr int NBUF = WK_NBUF, G = WK_G, D = WK_D, BM = 32 * TM, BUF = WK_BUF;
+    // Look-ahead: weights NSW - 1 sub-steps, activation copies D sub-steps.  The 128-row tile runs
+    // one tile per compute unit, all of them at once, so what the prologue requests before the first
+    // MFMA (D copies + NSW - 1 weight groups per wave, 152 KB per compute unit with 8 / 12) is
+    // issue-bound in the vector memory path: in-kernel time stamps showed 1.9 us until the requests
+    // were out and 3.1 us until the first MFMA.  4 / 8 is enough to cover the latency (a sub-step
+    // is ~570 cycles) and starts the loop sooner: 2048 x 4096 x 4096, same box, int8 weights
+    // 30.8 -> 30.25 us, int4 32.55 -> 32.15 us.  (The 64-row int4 tile measured the same with
+    // either depth and keeps the deeper one.)
+    constexpr int NSW = TM == 4 ? 4 : (TM == 2 && W4) ? 8 : 4;
+    constexpr int NBUF = WK_NBUF, G = WK_G, D = TM == 4 ? 8 : WK_D, BM = 32 * TM, BUF = WK_BUF;
     constexpr int UNR = 16;            // sub-steps per unrolled trip: multiple of NSW, NBUF, G and 2
     // int4 weights come in 1 KiB super-tiles of two k-tiles (16 bytes per lane).  When a
     // wave has two or more k-tiles per sub-step it takes WHOLE super-tiles (k-tiles
@@ -1674,6 +1686,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int m
         copy_a(t + D);
         if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
     }
+    RK_TS(1);
     // The tile's scales are fetched now, behind the prologue's loads, and handed
     // to the epilogue through LDS after the loop, so the epilogue does not start
     // with a round trip to memory: thread t holds the row scale of row t
@@ -1708,6 +1721,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int m
     static_for<4>([&](auto f_tag) { read_frag(afr[0][decltype(f_tag)::value], std::integral_constant<int, 0>{}, f_tag); });
     static_for<NWREG>([&](auto e_tag) { unpack_item(wop[0], wring[0], e_tag); });
     frags_wait(afr[0]);
+    RK_TS(2);
 
     int s = 0;
     for (; s + UNR <= ksteps; s += UNR) static_for<UNR>([&](auto slot) { k_step(slot); });
@@ -1716,6 +1730,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int m
             if (s + decltype(slot)::value < ksteps) k_step(slot);
         });
     __builtin_amdgcn_s_setprio(0);
+    RK_TS(3);
 
     // ---- epilogue.  Drain the look-ahead copies (they write LDS) and the scale
     // loads; then every wave is past its last fragment read and LDS is reused.
@@ -1772,6 +1787,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int m
             }
         }
         lds_barrier();
+        RK_TS(4);
 
         if (ksplit > 1) {
             // partial tile in accumulator order: [tile][part][owning wave][kept tile][q][lane] x 4 ints
@@ -1830,6 +1846,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(RK_GEMM_HEAD_PARAMS, int m
     };
     if (wk == 0) finish(std::integral_constant<int, 0>{});
     else finish(std::integral_constant<int, 1>{});
+    RK_TS(5);
 }
 #pragma clang diagnostic pop
 
@@ -2610,7 +2627,7 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
             opted_in[dev] = true;                                                                   \
         }                                                                                           \
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st,           \
-                           RK_GEMM_HEAD(g), mblocks, nblocks, ksplit, per, g);                      \
+                           g.A, g.W, g.M, g.K, mblocks, nblocks, ksplit, per, g);                   \
         if (ksplit > 1) mark(st, "gemm_wk_reduce_kernel");                                          \
         if (ksplit > 1)                                                                             \
             hipLaunchKernelGGL((gemm_wk_reduce_kernel<TM, W4, EPI>),                                \
