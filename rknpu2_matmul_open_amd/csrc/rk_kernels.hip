@@ -1937,7 +1937,13 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     constexpr bool KSPLIT = KS > 1;
     static_assert(!BAL || !KSPLIT, "the balanced variant does not split K");
     constexpr int CG = WAVES / KS; // column pairs per workgroup
-    constexpr int RING = 8; // (16 with K split four ways, a wave's whole share in flight, was measured slower)
+    // Steps of a wave in flight.  Shallow is faster here: every compute unit holds eight (four)
+    // waves that stream, and what a deeper ring adds is queueing in front of the memory system,
+    // not throughput.  Measured on one box, the MoE layer of 256 tokens (balanced launch):
+    // 74.7 us with 8 steps, 74.4 with 4, 70.5 with 2; the same layer with a workgroup per tile:
+    // 77.6 / 76.9 / 74.8; a dense 128-row int4 FFN and a 64-row int8 GEMM (K split over the
+    // waves): 51.8 / 51.1 / 53.8 and 9.15 / 8.8 / 9.6 us.  (12 and 16 steps were slower still.)
+    constexpr int RING = KSPLIT ? 4 : 2;
     constexpr int AT = W4 ? 2 : 1;   // activation tiles per step
     constexpr int LPS = AT + TN;
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
@@ -1947,7 +1953,7 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(wave_id());
-    // steps over K: k-tiles (a multiple of 8 = RING) or, for int4 weights, super-tiles (a multiple of 4)
+    // steps over K: k-tiles (a multiple of 8) or, for int4 weights, super-tiles (a multiple of 4): RING divides both
     const int KB = (int)rkh_align_up(g.K, RKH_K_ALIGN) / (32 * AT);
 
     [[maybe_unused]] constexpr int TSB = EPI == RKH_EPI_SWIGLU ? 4 : 0; // (debug stamps: the SwiGLU launch keeps its own slots)
