@@ -752,13 +752,21 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     RK_GEMV_HEAD_APPLY(g, q);
     RK_TS(0);
     static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
+    // Load instructions of a wave in flight.  One row, exact waits: four -- the quantization
+    // prologue and the first dot products start after half as many bytes, and nothing is gained
+    // by queueing more in front of the memory system (4096 x 14336 int4: 7.25 -> 6.8 us; int4
+    // 4096 x 4096 4.9 -> 4.1, 4096 x 11008 7.0 -> 6.6, 8192 x 1024 5.1 -> 4.5; int8 2048 x 2048
+    // 4.2 -> 3.6, 14336 x 4096 12.8 -> 12.5, the other int8 shapes within 1 %).  Several rows
+    // and the burst variant are faster with eight (two rows lose 2 - 9 % with four on most
+    // shapes; the burst variant 10.6 -> 11.4 us).
+    constexpr int UNR = (MR == 1 && !BURST) ? 4 : GEMV_UNROLL;
     static_assert(!BURST || (MR == 1 && !W4 && CW == 32), "the burst variant serves one int8 row, whole column blocks");
     constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
-    // (padding for the single-row variants of narrow matrices: their look-ahead of GEMV_UNROLL loads per wave, and
+    // (padding for the single-row variants of narrow matrices: their look-ahead of UNR loads per wave, and
     // one more step for the activations, runs up to that many load instructions past the end
     // of a chunk, 32 / CW tiles of 32 -- int4: 64 -- staged bytes each)
     constexpr bool ROLLING = MR == 1 && CW < 32; // see the K loop
-    constexpr int A_PAD = ROLLING ? GEMV_WAVES * (GEMV_UNROLL + 1) * TPL * (W4 ? 64 : 32) : 0;
+    constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
     __shared__ int red[GEMV_WAVES][MR][CW];
     __shared__ uint32_t row_max[MR];
@@ -805,14 +813,14 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // prologue (and with it the second batch of weight loads) would start only
     // then.  Fetched first they are back after one L2 round trip and the whole
     // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
-    v4i wpre[GEMV_UNROLL];
+    v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
     typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
     if constexpr (QT != 0) {
         const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
         if constexpr (BURST) {
 #pragma unroll
-            for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
@@ -828,7 +836,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!BURST) {
 #pragma unroll
-            for (int u = 0; u < GEMV_UNROLL; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         RK_TS(4);
@@ -905,7 +913,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         }
         __syncthreads();
 
-        // One group = GEMV_UNROLL tiles per wave.  Int4: a tile is a 64-deep super-tile.
+        // One group = UNR tiles per wave.  Int4: a tile is a 64-deep super-tile.
         // (counted in load instructions: one of them spans 32 / CW tiles; K is padded to 256 and a
         // chunk but the last holds a multiple of 4096 k, so the tile count is a multiple of that)
         const int tiles = (W4 ? kc >> 6 : kc >> 5) / TPL, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
@@ -941,8 +949,8 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
         };
         if constexpr (ROLLING) {
-            // A rolling window of GEMV_UNROLL loads per wave: as soon as a tile is used, the
-            // register it sat in takes the load of the tile GEMV_UNROLL places further on, so the
+            // A rolling window of UNR loads per wave: as soon as a tile is used, the
+            // register it sat in takes the load of the tile UNR places further on, so the
             // number of loads in flight does not drain between groups (a workgroup of a narrow
             // matrix walks a long K alone on its compute unit).  The fused path starts from the
             // group fetched ahead of the prologue (it has a single K chunk).
@@ -972,19 +980,19 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                     dot_digits(t.a[1], wu.z, wu.w, acc[0], acc_lo[0]);
                 }
             };
-            v4i w[GEMV_UNROLL];
+            v4i w[UNR];
 #pragma unroll
-            for (int u = 0; u < GEMV_UNROLL; ++u) {
+            for (int u = 0; u < UNR; ++u) {
                 if constexpr (QT != 0) w[u] = wpre[u];
                 else w[u] = load_unit(wave + u * GEMV_WAVES);
             }
             ActTile cur = read_act(wave);
-            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
+            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * UNR) {
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) {
+                for (int u = 0; u < UNR; ++u) {
                     const ActTile nxt = read_act(tb + (u + 1) * GEMV_WAVES);
                     dot_tile(w[u], cur);
-                    w[u] = load_unit(tb + (GEMV_UNROLL + u) * GEMV_WAVES);
+                    w[u] = load_unit(tb + (UNR + u) * GEMV_WAVES);
                     // (each load stays behind the use of its register; gathered at the end of the
                     // iteration, as the scheduler would have them, the window drains every time)
                     __builtin_amdgcn_sched_barrier(0);
@@ -992,7 +1000,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                 }
             }
         } else {
-            // A group of GEMV_UNROLL loads at a time.  Several rows: the rolling window above costs
+            // A group of UNR loads at a time.  Several rows: the rolling window above costs
             // those variants more registers than two workgroups per compute unit leave.  Wide
             // matrices: they are bound by memory throughput, not by a workgroup's own latency, and
             // a workgroup that asks for its next 64 KiB in one go is served faster than one that
@@ -1000,16 +1008,16 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             int tb = wave;
             if constexpr (QT != 0) {
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u)
+                for (int u = 0; u < UNR; ++u)
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(wpre[u], tb + u * GEMV_WAVES);
-                tb += GEMV_WAVES * GEMV_UNROLL;
+                tb += GEMV_WAVES * UNR;
             }
-            for (; tb < tiles; tb += GEMV_WAVES * GEMV_UNROLL) {
-                v4i w[GEMV_UNROLL];
+            for (; tb < tiles; tb += GEMV_WAVES * UNR) {
+                v4i w[UNR];
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u) w[u] = load_unit(tb + u * GEMV_WAVES);
+                for (int u = 0; u < UNR; ++u) w[u] = load_unit(tb + u * GEMV_WAVES);
 #pragma unroll
-                for (int u = 0; u < GEMV_UNROLL; ++u)
+                for (int u = 0; u < UNR; ++u)
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
             }
         }
