@@ -745,7 +745,10 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 // same box, against 10.6 us: a second group of tiles requested before the prologue (11.0 us; all
 // 16 loads of a wave requested at the start: 12.2), the wave index read into a scalar register
 // (10.85: the branches around the loads become scalar and the compiler counts the loads exactly
-// again), the column scales of the epilogue fetched with the first loads (10.7).
+// again), the column scales of the epilogue fetched with the first loads (10.7), a first group
+// of 4 / 6 / 10 / 12 tiles per wave with the rest in one group behind the prologue (11.8 / 11.1 /
+// 11.0 / 11.6), four tiles per group throughout (11.4), the exact-wait kernel with four loads
+// per wave in flight (10.7).
 template <int MR, bool W4, int QT, int CW, bool BURST = false>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
