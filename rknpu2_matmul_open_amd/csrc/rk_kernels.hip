@@ -1927,7 +1927,9 @@ __global__ __launch_bounds__(64) void gemm_wk_reduce_kernel(rkh_gemm_args g, int
 // share a compute unit.  An expert with more than 32 rows has one workgroup per
 // row block and column tile; they run side by side and the second one finds
 // the weights in L2 (taking all row blocks of an expert into one workgroup was
-// measured slower: fewer workgroups than compute units remain).
+// measured slower: fewer workgroups than compute units remain; units of two row
+// blocks that request the weights once measured the same: the loop waits for the
+// first pass from HBM, not for the second one from L2).
 // KS = 4 (decode-sized calls, whose handful of row blocks would leave most
 // compute units without a workgroup): the tile shrinks to 256 / KS columns and
 // KS waves share a column pair, taking 1/KS of K each; their accumulators are
