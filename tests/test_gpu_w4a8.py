@@ -105,6 +105,51 @@ def test_w4a8_k_beyond_one_part_of_the_times16_range(sess, oracle, M):
         w.close()
 
 
+@pytest.mark.parametrize("M", [1, 9, 130])
+def test_w4a8_k_at_the_api_limit(sess, oracle, M):
+    """K = INT32_MAX / 1024, the largest the reference accepts (src/rk_npu_w4a8.cpp:47): with
+    q = 127 against a column of -8 the sum is 2.13e9, just inside int32 -- which is what the limit
+    is for -- and it must come out exactly from the decode, streaming and large-tile kernels."""
+    N, K = 40, 2147483647 // 1024
+    rng = np.random.default_rng(M + 77)
+    B = _codes(rng, (K, N))
+    B[:, 0] = -8
+    B[:, 1] = 7
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 1e-4
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    A[0] = 127.0
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        want = oracle.w4a8(A, B, ws)
+        assert int(np.abs(want["acc"].astype(np.int64)).max()) > 2 ** 31 - 2 ** 25
+        rc, acc = wsp.run_i32(w, A)
+        assert rc == 0 and np.array_equal(acc, want["acc"])
+        rc, got = wsp.run_f32(w, A)
+        assert rc == 0 and np.array_equal(_bits32(got), _bits32(want["C"]))
+    finally:
+        wsp.close()
+        w.close()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 3_000_001, 40), (9, 3_000_001, 40), (70, 1_000_003, 33), (300_001, 300, 33)])
+def test_w4a8_millions_of_columns_or_rows(sess, oracle, M, N, K):
+    """No upper limit on M and N in the API (src/rk_npu_w4a8.cpp:47 bounds K only)."""
+    rng = np.random.default_rng(M + N + 1)
+    B = _codes(rng, (K, N))
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 1e-2
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    w = ops.W4A8Weights(sess, B, ws)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    try:
+        rc, got = wsp.run_f32(w, A)
+        want = oracle.w4a8(A, B, ws)["C"]
+        assert rc == 0 and np.array_equal(_bits32(got), _bits32(want))
+    finally:
+        wsp.close()
+        w.close()
+
+
 def test_w4a8_extremes_and_tiny_scale(sess, oracle):
     M, N, K = 4, 64, 2048
     B = np.full((K, N), -8, np.int8)

@@ -69,6 +69,31 @@ def test_i8i8i32_extremes_wrap(sess, oracle):
         op.close()
 
 
+@pytest.mark.parametrize("M", [1, 9, 64, 200])
+def test_i8i8i32_sums_far_beyond_int32_wrap_like_the_exact_product(sess, oracle, M):
+    """K = 3 million with extreme columns: the exact sums reach 4.9e10, eleven times the int32
+    range, and every kernel family (decode, weight stream, large tile with its K split) has to
+    return them modulo 2^32, whatever its order of summation."""
+    N, K = 48, 3_000_017
+    rng = np.random.default_rng(900 + M)
+    B = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    B[:, 0] = -128
+    B[:, 1] = 127
+    A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    A[0] = -128
+    op = ops.W8A8Linear(sess, capi.I8I8I32, M, B)
+    try:
+        rc, got = op.run(A)
+        assert rc == 0 and np.array_equal(got, oracle.gemm_i8(A, B))
+        # the two constant columns in closed form, independent of the oracle
+        row_sums = A.astype(np.int64).sum(axis=1)
+        assert -128 * int(row_sums[0]) > 10 * 2 ** 32
+        assert np.array_equal(got[:, 0], (row_sums * -128).astype(np.int32))   # (the cast wraps)
+        assert np.array_equal(got[:, 1], (row_sums * 127).astype(np.int32))
+    finally:
+        op.close()
+
+
 F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64, 128),
               (33, 100, 130), (64, 512, 512), (100, 300, 257), (130, 768, 1024),
               (650, 7000, 1100),  # large-tile kernel
@@ -144,6 +169,23 @@ def test_f32i8f32_dynamic_and_static(sess, oracle, M, N, K):
             assert rc == capi.RK_NPU_ERR_PARAM
         finally:
             op.close()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 3_000_001, 40), (9, 3_000_001, 40), (70, 1_000_003, 33), (300_001, 300, 33)])
+def test_f32i8f32_millions_of_columns_or_rows(sess, oracle, M, N, K):
+    """The API puts no upper limit on M and N: grids of ~100 000 column blocks or row blocks,
+    outputs of hundreds of MB, element offsets beyond 2^31 bytes."""
+    rng = np.random.default_rng(M + N)
+    B = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 1e-2
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    op = ops.W8A8Linear(sess, capi.F32I8F32_DYNAMIC, M, B, ws)
+    try:
+        rc, got = op.run(A)
+        want = oracle.w8a8(A, B, ws)["C"]
+        assert rc == 0 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    finally:
+        op.close()
 
 
 def test_rounding_ties_neighbours_saturation_and_nan(sess, oracle):
