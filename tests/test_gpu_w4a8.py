@@ -266,7 +266,9 @@ def test_swiglu_bit_exact_poly_and_close_to_libm(sess, oracle, M, N, K):
 FFN_SHAPES = [(1, 64, 64, 64), (2, 256, 2048, 300), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
               (128, 384, 2048, 256),
               # an intermediate beyond 2^17: the down projection's K is split into parts, M <= 8 and M > 8
-              (2, 64, 131072 + 2112, 40), (9, 64, 131072 + 2112, 40)]
+              (2, 64, 131072 + 2112, 40), (9, 64, 131072 + 2112, 40),
+              # many rows (large-tile kernels on both projections), a very long hidden size, many rows x few columns
+              (700, 264, 1056, 300), (1, 70000, 96, 40), (5, 70000, 96, 40), (3000, 96, 64, 33), (20000, 64, 32, 1)]
 
 
 @pytest.mark.parametrize("M,H,I,Nout", FFN_SHAPES)
