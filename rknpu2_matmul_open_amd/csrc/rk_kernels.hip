@@ -748,7 +748,9 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 // again), the column scales of the epilogue fetched with the first loads (10.7), a first group
 // of 4 / 6 / 10 / 12 tiles per wave with the rest in one group behind the prologue (11.8 / 11.1 /
 // 11.0 / 11.6), four tiles per group throughout (11.4), the exact-wait kernel with four loads
-// per wave in flight (10.7).
+// per wave in flight (10.7), 28 instead of 32 columns per workgroup (512 workgroups, two for
+// every compute unit, instead of 448 -- 11.85 us; the per-lane addresses this needs cost 0.4 us
+// already with 32 columns).
 template <int MR, bool W4, int QT, int CW, bool BURST = false>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
