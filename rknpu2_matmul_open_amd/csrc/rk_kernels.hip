@@ -870,7 +870,10 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                     mx = fmaxf(mx, fabsf(v[j]));
                     bad |= not_finite(v[j]);
                 }
-                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
+                // (non-negative floats order like their bits.  For one row, a shuffle reduction per wave
+                // and one atomic per wave instead of 64 on the same address measured slower: 4096 x 14336
+                // int8 10.65 -> 10.7 us, int4 6.8 -> 7.2 us)
+                atomicMax(&row_max[m], __float_as_uint(mx));
             }
         }
         __syncthreads();
