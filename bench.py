@@ -441,6 +441,55 @@ def bench_c0(sess, ops, capi, workloads, steps, warmup):
     return out
 
 
+def bench_llm_i8(sess, ops, capi, steps, warmup):
+    """The reference's own quick benchmark (examples/bench_llm_i8.cpp:43-47,288-294): hidden, FFN-up
+    and FFN-down projections of a 7B decoder as exact int8 x int8 -> int32 products at M = 1, 4
+    and 128, reported its way -- K*N bytes / t as "weight GB/s" below 128 rows, 2*M*K*N / t as
+    GOPS at 128 -- and, like it, checked on sampled outputs against the exact integer product.
+    Here through the device-pointer call, every step on another copy of the matrix (HBM)."""
+    rng = np.random.default_rng(1234)
+    lib = sess.lib
+    rows = []
+    for name, K, N in (("hidden", 4096, 4096), ("ffn_up", 4096, 11008), ("ffn_down", 11008, 4096)):
+        B = rng.integers(-128, 128, (K, N)).astype(np.int8)
+        copies = max(2, int(400e6 // (K * N)))
+        lins = [ops.W8A8Linear(sess, capi.I8I8I32, 1, B) for _ in range(copies)]
+        cols = rng.choice(N, 64, replace=False)
+        for M in (1, 4, 128):
+            A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+            dA, dC = sess.to_device(A), sess.empty_device(M * N * 4)
+            strategy = ops.default_strategy(capi.I8I8I32, M, N, K)
+            ws = lib.rk_npu_matmul_workspace_create(sess.domain, C.byref(strategy))
+            if not ws:
+                raise RuntimeError("workspace_create")
+            turn = [0]
+
+            def step():
+                turn[0] += 1
+                rc = lib.rk_npu_i8i8i32_run_device(ws, lins[turn[0] % copies].w, dA, dC)
+                if rc:
+                    raise RuntimeError("i8i8i32_run_device rc=%d" % rc)
+
+            us = sess.time_us(step, steps, warmup)
+            got = sess.from_device(dC, (M, N), np.int32)
+            exact = A.astype(np.int64) @ B[:, cols].astype(np.int64)
+            row = {"projection": name, "M": M, "K": K, "N": N, "us": us,
+                   "pass": bool(np.array_equal(got[:, cols], exact.astype(np.int32)))}
+            if M < 128:
+                row["weight_GBps"] = K * N / us / 1e3
+            else:
+                row["GOPS"] = 2.0 * M * K * N / us / 1e3
+            rows.append(row)
+            lib.rk_npu_matmul_workspace_free(ws)
+            sess.free_device(dA)
+            sess.free_device(dC)
+        for l in lins:
+            l.close()
+    return {"workload": "the reference's bench_llm_i8 grid: rk_npu_i8i8i32 at M = 1 / 4 / 128, its reporting convention "
+                        "(weight GB/s = K*N/t below 128 rows, GOPS = 2*M*K*N/t at 128), weights from HBM, no reference "
+                        "figures are published for it", "rows": rows}
+
+
 def bench_copy(sess, steps):
     """Calibration for the rocprofv3 --pmc traffic figures: a plain device-to-device
     copy of a known size (256 MiB read + 256 MiB written per launch)."""
@@ -479,7 +528,7 @@ def main():
                     help="all: the headline line with every BASELINE configuration under \"also\" (default); "
                          "c1: config 1, config 2 and the int4 GEMV only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default=None, choices=["c0", "c1", "c1w4", "c2", "c2w8", "c3", "c4", "copy", "probes"],
+    ap.add_argument("--only", default=None, choices=["c0", "c1", "c1w4", "c2", "c2w8", "c3", "c4", "llm_i8", "copy", "probes"],
                     help="profiling aid: run one configuration's loop only")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -500,6 +549,10 @@ def main():
         print(json.dumps(practical_ceilings(sess)))
         sess.close()
         return
+    if args.only == "llm_i8":
+        print(json.dumps(bench_llm_i8(sess, ops, capi, args.steps, args.warmup)))
+        sess.close()
+        return
     if args.only:
         fn = {"c0": bench_c0, "c1w4": bench_c1w4, "c2": bench_c2, "c2w8": bench_c2w8, "c3": bench_c3, "c4": bench_c4}.get(args.only)
         res = (bench_c1(sess, ops, capi, workloads, args.steps, args.warmup, False)
@@ -518,6 +571,8 @@ def main():
         for name, fn in (("c0", bench_c0), ("c3", bench_c3), ("c4", bench_c4)):
             log("config %s" % name)
             also[name] = fn(sess, ops, capi, workloads, args.steps, args.warmup)
+        log("the reference's bench_llm_i8 grid")
+        also["llm_i8"] = bench_llm_i8(sess, ops, capi, args.steps, args.warmup)
     log("practical ceilings (read-only stream, pure MFMA loop)")
     practical = practical_ceilings(sess)
     log("config 1 (decode GEMV)")

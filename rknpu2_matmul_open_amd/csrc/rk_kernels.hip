@@ -713,6 +713,8 @@ constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
 constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
 
 // QT: 0 = activations come quantized from the tiled buffer g.A;
+//     3 = int8 rows as the caller holds them (row-major q.src): staged from there, no launch of
+//     the re-tiling kernel in front;
 //     1 / 2 = fused per-token quantization of fp16 / fp32 rows q.src (every
 //     workgroup quantizes the few rows itself -- they are L2 hits after the first
 //     -- which saves a kernel launch per decode step; workgroup 0 also writes the
@@ -757,6 +759,8 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     RK_GEMV_HEAD_APPLY(g, q);
     RK_TS(0);
     static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
+    constexpr bool FUSEQ = QT == 1 || QT == 2; // the kernel quantizes the rows itself
+    static_assert(QT != 3 || !W4, "int8 rows as given: the exact int8 x int8 product only");
     // Load instructions of a wave in flight.  One row, exact waits: four -- the quantization
     // prologue and the first dot products start after half as many bytes, and nothing is gained
     // by queueing more in front of the memory system (4096 x 14336 int4: 7.25 -> 6.8 us; int4
@@ -820,8 +824,8 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
     v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
-    typename RowLoader<QT_T>::Raw araw[QT != 0 ? GEMV_QCHUNKS : 1];
-    if constexpr (QT != 0) {
+    typename RowLoader<QT_T>::Raw araw[FUSEQ ? GEMV_QCHUNKS : 1];
+    if constexpr (FUSEQ) {
         const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
         if constexpr (BURST) {
 #pragma unroll
@@ -846,7 +850,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         }
         RK_TS(4);
     }
-    if constexpr (QT != 0) {
+    if constexpr (FUSEQ) {
         using T = QT_T;
         const int t = threadIdx.x;
         const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
@@ -917,6 +921,26 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                 const int m = idx / chunks, c = idx - m * chunks;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
+            }
+        } else if constexpr (QT == 3) {
+            // int8 rows as the caller holds them (row-major, any alignment, K not padded); the first
+            // workgroup also leaves the tiled copy a launch of the re-tiling kernel would have left
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks, gc = (kc0 >> 4) + c;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (m < g.M) {
+                    const int8_t* src = static_cast<const int8_t*>(q.src) + (size_t)m * g.K + (size_t)gc * 16;
+                    if (gc * 16 + 16 <= g.K && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+                        v = *reinterpret_cast<const uint4*>(src);
+                    } else {
+                        uint32_t w[4] = {0, 0, 0, 0};
+                        for (int j = 0; j < 16; ++j)
+                            if (gc * 16 + j < g.K) w[j >> 2] |= (uint32_t)(uint8_t)src[j] << ((j & 3) * 8);
+                        v = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                    if (first_wg && q.dst) store_codes(q.dst + tiled_chunk_offset(m, gc, KB), v);
+                }
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
             }
         }
         __syncthreads();
@@ -991,7 +1015,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             v4i w[UNR];
 #pragma unroll
             for (int u = 0; u < UNR; ++u) {
-                if constexpr (QT != 0) w[u] = wpre[u];
+                if constexpr (FUSEQ) w[u] = wpre[u];
                 else w[u] = load_unit(wave + u * GEMV_WAVES);
             }
             ActTile cur = read_act(wave);
@@ -1014,7 +1038,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             // a workgroup that asks for its next 64 KiB in one go is served faster than one that
             // trickles the requests out a tile at a time (4096 x 14336, int8: 11.5 against 11.9 us).
             int tb = wave;
-            if constexpr (QT != 0) {
+            if constexpr (FUSEQ) {
 #pragma unroll
                 for (int u = 0; u < UNR; ++u)
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(wpre[u], tb + u * GEMV_WAVES);
@@ -1053,7 +1077,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         if (W4 && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
         if (n < g.N)
             store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
-                      QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
+                      FUSEQ ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
                       g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
@@ -2683,19 +2707,30 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     // (RK_NPU_HIP_GEMV_COLS = 8 / 16 / 32 forces the choice: tuning aid)
     static const char* forced = getenv("RK_NPU_HIP_GEMV_COLS");
     const int want = forced ? atoi(forced) : 0;
-    const int cw = want == 8 || want == 16 || want == 32 ? want : pblocks <= 64 ? 8 : pblocks <= 256 ? 16 : 32;
+    // Beyond 256 blocks: whole blocks -- unless the rows come as int8 (no quantization prologue that every
+    // workgroup repeats) and halves leave the fullest compute unit with fewer columns: 344 blocks, an
+    // 11008-column projection, 2 x 32 against 3 x 16 columns, one row 10.1 -> 9.3 us, four rows
+    // 12.3 -> 10.9.  (448 blocks: 2 x 32 = 4 x 16, and whole blocks are a quarter faster.  With the
+    // quantization fused, halves cost the same 344-block matrix 6 % to 18 % for 2 to 8 rows.)
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    const bool halves = fuse && fuse->in_dtype == RKH_I8 &&
+                        ((2 * pblocks + cus - 1) / cus) * 16 < ((pblocks + cus - 1) / cus) * 32;
+    const int cw = want == 8 || want == 16 || want == 32 ? want : pblocks <= 64 ? 8 : pblocks <= 256 || halves ? 16 : 32;
     const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
-    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : fuse->in_dtype == RKH_F32 ? 2 : 3;
+    if (qt == 3 && g.w_int4) return RKH_ERR_RUNTIME; // (gemv_can_fuse lets int8 rows through for int8 weights only)
+    const char* label = qt == 3 ? "gemv_kernel (int8 rows)" : qt ? "gemv_kernel (fused quantize)" : "gemv_kernel";
     if (MR == 1 && !g.w_int4 && cw == 32) { // (the burst variant, see gemv_kernel)
-        mark(st, qt ? "gemv_kernel<burst> (fused quantize)" : "gemv_kernel<burst>");
+        mark(st, qt == 3 ? "gemv_kernel<burst> (int8 rows)" : qt ? "gemv_kernel<burst> (fused quantize)" : "gemv_kernel<burst>");
         if (qt == 0) hipLaunchKernelGGL((gemv_kernel<1, false, 0, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
         else if (qt == 1) hipLaunchKernelGGL((gemv_kernel<1, false, 1, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
-        else hipLaunchKernelGGL((gemv_kernel<1, false, 2, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else if (qt == 2) hipLaunchKernelGGL((gemv_kernel<1, false, 2, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else hipLaunchKernelGGL((gemv_kernel<1, false, 3, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
         RKH_CHECK(hipGetLastError());
         return RKH_OK;
     }
-    mark(st, qt ? "gemv_kernel (fused quantize)" : "gemv_kernel");
+    mark(st, label);
 #define RK_GEMV(W4, QT)                                                                        \
     do {                                                                                       \
         if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
@@ -2706,7 +2741,8 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     if (g.w_int4) {
         if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
     } else {
-        if (qt == 0) RK_GEMV(false, 0); else if (qt == 1) RK_GEMV(false, 1); else RK_GEMV(false, 2);
+        if (qt == 0) RK_GEMV(false, 0); else if (qt == 1) RK_GEMV(false, 1); else if (qt == 2) RK_GEMV(false, 2);
+        else RK_GEMV(false, 3);
     }
 #undef RK_GEMV
     RKH_CHECK(hipGetLastError());
@@ -2755,6 +2791,8 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
     if (g.w_int4 && !g.w_colsum) return false;
     if (g.blk_expert || g.M > 8 || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
+    // int8 rows as given (the exact int8 x int8 product): staged by the kernel in K chunks, any K
+    if (q.in_dtype == RKH_I8) return q.mode == RKH_Q_COPY_I8 && !g.w_int4 && !swiglu;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
     const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;

@@ -215,6 +215,52 @@ def _offset_copy(sess, array, elems):
     return base, p
 
 
+# int8 rows as given (the exact int8 x int8 product, the call the reference's bench_llm_i8 times):
+# for M <= 8 the GEMV stages the caller's row-major rows itself, one launch.  Every column width
+# (<= 64 / 65..256 / > 256 column blocks), ragged K (tail chunk, rows that start off a 16-byte
+# boundary because K is odd), K beyond one staging chunk (32768 / rows), wide matrices with
+# several groups of loads per wave, 5..8 rows; the last two take the two-kernel route.
+I8_SHAPES = [(1, 64, 64), (1, 200, 203), (1, 513, 1000), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520),
+             (1, 11008, 4096), (1, 9000, 4100), (1, 300, 40001), (2, 14336, 4096), (2, 3000, 700), (3, 65, 33),
+             (4, 9000, 301), (4, 4100, 9001), (8, 128, 4096), (8, 8300, 2000), (7, 5000, 4100), (2, 2500, 20003),
+             (1, 14336, 4096), (4, 14336, 600), (8, 14336, 300), (2, 100, 300),  # whole blocks (one row: the burst variant); two rows, 8 columns
+             (16, 300, 500), (130, 520, 777)]
+
+
+@pytest.mark.parametrize("M,N,K", I8_SHAPES)
+@pytest.mark.parametrize("offset", [0, 1])
+def test_i8i8i32_device(sess, oracle, M, N, K, offset):
+    rng = np.random.default_rng(M * 7 + N + K + offset)
+    A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    B = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    A[0, : min(K, 40)] = -128
+    B[: min(K, 40), 0] = -128
+    op = ops.W8A8Linear(sess, capi.I8I8I32, M, B)
+    baseA, dA = _offset_copy(sess, A, offset)      # offset 1: rows only byte-aligned
+    baseC = sess.empty_device(M * N * 4 + 64)
+    dC = baseC + 4 * offset
+    try:
+        want = oracle.gemm_i8(A, B)
+        for _ in range(2):
+            assert op.run_device(dA, dC) == 0
+            assert sess.sync() == 0
+            assert np.array_equal(sess.from_device(dC, (M, N), np.int32), want)
+        # the workspace holds the rows as a two-kernel run would have left them
+        q = np.empty((M, K), np.int8)
+        s = np.empty(M, np.float32)
+        assert sess.lib.rk_npu_matmul_workspace_read_quantized(op.ws, capi.ptr(q), capi.ptr(s)) == 0
+        assert np.array_equal(q, A)
+        # ... so the GEMM can be run again on them
+        assert sess.lib.rk_npu_hip_upload(sess.ctx, dC, capi.ptr(np.zeros((M, N), np.int32)), M * N * 4) == 0
+        assert sess.lib.rk_npu_matmul_workspace_rerun_gemm_device(op.ws, op.w, dC) == 0
+        assert sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.int32), want)
+    finally:
+        sess.free_device(baseA)
+        sess.free_device(baseC)
+        op.close()
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 9000, 520), (1, 2100, 1000), (4, 300, 200), (40, 300, 260), (300, 520, 200)])
 @pytest.mark.parametrize("f16", [True, False])
 def test_w8a8_device_pointers_with_element_alignment_only(sess, oracle, M, N, K, f16):

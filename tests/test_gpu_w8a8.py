@@ -188,6 +188,29 @@ def test_f32i8f32_millions_of_columns_or_rows(sess, oracle, M, N, K):
         op.close()
 
 
+@pytest.mark.parametrize("M,N,K,f16", [(1, 300, 600_000, True), (2, 520, 150_000, False), (8, 9000, 40_000, False),
+                                       (4, 200, 140_000, True), (3, 64, 100_003, False)])
+def test_static_scales_on_rows_beyond_the_pinned_mirror(sess, oracle, M, N, K, f16):
+    """Decode-sized calls whose rows exceed 1 MiB are uploaded instead of being read in place from
+    the pinned mirror; the caller's scales go through their own mirror."""
+    c = workloads.w8a8_case(M, K, N, seed_w=M + N + 5, seed_a=K + 17)
+    a_scale = (np.random.default_rng(M + K).random(M).astype(np.float32) + 0.2) * 0.03
+    if f16:
+        A, kind = c["A"], capi.F16I8F16_STATIC
+    else:
+        A, kind = oracle.half_to_float(c["A"]).astype(np.float32).reshape(M, K) * 2.0, capi.F32I8F32_STATIC
+    op = ops.W8A8Linear(sess, kind, M, c["B"], c["w_scale"])
+    try:
+        for _ in range(2):
+            rc, got = op.run(A, a_scale)
+            want = oracle.w8a8(A, c["B"], c["w_scale"], a_scale_static=a_scale)
+            assert rc == 0 and np.array_equal(got.view(np.uint8), want["C"].view(np.uint8))
+            q, s = op.read_quantized()
+            assert np.array_equal(q, want["q"]) and np.array_equal(s.view(np.uint32), a_scale.view(np.uint32))
+    finally:
+        op.close()
+
+
 def test_rounding_ties_neighbours_saturation_and_nan(sess, oracle):
     """Static scale 1 makes the code round-half-away(x) itself: every tie k + 0.5, the floats on either
     side of it, the largest float below 0.5 (where x + 0.5 rounds up to 1.0 in fp32), saturation beyond
