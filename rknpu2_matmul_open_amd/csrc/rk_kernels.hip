@@ -1985,7 +1985,11 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // 74.7 us with 8 steps, 74.4 with 4, 70.5 with 2; the same layer with a workgroup per tile:
     // 77.6 / 76.9 / 74.8; a dense 128-row int4 FFN and a 64-row int8 GEMM (K split over the
     // waves): 51.8 / 51.1 / 53.8 and 9.15 / 8.8 / 9.6 us.  (12 and 16 steps were slower still.)
-    constexpr int RING = KSPLIT ? 4 : 2;
+    // A workgroup per tile without a K split (dense GEMMs of 65..128 rows on wide matrices, mid-sized
+    // grouped calls): four -- a wave walks the whole K alone, 128 steps for K = 4096, and with two
+    // it waits out a full memory latency per step: int8 128 x 4096 x 11008 took 37.9 us with 2,
+    // 25.5 with 4, 25.9 with 8 (x 14336: 39.1 / 27.2 / 28.3).
+    constexpr int RING = KSPLIT ? 4 : BAL ? 2 : 4;
     constexpr int AT = W4 ? 2 : 1;   // activation tiles per step
     constexpr int LPS = AT + TN;
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
@@ -2572,7 +2576,9 @@ int compute_units() {
     }
     return cached[dev];
 }
-constexpr long DENSE_KS4_BELOW = 128; // dense use of the same kernel: every row block is live
+// dense use of the same kernel: every row block is live.  (256 or 512 instead, int8, 128 rows, K = 4096:
+// 11008 columns 25.6 -> 23.4 us, 14336 columns 27.3 -> 30.4 us.)
+constexpr long DENSE_KS4_BELOW = 128;
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
 // 256-column tile); blocks beyond the live count exit at once.  When that grid
 // would leave compute units idle (max_blocks is the caller's bound for this
