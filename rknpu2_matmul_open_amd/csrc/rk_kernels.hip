@@ -2794,9 +2794,29 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 
 // The decode path can quantize inside the GEMV when the rows fit the kernel's
 // LDS staging and per-thread register cache.
+// Whether the streaming MFMA kernel can take this dense GEMM at all (int4 codes ride as 16 * code).
+bool dense_stream_fits(const rkh_gemm_args& g) { return !g.w_int4 || g.K <= 131072; }
+
+// Most rows the dot-product kernels take for this matrix: eight, but four on a matrix of more than
+// 256 column blocks, where five to eight rows are faster as one 32-row block of the streaming MFMA
+// kernel behind a quantization launch (fp16 rows, every step from HBM, dot products against
+// stream, us: 4096 x 11008 int8 17.2 - 20.5 against 15.3 - 15.5, int4 15.5 - 18.9 against 12.3 - 12.5;
+// 4096 x 14336 18.8 - 21.9 against 16.2 - 16.5, int4 16.1 - 19.3 against 12.8 - 12.9; on narrower
+// matrices the dot products win: 4096 x 4096 9.5 - 11.6 against 13.6, 11008 x 4096 22.6 against 27.3;
+// up to four rows they win everywhere).  RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
+int gemv_max_rows(const rkh_gemm_args& g) {
+    static const int rows = [] {
+        const char* e = getenv("RK_NPU_HIP_GEMV_MAX_ROWS");
+        const int v = e ? atoi(e) : 8;
+        return v >= 1 && v <= 8 ? v : 8;
+    }();
+    const bool wide = (g.N + 31) / 32 > 256;
+    return wide && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
+}
+
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
     if (g.w_int4 && !g.w_colsum) return false;
-    if (g.blk_expert || g.M > 8 || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
+    if (g.blk_expert || g.M > gemv_max_rows(g) || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
     // int8 rows as given (the exact int8 x int8 product): staged by the kernel in K chunks, any K
     if (q.in_dtype == RKH_I8) return q.mode == RKH_Q_COPY_I8 && !g.w_int4 && !swiglu;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
@@ -3070,7 +3090,7 @@ static DensePlan effective_plan(int M, int N, int K, int w_int4) {
 // from HBM) takes 47.4 vs 53.9 us at 16 rows, 49.4 vs 47.0 at 64, 63.0 vs 56.3 at 128.
 constexpr int DENSE_STREAM_MAX_M = 128, DENSE_STREAM_SWIGLU_MAX_M = 32;
 static bool dense_streams(const rkh_gemm_args& g) {
-    if (g.blk_expert || g.M <= 8 || g.M > DENSE_STREAM_MAX_M) return false;
+    if (g.blk_expert || g.M <= gemv_max_rows(g) || g.M > DENSE_STREAM_MAX_M) return false;
     if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
     return !g.w_int4 || g.K <= 131072;
 }
@@ -3086,7 +3106,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     hipStream_t st = (hipStream_t)stream;
     const bool grouped = g.blk_expert != nullptr;
     const bool gemv_ok = !g.w_int4 || g.w_colsum; // (the int4 GEMV kernels need the column sums)
-    if (!grouped && g.M <= 8 && g.epilogue != RKH_EPI_SWIGLU && gemv_ok) return dispatch_gemv(st, g, nullptr);
+    if (!grouped && g.M <= gemv_max_rows(g) && g.epilogue != RKH_EPI_SWIGLU && gemv_ok) return dispatch_gemv(st, g, nullptr);
     if (gemv_swiglu_applies(g) && gemv_ok) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
