@@ -3046,19 +3046,41 @@ static int min_ksplit(int K, int w_int4) {
     return w_int4 ? (int)((rkh_align_up(K, RKH_K_ALIGN) + 131071) / 131072) : 1;
 }
 static long dense_tiles(int M, int N, int bm) { return (long)((M + bm - 1) / bm) * ((N + 255) / 256); }
+// Tile rows (128 / 64 / 32) and K split of a dense launch of the large-tile kernel: the candidate
+// with the smallest estimated time.  The estimate is linear in what a workgroup pulls through its
+// compute unit (K / split x (tile rows + 256 weight columns) bytes -- a compute unit moves about
+// 100 GB/s from L2, which is what bounds tiles this small), its MFMA count, the rounds the grid takes
+// on the device, and, for a split, the second launch and the int32 partial tiles written and read
+// back; the coefficients are a least-squares fit to measured times (int8, fp16 in / out, 4096 x 4096,
+// 4096 x 11008, 11008 x 4096, 4096 x 14336 at 192 to 1024 rows, nine forced plans each: the fit
+// picks the fastest or second-fastest plan for all of them).  Against the earlier rule (shrink
+// the tile until 160 tiles exist, then split): K = 11008, N = 4096 at 192 / 256 / 512 / 1024 rows
+// 50.0 -> 33.5, 53.9 -> 44.9, 71.7 -> 55.0, 82.6 -> 78.4 us; 4096 x 11008 at 192 rows 36.6 -> 31.0.
 static DensePlan dense_plan(int M, int N, int K, int w_int4) {
     const int kp = (int)rkh_align_up(K, RKH_K_ALIGN);
-    int bm = M > 64 ? 128 : M > 32 ? 64 : 32;
-    while (bm > 32 && dense_tiles(M, N, bm) < 160) bm >>= 1;
-    const long tiles = dense_tiles(M, N, bm);
-    int s = 1;
-    if (tiles < 160) {
-        s = (int)((256 + tiles - 1) / tiles);
-        const int max_s = kp / 1024 > 0 ? kp / 1024 : 1; // at least 1024 k per part
-        if (s > max_s) s = max_s;
-    }
     const int need = min_ksplit(K, w_int4);
-    return {bm, s > need ? s : need};
+    constexpr int cus = 256; // (a constant: the plan also sizes the workspace's scratch, before any launch)
+    const int max_bm = M > 64 ? 128 : M > 32 ? 64 : 32;
+    DensePlan best{max_bm, need};
+    double best_cost = 1e30;
+    for (int bm = max_bm; bm >= 32; bm >>= 1) {
+        const long tiles = dense_tiles(M, N, bm);
+        for (int ks = need; ks <= (need > 16 ? need : 16); ks *= 2) {
+            if (ks != need && kp / ks < 1024) break; // at least 1024 k per part
+            const double kpart = (double)kp / ks;
+            const double rounds = (double)((tiles * ks + cus - 1) / cus);
+            const double mem_kb = kpart * (bm + (w_int4 ? 128 : 256)) / 1e3;
+            const double kmfma = (bm / 32) * 8 * (kpart / 32) / 1e3;
+            const double part_mb = ks > 1 ? (double)tiles * ks * bm * 256 * 4 / 1e6 : 0.0;
+            if (ks != need && part_mb > 512.0) break; // (scratch the workspace would have to hold)
+            const double cost = rounds * (0.0156 * mem_kb + 0.050 * kmfma + 0.54) + (ks > 1 ? 2.9 + 0.41 * part_mb : 0.0);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = {bm, ks};
+            }
+        }
+    }
+    return best;
 }
 // RK_NPU_HIP_GEMM_PLAN="rows:ksplit" forces the workgroup tile rows (32 / 64 /
 // 128) and the K split of dense launches (tuning aid).
@@ -3090,7 +3112,9 @@ static DensePlan effective_plan(int M, int N, int K, int w_int4) {
 // from HBM) takes 47.4 vs 53.9 us at 16 rows, 49.4 vs 47.0 at 64, 63.0 vs 56.3 at 128.
 constexpr int DENSE_STREAM_MAX_M = 128, DENSE_STREAM_SWIGLU_MAX_M = 32;
 static bool dense_streams(const rkh_gemm_args& g) {
-    if (g.blk_expert || g.M <= gemv_max_rows(g) || g.M > DENSE_STREAM_MAX_M) return false;
+    static const char* forced = getenv("RK_NPU_HIP_STREAM_MAX_ROWS"); // (tuning aid)
+    const int max_rows = forced ? atoi(forced) : DENSE_STREAM_MAX_M;
+    if (g.blk_expert || g.M <= gemv_max_rows(g) || g.M > max_rows) return false;
     if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
     return !g.w_int4 || g.K <= 131072;
 }
