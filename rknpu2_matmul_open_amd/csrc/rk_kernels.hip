@@ -3049,7 +3049,7 @@ static long dense_tiles(int M, int N, int bm) { return (long)((M + bm - 1) / bm)
 // Tile rows (128 / 64 / 32) and K split of a dense launch of the large-tile kernel: the candidate
 // with the smallest estimated time.  The estimate is linear in what a workgroup pulls through its
 // compute unit (K / split x (tile rows + 256 weight columns) bytes -- a compute unit moves about
-// 100 GB/s from L2, which is what bounds tiles this small), its MFMA count, the rounds the grid takes
+// 100 GB/s from L2, which is what bounds tiles this small) or its MFMA count, the rounds the grid takes
 // on the device, and, for a split, the second launch and the int32 partial tiles written and read
 // back; the coefficients are a least-squares fit to measured times (int8, fp16 in / out, 4096 x 4096,
 // 4096 x 11008, 11008 x 4096, 4096 x 14336 at 192 to 1024 rows, nine forced plans each: the fit
@@ -3073,7 +3073,10 @@ static DensePlan dense_plan(int M, int N, int K, int w_int4) {
             const double kmfma = (bm / 32) * 8 * (kpart / 32) / 1e3;
             const double part_mb = ks > 1 ? (double)tiles * ks * bm * 256 * 4 / 1e6 : 0.0;
             if (ks != need && part_mb > 512.0) break; // (scratch the workspace would have to hold)
-            const double cost = rounds * (0.0156 * mem_kb + 0.050 * kmfma + 0.54) + (ks > 1 ? 2.9 + 0.41 * part_mb : 0.0);
+            // (4.4 us per 1000 MFMAs of a workgroup: 250 per SIMD, 32 cycles each, at the 1.8 GHz the matrix
+            // pipes sustain -- the bound of the 128-row tile with int4 weights, whose bytes are few)
+            const double loop_us = 0.0156 * mem_kb > 4.4 * kmfma ? 0.0156 * mem_kb : 4.4 * kmfma;
+            const double cost = rounds * (loop_us + 0.54) + (ks > 1 ? 2.9 + 0.41 * part_mb : 0.0);
             if (cost < best_cost) {
                 best_cost = cost;
                 best = {bm, ks};
