@@ -219,12 +219,16 @@ def _offset_copy(sess, array, elems):
 # for M <= 8 the GEMV stages the caller's row-major rows itself, one launch.  Every column width
 # (<= 64 / 65..256 / > 256 column blocks), ragged K (tail chunk, rows that start off a 16-byte
 # boundary because K is odd), K beyond one staging chunk (32768 / rows), wide matrices with
-# several groups of loads per wave, 5..8 rows; the last two take the two-kernel route.
+# several groups of loads per wave, 5..8 rows; (16, 300, 500) and (130, 520, 777) take the two-kernel route.
 I8_SHAPES = [(1, 64, 64), (1, 200, 203), (1, 513, 1000), (1, 4096, 4096), (1, 2100, 8200), (1, 9000, 520),
              (1, 11008, 4096), (1, 9000, 4100), (1, 300, 40001), (2, 14336, 4096), (2, 3000, 700), (3, 65, 33),
              (4, 9000, 301), (4, 4100, 9001), (8, 128, 4096), (8, 8300, 2000), (7, 5000, 4100), (2, 2500, 20003),
              (1, 14336, 4096), (4, 14336, 600), (8, 14336, 300), (2, 100, 300),  # whole blocks (one row: the burst variant); two rows, 8 columns
-             (16, 300, 500), (130, 520, 777)]
+             (16, 300, 500), (130, 520, 777),
+             # 9..128 rows on the streaming kernel behind the re-tiling launch (K split over the waves / not; a K
+             # of one and of three k-tiles; ragged last row block)
+             (16, 300, 512), (33, 4100, 4096), (128, 11008, 4096), (100, 64, 32), (9, 8448, 96), (64, 520, 2080),
+             (97, 9000, 288), (128, 4096, 11008)]
 
 
 @pytest.mark.parametrize("M,N,K", I8_SHAPES)
