@@ -218,6 +218,34 @@ typedef struct rkh_moe_combine_args {
 } rkh_moe_combine_args;
 int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args);
 
+/* A MoE layer for a handful of tokens in two launches instead of five, same results: (1) per
+ * (assignment, 32 middle columns) the token is quantized, multiplied with the gate and up blocks
+ * of its expert and passed through SwiGLU -> hidden + partial row maxima; (2) per (token, 32
+ * output columns) each live slot's hidden row is re-quantized from the partial maxima, multiplied
+ * with the expert's down block, scaled and accumulated in slot order.  Everything device-resident.
+ * Returns RKH_ERR_RUNTIME for shapes it does not take (rkh_moe_decode_applies). */
+typedef struct rkh_moe_decode_args {
+    const float* x;          /* [rows, H] fp32 tokens                                */
+    const int32_t* ids;      /* [rows, top_k]                                        */
+    const float* routes;     /* [rows, top_k]                                        */
+    int rows, top_k, experts, shared; /* experts = routed count; the shared one is expert `experts` */
+    int H, I;
+    const uint8_t* gate_W;   /* int8 experts: tiled [2I x H] images, gate / up blocks interleaved */
+    const uint8_t* gate_W4;  /* int4 experts (the first int4_experts of the bank)    */
+    const uint8_t* down_W;
+    const uint8_t* down_W4;
+    int int4_experts;
+    size_t gate_stride, gate_stride4, down_stride, down_stride4; /* bytes between experts */
+    const float* gate_scales; /* [experts + shared][2I]                              */
+    const float* down_scales; /* [experts + shared][H]                               */
+    float* hidden;           /* scratch [rows * (top_k + shared)][I]                 */
+    uint32_t* row_max_bits;  /* scratch [rows * (top_k + shared)][I / 32]            */
+    float* out;              /* [rows, H]                                            */
+    int* bad_flag;           /* OR 1 on a rejected token or routing entry, may be NULL */
+} rkh_moe_decode_args;
+int rkh_moe_decode_applies(int rows, int H, int I);
+int rkh_moe_decode(void* stream, const rkh_moe_decode_args* args);
+
 
 /* ---- measurement probes (practical ceilings beside the datasheet peaks) ---- */
 /* One read-only pass over [src, src + bytes): a workgroup of 512 lanes per `span` bytes

@@ -2488,6 +2488,307 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* h_Y, cons
 }
 
 
+// ------------------------------------------------ MoE layer for a handful of tokens
+// With a few tokens the five launches of the layer (route + scatter, grouped gate/up, middle
+// re-quantization, grouped down, combine) are almost all latency, and the grouped MFMA kernel
+// works on 32-row blocks with one live row.  These two kernels do the same arithmetic with dot
+// products, one workgroup of eight waves per (assignment, 32 columns):
+//   gate:  token -> int8 (every workgroup quantizes its token itself, the row is an L2 hit after
+//          the first), gate and up blocks of the assignment's expert streamed like a decode GEMV,
+//          SwiGLU, the fp32 middle and its partial maximum per 32 columns;
+//   down:  per token and 32 output columns, the live slots in slot order: the slot's middle row
+//          re-quantized from the partial maxima, the expert's down block, dequantization and the
+//          fma into the token's sum -- the combine's order and rounding.
+// No routing tables: an assignment is live iff its coefficient is non-zero and its id in range
+// (the shared expert: always), which both kernels read from the caller's arrays.
+constexpr int MOE_DECODE_MAX_K = 32768; // int8 codes of a token / a middle row staged in LDS
+
+struct MoeSlot { int expert; float coeff; bool live, bad; };
+__device__ __forceinline__ MoeSlot moe_slot(const rkh_moe_decode_args& a, int t, int s) {
+    if (s >= a.top_k) return {a.experts, 1.0f, true, false};
+    const int id = a.ids[(size_t)t * a.top_k + s];
+    const float c = a.routes[(size_t)t * a.top_k + s];
+    const bool id_ok = (unsigned)id < (unsigned)a.experts;
+    return {id, c, c != 0.0f && id_ok, !id_ok || not_finite(c) || c < 0.0f};
+}
+
+// One 1 KiB tile of a tiled expert image against the staged int8 row: a k-tile of int8 codes, or
+// an int4 super-tile of two k-tiles, multiplied as 16 * code (the sum is shifted back at the end).
+// `idx` counts tiles of the column block, `w` is the lane's 16 bytes of the tile.
+__device__ __forceinline__ void moe_dot_tile(bool int4, const uint8_t* a_lds, int idx, int half, const v4i& w, int& acc) {
+    if (!int4) {
+        const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)(idx * 2 + half) * 16);
+        acc = __builtin_amdgcn_sdot4(av.x, w.x, acc, false);
+        acc = __builtin_amdgcn_sdot4(av.y, w.y, acc, false);
+        acc = __builtin_amdgcn_sdot4(av.z, w.z, acc, false);
+        acc = __builtin_amdgcn_sdot4(av.w, w.w, acc, false);
+    } else {
+        const v4i a0 = *reinterpret_cast<const v4i*>(a_lds + (size_t)(idx * 4 + half) * 16);
+        const v4i a1 = *reinterpret_cast<const v4i*>(a_lds + (size_t)(idx * 4 + 2 + half) * 16);
+        // a word holds eight codes: byte j = k + j (low nibble) and k + 4 + j (high nibble)
+        acc = __builtin_amdgcn_sdot4(a0.x, (w.x << 4) & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a0.y, w.x & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a0.z, (w.y << 4) & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a0.w, w.y & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a1.x, (w.z << 4) & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a1.y, w.z & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a1.z, (w.w << 4) & (int)0xF0F0F0F0, acc, false);
+        acc = __builtin_amdgcn_sdot4(a1.w, w.w & (int)0xF0F0F0F0, acc, false);
+    }
+}
+__device__ __forceinline__ v4i moe_load_tile(const uint8_t* block, int idx, int tiles, int lane) {
+    return idx < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(block + (size_t)idx * 1024 + lane * 16))
+                       : v4i{0, 0, 0, 0};
+}
+
+constexpr int MOE_DECODE_PREFETCH = 4; // tiles per wave and column block requested ahead of the quantization
+
+__global__ __launch_bounds__(512) void moe_decode_gate_kernel(rkh_moe_decode_args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[MOE_DECODE_MAX_K];
+    __shared__ int red[2][8][32];
+    __shared__ float wave_max[8];
+    __shared__ int wave_bad[8];
+    const int slots = a.top_k + a.shared;
+    const int j = blockIdx.x, asg = blockIdx.y, t = asg / slots, s = asg - t * slots;
+    const int tid = threadIdx.x, lane = lane_id(), wave = wave_id(), half = lane >> 5;
+    const MoeSlot slot = moe_slot(a, t, s);
+    const bool reporter = j == 0 && tid == 0;
+    if (slot.bad && reporter && a.bad_flag) atomicOr(a.bad_flag, 1);
+    if (!slot.live) return;
+
+    // ---- gate block 2j and up block 2j + 1 of the expert: the first tiles are requested now
+    const int H = a.H, Hp = (int)rkh_align_up(H, RKH_K_ALIGN), nchunks = (H + 15) >> 4;
+    const int e = slot.expert;
+    const bool int4 = e < a.int4_experts;
+    const int tiles = int4 ? Hp / 64 : Hp / 32; // per column block
+    const size_t block_bytes = (size_t)tiles * 1024;
+    const uint8_t* wb = (int4 ? a.gate_W4 + (size_t)e * a.gate_stride4
+                              : a.gate_W + (size_t)(e - a.int4_experts) * a.gate_stride) + (size_t)(2 * j) * block_bytes;
+    v4i pre[2][MOE_DECODE_PREFETCH];
+#pragma unroll
+    for (int u = 0; u < MOE_DECODE_PREFETCH; ++u)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) pre[b][u] = moe_load_tile(wb + b * block_bytes, wave + 8 * u, tiles, lane);
+
+    // ---- the token as int8 codes in LDS (s = max > 0 ? max / 127 : 1, ties to even)
+    const float* row = a.x + (size_t)t * H;
+    const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+    constexpr int CACHE = MOE_DECODE_MAX_K / 16 / 512; // chunks per thread
+    float v[CACHE][16];
+    float mx = 0.0f;
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < CACHE; ++i) {
+        const int c = tid + i * 512;
+        if (c < nchunks) {
+            RowLoader<float>::load16(row, c * 16, H, vec, v[i]);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                mx = fmaxf(mx, fabsf(v[i][q]));
+                bad |= not_finite(v[i][q]);
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const unsigned long long bad_mask = __ballot(bad);
+    if (lane == 0) {
+        wave_max[wave] = mx;
+        wave_bad[wave] = bad_mask != 0ull;
+    }
+    __syncthreads();
+    mx = 0.0f;
+    int any_bad = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        mx = fmaxf(mx, wave_max[w]);
+        any_bad |= wave_bad[w];
+    }
+    const float scale = mx > 0.0f ? mx / 127.0f : 1.0f;
+    const float inv = 1.0f / scale;
+    // (a non-finite token, or a maximum so small that the scale or its inverse leaves the fp32 range)
+    if (reporter && a.bad_flag && (any_bad || !(scale > 0.0f) || not_finite(inv))) atomicOr(a.bad_flag, 1);
+#pragma unroll
+    for (int i = 0; i < CACHE; ++i) {
+        const int c = tid + i * 512;
+        if (c < nchunks) *reinterpret_cast<uint4*>(a_lds + (size_t)c * 16) = quantize16<true>(v[i], inv);
+    }
+    for (int c = nchunks + tid; c < Hp / 16; c += 512) *reinterpret_cast<uint4*>(a_lds + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+
+    // ---- dot products: the waves take the tiles of both blocks in turn
+    int acc[2] = {0, 0};
+#pragma unroll
+    for (int u = 0; u < MOE_DECODE_PREFETCH; ++u)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+            if (wave + 8 * u < tiles) moe_dot_tile(int4, a_lds, wave + 8 * u, half, pre[b][u], acc[b]);
+#pragma unroll 2
+    for (int idx = wave + 8 * MOE_DECODE_PREFETCH; idx < tiles; idx += 8) {
+        const v4i w0 = moe_load_tile(wb, idx, tiles, lane), w1 = moe_load_tile(wb + block_bytes, idx, tiles, lane);
+        moe_dot_tile(int4, a_lds, idx, half, w0, acc[0]);
+        moe_dot_tile(int4, a_lds, idx, half, w1, acc[1]);
+    }
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        int p = acc[b];
+        p += __shfl_xor(p, 32);
+        if (lane < 32) red[b][wave][lane] = p;
+    }
+    __syncthreads();
+    if (tid < 32) {
+        int gate = 0, up = 0;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            gate += red[0][w][tid];
+            up += red[1][w][tid];
+        }
+        if (int4) {
+            gate >>= 4;
+            up >>= 4;
+        }
+        const int n = j * 32 + tid; // (I is a multiple of 32)
+        // (fetched here, not with the first tiles: requested early the two scales made the kernel a
+        // third slower for four and eight tokens)
+        const float* ws = a.gate_scales + (size_t)e * 2 * a.I;
+        const float gf = dequant(gate, scale, ws[n]);
+        const float uf = dequant(up, scale, ws[a.I + n]);
+        const float y = __fmul_rn(silu_poly(gf), uf);
+        a.hidden[(size_t)asg * a.I + n] = y;
+        uint32_t bits = __float_as_uint(y) & 0x7fffffffu;
+#pragma unroll
+        for (int d = 16; d > 0; d >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, d));
+        if (tid == 0) a.row_max_bits[(size_t)asg * (a.I / 32) + j] = bits;
+    }
+}
+
+// One workgroup per (token, 32 output columns).  The live slots' middle rows are re-quantized side
+// by side in LDS first (a wave per slot; row and partial maxima requested together), then the eight
+// waves walk the slots' down blocks in one sequence of groups of tiles with the next group's loads
+// always in flight -- also across the boundary between two slots, and the first group ahead of the
+// re-quantization -- and the first 32 threads add the slots' dequantized values in slot order.
+constexpr int MOE_DECODE_SLOTS = ROUTE_MAX_TOPK + 1;
+constexpr int MOE_DECODE_DOWN_K = 3584; // longest middle row (padded): nine of them fit the staging area
+static_assert(MOE_DECODE_SLOTS * MOE_DECODE_DOWN_K <= MOE_DECODE_MAX_K, "staging area");
+__global__ __launch_bounds__(512) void moe_decode_down_kernel(rkh_moe_decode_args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[MOE_DECODE_MAX_K]; // live slot i at i * Ip
+    __shared__ int red[MOE_DECODE_SLOTS][8][32];
+    __shared__ float live_scale[MOE_DECODE_SLOTS], live_coeff[MOE_DECODE_SLOTS];
+    __shared__ int live_expert[MOE_DECODE_SLOTS], live_slot[MOE_DECODE_SLOTS];
+    __shared__ int live_count;
+    const int slots = a.top_k + a.shared;
+    const int pb = blockIdx.x, t = blockIdx.y;
+    const int tid = threadIdx.x, lane = lane_id(), wave = wave_id(), half = lane >> 5;
+    const int I = a.I, Ip = (int)rkh_align_up(I, RKH_K_ALIGN), nchunks = I >> 4, parts = I / 32;
+    if (tid == 0) { // the live slots in slot order
+        int n = 0;
+        for (int s = 0; s < slots; ++s) {
+            const MoeSlot slot = moe_slot(a, t, s);
+            if (slot.live) {
+                live_expert[n] = slot.expert;
+                live_coeff[n] = slot.coeff;
+                live_slot[n] = s;
+                ++n;
+            }
+        }
+        live_count = n;
+    }
+    __syncthreads();
+    const int nlive = live_count;
+    // a slot's tiles are walked in groups of 8 waves x PF tiles
+    constexpr int PF = MOE_DECODE_PREFETCH;
+    auto block_of = [&](int li, bool& int4, int& tiles) -> const uint8_t* {
+        const int e = live_expert[li];
+        int4 = e < a.int4_experts;
+        tiles = int4 ? Ip / 64 : Ip / 32;
+        return (int4 ? a.down_W4 + (size_t)e * a.down_stride4
+                     : a.down_W + (size_t)(e - a.int4_experts) * a.down_stride) + (size_t)pb * tiles * 1024;
+    };
+    auto load_group = [&](int li, int grp, v4i* regs) {
+        bool int4;
+        int tiles;
+        const uint8_t* wb = block_of(li, int4, tiles);
+#pragma unroll
+        for (int u = 0; u < PF; ++u) regs[u] = moe_load_tile(wb, (grp * PF + u) * 8 + wave, tiles, lane);
+    };
+    v4i cur[PF], nxt[PF];
+    if (nlive > 0) load_group(0, 0, cur);
+
+    // ---- the middle rows (max != 0 ? max / 127 : 1, ties to even)
+    for (int li = wave; li < nlive; li += 8) {
+        const int asg = t * slots + live_slot[li];
+        const float* hrow = a.hidden + (size_t)asg * I;
+        constexpr int CACHE = (MOE_DECODE_DOWN_K / 16 + 63) / 64; // chunks per lane
+        float v[CACHE][16];
+#pragma unroll
+        for (int i = 0; i < CACHE; ++i) {
+            const int c = lane + 64 * i;
+            if (c < nchunks) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 f = *reinterpret_cast<const float4*>(hrow + c * 16 + q * 4);
+                    v[i][q * 4] = f.x; v[i][q * 4 + 1] = f.y; v[i][q * 4 + 2] = f.z; v[i][q * 4 + 3] = f.w;
+                }
+            }
+        }
+        uint32_t bits = 0;
+        for (int i = lane; i < parts; i += 64) bits = max(bits, a.row_max_bits[(size_t)asg * parts + i]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
+        const float mx = __uint_as_float(bits);
+        const float scale = mx != 0.0f ? mx / 127.0f : 1.0f;
+        const float inv = 1.0f / scale;
+        if (lane == 0) live_scale[li] = scale;
+#pragma unroll
+        for (int i = 0; i < CACHE; ++i) {
+            const int c = lane + 64 * i;
+            if (c < Ip / 16)
+                *reinterpret_cast<uint4*>(a_lds + (size_t)li * Ip + (size_t)c * 16) =
+                    c < nchunks ? quantize16<true>(v[i], inv) : make_uint4(0, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+
+    // ---- the down blocks
+    for (int li = 0; li < nlive; ++li) {
+        bool int4;
+        int tiles;
+        block_of(li, int4, tiles);
+        const int groups = (tiles + 8 * PF - 1) / (8 * PF);
+        const uint8_t* codes = a_lds + (size_t)li * Ip;
+        int acc = 0;
+        for (int grp = 0; grp < groups; ++grp) {
+            const bool last = grp + 1 == groups;
+            if (!last) load_group(li, grp + 1, nxt);
+            else if (li + 1 < nlive) load_group(li + 1, 0, nxt);
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int idx = (grp * PF + u) * 8 + wave;
+                if (idx < tiles) moe_dot_tile(int4, codes, idx, half, cur[u], acc);
+            }
+#pragma unroll
+            for (int u = 0; u < PF; ++u) cur[u] = nxt[u];
+        }
+        acc += __shfl_xor(acc, 32);
+        if (lane < 32) red[li][wave][lane] = acc;
+    }
+    __syncthreads();
+    if (tid < 32) {
+        const int n = pb * 32 + tid; // (H is a multiple of 32)
+        float sum = 0.0f;
+        for (int li = 0; li < nlive; ++li) {
+            int acc = 0;
+#pragma unroll
+            for (int w = 0; w < 8; ++w) acc += red[li][w][tid];
+            const int e = live_expert[li];
+            if (e < a.int4_experts) acc >>= 4;
+            const float y = dequant(acc, live_scale[li], a.down_scales[(size_t)e * a.H + n]);
+            sum = fmaf(y, live_coeff[li], sum);
+        }
+        a.out[(size_t)t * a.H + n] = sum;
+    }
+}
+
 // ------------------------------------------------------ measurement probes
 // What the memory system and the matrix pipes give on the box the benchmark runs
 // on, to put beside the datasheet peaks: a read-only stream over a footprint and
@@ -3193,6 +3494,25 @@ int rkh_moe_combine(void* stream, const rkh_moe_combine_args* args) {
     mark((hipStream_t)stream, "moe_combine_kernel");
     hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, (hipStream_t)stream, args->Y, args->dest_rows,
                        args->routes, args->out, args->rows, args->top_k, args->shared, args->H);
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+int rkh_moe_decode_applies(int rows, int H, int I) {
+    static const char* forced = getenv("RK_NPU_HIP_MOE_DECODE_ROWS"); // (tuning aid: 0 switches the path off)
+    const int max_rows = forced ? atoi(forced) : 8;
+    return rows >= 1 && rows <= max_rows && H >= 32 && H % 32 == 0 && H <= MOE_DECODE_MAX_K && I >= 32 && I % 32 == 0 &&
+           rkh_align_up(I, RKH_K_ALIGN) <= (size_t)MOE_DECODE_DOWN_K; // (nine middle rows side by side in LDS)
+}
+
+int rkh_moe_decode(void* stream, const rkh_moe_decode_args* args) {
+    const rkh_moe_decode_args& a = *args;
+    if (!rkh_moe_decode_applies(a.rows, a.H, a.I) || a.top_k < 1) return RKH_ERR_RUNTIME;
+    const int slots = a.top_k + (a.shared ? 1 : 0);
+    mark((hipStream_t)stream, "moe_decode_gate_kernel");
+    hipLaunchKernelGGL(moe_decode_gate_kernel, dim3(a.I / 32, a.rows * slots), dim3(512), 0, (hipStream_t)stream, a);
+    mark((hipStream_t)stream, "moe_decode_down_kernel");
+    hipLaunchKernelGGL(moe_decode_down_kernel, dim3(a.H / 32, a.rows), dim3(512), 0, (hipStream_t)stream, a);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }

@@ -134,11 +134,49 @@ namespace {
 // f32, else int8 [rows, H] with d_scales[rows].
 int enqueue(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int rows,
             const void* d_input, bool f32, const float* d_scales, const int32_t* d_ids,
-            const float* d_routes, float* d_out, StageTimer* timer) {
+            const float* d_routes, float* d_out, StageTimer* timer, bool device_resident = false) {
     const auto& wc = ws->config.weights;
     const int H = wc.hidden, I = wc.intermediate;
     void* stream = ws->owner.ctx->stream;
     auto mark = [&] { if (timer) timer->mark(); };
+    // A handful of fp32 tokens whose rows and routing table lie in device memory: two launches of
+    // dot-product kernels instead of the five of the grouped path (every workgroup of a token reads
+    // its row and its routing entries, which is why operands in the pinned host mirrors do not qualify).
+    if (device_resident && f32 && rkh_moe_decode_applies(rows, H, I)) {
+        rkh_moe_decode_args a{};
+        a.x = static_cast<const float*>(d_input);
+        a.ids = d_ids;
+        a.routes = d_routes;
+        a.rows = rows;
+        a.top_k = ws->config.top_k;
+        a.experts = wc.routed_experts;
+        a.shared = wc.shared_expert ? 1 : 0;
+        a.H = H;
+        a.I = I;
+        a.gate_W = w->gate_up ? w->gate_up.as<>() : nullptr;
+        a.gate_W4 = w->gate_up4 ? w->gate_up4.as<>() : nullptr;
+        a.down_W = w->down ? w->down.as<>() : nullptr;
+        a.down_W4 = w->down4 ? w->down4.as<>() : nullptr;
+        a.int4_experts = w->count4;
+        a.gate_stride = w->gate_stride;
+        a.gate_stride4 = w->gate_stride4;
+        a.down_stride = w->down_stride;
+        a.down_stride4 = w->down_stride4;
+        a.gate_scales = w->gate_scales.as<float>();
+        a.down_scales = w->down_scales.as<float>();
+        a.hidden = ws->hidden.as<float>();
+        a.row_max_bits = ws->row_max.as<uint32_t>();
+        a.out = d_out;
+        a.bad_flag = ws->flag.device();
+        mark(); // 1: schedule
+        mark(); // 2: input
+        const int rc = rkh_moe_decode(stream, &a);
+        mark(); // 3: gate
+        mark(); // 4: middle
+        mark(); // 5: down
+        mark(); // 6: combine
+        return map_error(rc);
+    }
     // most row blocks this call can produce (the workspace's max_blocks is the same bound for max_rows)
     const int routed = rows * ws->config.top_k;
     const int call_blocks = std::min(ws->max_blocks, routed / 32 + std::min(wc.routed_experts, routed) +
@@ -734,7 +772,7 @@ int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w
     if (rc) return rc;
     std::lock_guard<std::mutex> submit(ws->owner.ctx->submit_mutex);
     note_pending_flag(ws->owner.ctx, ws->flag.device());
-    return enqueue(ws, w, rows, input, true, nullptr, ids, routes, out, nullptr);
+    return enqueue(ws, w, rows, input, true, nullptr, ids, routes, out, nullptr, true);
 }
 
 } // extern "C"
