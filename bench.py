@@ -406,6 +406,37 @@ def bench_c4(sess, ops, capi, workloads, steps, warmup):
            "roofline": _hbm("whole step; dominant: gemm_stream_kernel<SwiGLU> (grouped gate/up, 134 MB of expert weights)",
                             algo_bytes, step_us, "moe_c4", algorithmic_ops=ops_count),
            "kernels": _kernels(sess, ops, step)}
+
+    # The same layer at decode size: 1, 4 and 8 tokens per call.  Every step takes the next tokens of the
+    # 256 (another set of experts) and the other bank, so the expert weights come from HBM here too.
+    want = None
+    decode = []
+    for rows in (1, 4, 8):
+        at = [0]
+
+        def small_step():
+            first = (at[0] * rows) % (c["T"] - rows + 1)
+            bank = banks[at[0] % MOE_COPIES]
+            at[0] += 1
+            rc = sess.lib.rk_npu_moe_w8_run_f32_device(moe.ws, bank.w, rows, dx + first * c["H"] * 4,
+                                                        dids + first * c["top_k"] * 4, drt + first * c["top_k"] * 4, dout)
+            if rc:
+                raise RuntimeError("moe rc=%d" % rc)
+
+        us = sess.time_us(small_step, steps, warmup)
+        # the rows of the last call against the same tokens' rows of the 256-token call (grouped path)
+        last = ((at[0] - 1) * rows) % (c["T"] - rows + 1)
+        got = sess.from_device(dout, (rows, c["H"]), np.float32)
+        if want is None:
+            step()
+            if sess.sync():
+                raise RuntimeError("sync")
+            want = sess.from_device(dout, (c["T"], c["H"]), np.float32)
+        decode.append({"tokens": rows, "us": us,
+                       "equals_rows_of_the_256_token_call": bool(np.array_equal(got.view(np.uint32),
+                                                                                want[last:last + rows].view(np.uint32)))})
+    out["decode_sized_calls"] = {"note": "1 / 4 / 8 tokens per call through the same device-pointer call: two launches of "
+                                         "dot-product kernels instead of five of the grouped path", "rows": decode}
     for d in (dx, dids, drt, dout):
         sess.free_device(d)
     for b in banks:
