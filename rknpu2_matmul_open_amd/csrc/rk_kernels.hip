@@ -16,6 +16,8 @@
 //                                       (grouped by expert) and dense GEMMs of 9..128 rows (HBM)
 //   moe_scatter_kernel                  route by expert + quantize tokens into sorted rows (latency)
 //   moe_combine_kernel                  weighted sum of expert outputs in slot order     (HBM, small)
+//   moe_decode_gate_kernel / moe_decode_down_kernel   the MoE layer for up to eight tokens in two
+//                                       launches: dot products, no routing tables          (latency, HBM)
 //   stream_read_probe_kernel / mfma_i8_probe_kernel   measurement probes (practical ceilings)
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
