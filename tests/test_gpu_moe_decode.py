@@ -42,7 +42,8 @@ def _run_device(sess, moe, x, ids, routes):
 
 
 # (T, H, I, E, top_k, shared): every token count of the path, the smallest and large geometries, a K
-# that is not a multiple of the 256 the weights are padded to, the widest middle, many slots
+# that is not a multiple of the 256 the weights are padded to, many slots, the longest token row; and a
+# middle too long for the path (8192: that call takes the grouped path and must agree all the same)
 CASES = [(1, 64, 32, 3, 2, 1), (1, 2048, 1024, 32, 4, 0), (2, 128, 64, 6, 2, 0), (3, 96, 160, 5, 3, 1),
          (4, 2048, 1024, 32, 4, 1), (5, 416, 96, 9, 8, 0), (7, 64, 8192, 4, 2, 1), (8, 4096, 512, 16, 4, 0),
          (8, 160, 32, 40, 8, 1), (6, 32768, 32, 2, 1, 0)]
@@ -184,3 +185,31 @@ def test_the_same_tokens_in_a_larger_call_give_the_same_rows(sess, oracle):
             assert np.array_equal(small.view(np.uint32), big[first:first + 8].view(np.uint32))
     finally:
         moe.close()
+
+
+def test_random_geometries(sess, oracle):
+    """Seeded random layer geometries, routings (with dropped and duplicate slots) and token counts."""
+    rng = np.random.default_rng(20240611)
+    for case in range(24):
+        T = int(rng.integers(1, 9))
+        H = int(rng.integers(2, 33)) * 32
+        I = int(rng.integers(1, 17)) * 32
+        E = int(rng.integers(1, 13))
+        top_k = int(rng.integers(1, min(E, 8) + 1))
+        shared = int(rng.integers(0, 2))
+        flavour = "quant" if (H % 64 == 0 and I % 64 == 0 and case % 3 == 0) else "w8"
+        lo, hi = (-8, 7) if flavour == "quant" else (-127, 127)
+        experts = _experts(rng, H, I, E + shared, lo, hi)
+        x = (rng.standard_normal((T, H)) * float(rng.choice([0.01, 1.0, 50.0]))).astype(np.float32)
+        ids = rng.integers(0, E, (T, top_k)).astype(np.int32)            # duplicates allowed
+        routes = rng.random((T, top_k), dtype=np.float32)
+        routes[rng.random((T, top_k)) < 0.2] = 0.0                       # dropped slots
+        moe = ops.MoeW8(sess, H, I, E, shared, top_k, 8, experts, flavour=flavour)
+        try:
+            rc, sync, got = _run_device(sess, moe, x, ids, routes)
+            rc2, want = oracle.moe_w8(experts, H, I, E, shared, top_k, ids, routes, input_f32=x)
+            what = (case, T, H, I, E, top_k, shared, flavour)
+            assert rc == 0 and sync == 0 and rc2 == 0, what
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), what
+        finally:
+            moe.close()
