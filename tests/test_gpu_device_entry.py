@@ -340,3 +340,29 @@ def test_moe_device_pointers_with_element_alignment_only(sess, oracle, T):
         for d in (bx, bi, br, bo):
             sess.free_device(d)
         moe.close()
+
+
+def test_i8i8i32_device_random_shapes(sess, oracle):
+    """Seeded random shapes through every route of the exact int8 x int8 product: one to eight rows
+    (dot products, rows staged by the kernel), up to 128 rows (streaming kernel), more (large tiles,
+    with whatever tile height and K split the plan picks)."""
+    rng = np.random.default_rng(987654)
+    for case in range(36):
+        M = int(rng.choice([rng.integers(1, 9), rng.integers(9, 129), rng.integers(129, 700)]))
+        N = int(rng.choice([rng.integers(1, 300), rng.integers(300, 3000), rng.integers(3000, 12000)]))
+        K = int(rng.choice([rng.integers(1, 200), rng.integers(200, 3000), rng.integers(3000, 12000)]))
+        A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        B = rng.integers(-128, 128, (K, N)).astype(np.int8)
+        op = ops.W8A8Linear(sess, capi.I8I8I32, M, B)
+        offset = case % 2
+        baseA, dA = _offset_copy(sess, A, offset)
+        dC = sess.empty_device(M * N * 4)
+        try:
+            assert op.run_device(dA, dC) == 0, (case, M, N, K)
+            assert sess.sync() == 0, (case, M, N, K)
+            got = sess.from_device(dC, (M, N), np.int32)
+            assert np.array_equal(got, oracle.gemm_i8(A, B)), (case, M, N, K)
+        finally:
+            sess.free_device(baseA)
+            sess.free_device(dC)
+            op.close()
