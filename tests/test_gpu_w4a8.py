@@ -448,3 +448,42 @@ def test_k_tile_resolution_against_reference_golden(sess):
             assert bool(h) == bool(ok), (case["recipe"], tile)
             if h:
                 sess.lib.rk_npu_w4a8_weights_free(h)
+
+
+def test_random_shapes_through_the_launch_plan(sess, oracle):
+    """Seeded random shapes of more than 128 rows: whatever tile height and K split the dense plan
+    picks (long K with few columns is split over workgroups, wide matrices are not), the int32 sums
+    and the fp32 output are the oracle's, for int4 weights here and int8 weights below."""
+    rng = np.random.default_rng(424242)
+    for case in range(20):
+        M = int(rng.integers(129, 900))
+        N = int(rng.choice([rng.integers(1, 300), rng.integers(300, 2500)]))
+        K = int(rng.choice([rng.integers(1, 300), rng.integers(300, 3000), rng.integers(3000, 14000)]))
+        B = _codes(rng, (K, N))
+        ws = (rng.random(N).astype(np.float32) + 0.5) * 0.01
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        w = ops.W4A8Weights(sess, B, ws)
+        wsp = ops.W4A8Workspace(sess, M, N, K)
+        try:
+            want = oracle.w4a8(A, B, ws)
+            rc, acc = wsp.run_i32(w, A)
+            assert rc == 0 and np.array_equal(acc, want["acc"]), (case, M, N, K)
+            rc, got = wsp.run_f32(w, A)
+            assert rc == 0 and np.array_equal(_bits32(got), _bits32(want["C"])), (case, M, N, K)
+        finally:
+            wsp.close()
+            w.close()
+    for case in range(20):
+        M = int(rng.integers(129, 900))
+        N = int(rng.choice([rng.integers(1, 300), rng.integers(300, 2500)]))
+        K = int(rng.choice([rng.integers(1, 300), rng.integers(300, 3000), rng.integers(3000, 14000)]))
+        B = rng.integers(-127, 128, (K, N)).astype(np.int8)
+        ws = (rng.random(N).astype(np.float32) + 0.5) * 0.01
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        op = ops.W8A8Linear(sess, capi.F32I8F32_DYNAMIC, M, B, ws)
+        try:
+            rc, got = op.run(A)
+            want = oracle.w8a8(A, B, ws)["C"]
+            assert rc == 0 and np.array_equal(_bits32(got), _bits32(want)), (case, M, N, K)
+        finally:
+            op.close()
