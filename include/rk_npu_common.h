@@ -4,7 +4,8 @@
  *
  * This header keeps the caller-visible names and values of the reference's
  * include/rk_npu_common.h:28-37 (error codes), :76-77 (opaque ctx / domain),
- * :126-135 (open / close / domain create / free / id) and :156 (strerror), so
+ * :126-135 (open / close / domain create / free / id), :147-153 (reclaim hook) and :156
+ * (strerror), so
  * code written against the reference links against this library unchanged.
  *
  * What is different underneath: a context owns one HIP device and one HIP
@@ -69,6 +70,19 @@ typedef struct {
 } rk_npu_domain_memory_stats;
 int rk_npu_iommu_domain_memory_stats(const rk_npu_iommu_domain* domain,
                                      rk_npu_domain_memory_stats* stats);
+
+/*
+ * Optional reclaim hook of a domain tag (reference include/rk_npu_common.h:147-153,
+ * src/rk_npu_core.cpp:176-210).  When a device allocation made for this (context, domain id)
+ * reports out-of-memory, the hook is called once and the allocation is tried once more; of
+ * several allocations that fail together only the first runs the hook.  The hook may free
+ * handles of this library but must not create any.  Install or clear it (reclaim == NULL)
+ * while no thread is creating handles in the domain, and keep `cookie` alive while it is
+ * installed.  The hook belongs to the (context, domain id) pair, not to the domain object it
+ * was installed through: freeing that object does not clear it.
+ */
+typedef void (*rk_npu_reclaim_idle_fn)(void* cookie);
+void rk_npu_iommu_domain_set_reclaim(rk_npu_iommu_domain* domain, rk_npu_reclaim_idle_fn reclaim, void* cookie);
 
 /* Fixed English text for a return code (reference include/rk_npu_common.h:156). */
 const char* rk_npu_strerror(int code);

@@ -155,9 +155,12 @@ int rk_npu_hip_profile_end(rk_npu_ctx* ctx, char* names, size_t names_bytes, dou
  * sequence with one submission.  For decode loops, whose kernels are short enough that the
  * per-launch submission cost shows.  Run the sequence once eagerly before capturing it (first
  * use of a kernel may set function attributes); do not call rk_npu_hip_sync, blocking
- * reference calls or allocation calls on the context while capturing.  Rejected input is
- * reported by rk_npu_hip_sync after a replay as after eager calls, provided the sequence was
- * also enqueued eagerly since the previous sync (that registers the workspaces' flags). */
+ * reference calls or allocation calls on the context while capturing.  Rejected input (NaN /
+ * Inf rows, expert ids out of range, negative coefficients) is reported by the next
+ * rk_npu_hip_sync after a replay exactly as after the eager calls: the graph remembers the
+ * workspaces it recorded and every launch registers their flags again.  A graph is launched on
+ * the context it was captured on; free the workspaces it uses only when it is no longer
+ * launched. */
 typedef struct rk_npu_hip_graph rk_npu_hip_graph;
 int rk_npu_hip_capture_begin(rk_npu_ctx* ctx);
 rk_npu_hip_graph* rk_npu_hip_capture_end(rk_npu_ctx* ctx);

@@ -145,8 +145,9 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
  *                expert_ids.
  *
  * Packed record of one INT4 expert, rk_npu_moe_quant_expert_blob_bytes() bytes
- * (0 for W8 handles): {u32 magic "RKHM", u32 RK_NPU_MOE_QUANT_BLOB_VERSION,
- * u32 hidden, u32 intermediate}, the gate/up image (align256(2*intermediate) *
+ * (0 for W8 handles): a 40-byte header {u32 magic "RKH4", u32
+ * RK_NPU_MOE_QUANT_BLOB_VERSION, u32 hidden, u32 intermediate, u32 layout revision (2), u32 0,
+ * u64 gate/up image bytes, u64 down image bytes}, the gate/up image (align256(2*intermediate) *
  * align256(hidden) / 2 bytes) and the down image (align256(hidden) *
  * align256(intermediate) / 2 bytes) in this library's execution layout -- 1 KiB
  * tiles of 32 columns x 64 k, two codes per byte, gate/up column blocks
@@ -155,7 +156,9 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* workspace,
  * RK3588 build's) and identical between the all-INT4 and the mixed bank of one
  * geometry.  export / import accept a larger buffer than the record, reject a
  * shorter one, a W8 handle, the shared int8 expert, an out-of-range slot, a
- * foreign header and non-finite or non-positive scales with RK_NPU_ERR_PARAM;
+ * foreign header (another magic, blob version, geometry, layout revision or image size: records
+ * written by an earlier build of this library, which held the codes as int8 tiles under the
+ * magic "RKHM", are rejected) and non-finite or non-positive scales with RK_NPU_ERR_PARAM;
  * a rejected import leaves the slot unchanged.  Import only between blocking
  * runs that use the bank.  The timed import reports validate_us (header and
  * scale checks), copy_us (scales), gate_sync_us / down_sync_us (the two weight

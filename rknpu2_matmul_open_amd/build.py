@@ -32,13 +32,21 @@ FLAGS = [
 # s_waitcnt by hand: they rely on this compiler not copying or re-using a load's destination
 # register between the load and the wait that covers it.  The kernels were validated (parity
 # suite on an MI355X) with the compiler named here; any other one may schedule differently, so
-# a build with it says so loudly and the parity suite has to be run again before its results
-# are trusted.
+# a build with it is REFUSED unless the caller opts in with RK_NPU_HIP_ALLOW_UNVALIDATED_HIPCC=1,
+# and then says so loudly: the parity suite (`pytest tests -m gpu` on an MI355X) has to be run
+# again before the results of such a build are trusted.  The same holds after any change to
+# those kernels' load / wait sequences.
 VALIDATED_HIPCC = "HIP version: 7.2.26015"
+ALLOW_ENV = "RK_NPU_HIP_ALLOW_UNVALIDATED_HIPCC"
+
+
+class UnvalidatedToolchain(RuntimeError):
+    pass
 
 
 def check_toolchain(hipcc):
-    """Returns the compiler's version line; warns on stderr when it is not the validated one."""
+    """Returns the compiler's version line.  A compiler other than the validated one raises
+    UnvalidatedToolchain, or -- with RK_NPU_HIP_ALLOW_UNVALIDATED_HIPCC=1 -- warns on stderr."""
     try:
         out = subprocess.run([hipcc, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                              text=True, check=False).stdout
@@ -46,10 +54,13 @@ def check_toolchain(hipcc):
         raise RuntimeError("cannot run %s: %s" % (hipcc, e))
     line = next((l.strip() for l in out.splitlines() if l.startswith("HIP version:")), "")
     if not line.startswith(VALIDATED_HIPCC):
-        sys.stderr.write(
-            "\n[build] WARNING: %s reports %r, the inline-assembly load kernels (gemm_wk_kernel,\n"
-            "[build] gemm_stream_kernel) were validated with %r.  Run `pytest tests -m gpu` on an\n"
-            "[build] MI355X before trusting results of this build.\n\n" % (hipcc, line or out[:80], VALIDATED_HIPCC))
+        what = ("%s reports %r, the inline-assembly load kernels (gemm_wk_kernel, gemm_stream_kernel) were "
+                "validated with %r" % (hipcc, line or out[:80], VALIDATED_HIPCC))
+        if os.environ.get(ALLOW_ENV) != "1":
+            raise UnvalidatedToolchain(what + ".  Set %s=1 to build anyway, then run `pytest tests -m gpu` "
+                                       "on an MI355X before trusting the build." % ALLOW_ENV)
+        sys.stderr.write("\n[build] WARNING: %s.\n[build] Run `pytest tests -m gpu` on an MI355X before "
+                         "trusting results of this build.\n\n" % what)
     return line
 
 

@@ -206,6 +206,7 @@ class MoeImportTimings(C.Structure):
 
 
 P = C.c_void_p
+ReclaimIdleFn = C.CFUNCTYPE(None, C.c_void_p)   # rk_npu_reclaim_idle_fn
 _PROTOTYPES = {
     # rk_npu_common.h
     "rk_npu_open": (P, [C.c_char_p]),
@@ -214,6 +215,7 @@ _PROTOTYPES = {
     "rk_npu_iommu_domain_free": (None, [P]),
     "rk_npu_iommu_domain_id": (C.c_uint32, [P]),
     "rk_npu_iommu_domain_memory_stats": (C.c_int, [P, C.POINTER(DomainMemoryStats)]),
+    "rk_npu_iommu_domain_set_reclaim": (None, [P, P, P]),
     "rk_npu_strerror": (C.c_char_p, [C.c_int]),
     # rk_npu_quant_matmul.h
     "rk_npu_matmul_autotune_config_init": (None, [C.POINTER(MatmulAutotuneConfig), C.c_int, C.c_int, C.c_int]),

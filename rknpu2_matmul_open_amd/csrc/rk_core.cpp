@@ -3,6 +3,7 @@
 // (src/rk_npu_core.cpp:98-183: open / close / strerror / domain handles); the
 // GEM / dmabuf half of that file has no equivalent because HBM allocations are
 // private to this library.
+#include <algorithm>
 #include <cerrno>
 #include <cstdlib>
 #include <new>
@@ -11,6 +12,13 @@
 
 #include "rk_host.h"
 #include "rk_npu_hip.h"
+
+// A recorded sequence of launches, and the rejected-input flags of the workspaces it uses.
+struct rk_npu_hip_graph {
+    void* exec = nullptr;
+    rk_npu_ctx* ctx = nullptr;
+    std::vector<int*> flags;
+};
 
 namespace {
 std::atomic<uint64_t> g_next_ctx_id{1};
@@ -24,7 +32,26 @@ int DeviceBuffer::alloc(const Owner& owner, size_t bytes, bool zero) {
     void* p = nullptr;
     // round to whole 32-bit words so the fill kernel can clear it
     const size_t rounded = (bytes + 15) / 16 * 16;
+    auto& domain = owner.ctx->memory[owner.domain_id];
+    const uint64_t epoch = domain.reclaim_epoch.load(std::memory_order_relaxed);
     int rc = rkh_malloc(owner.ctx->device, &p, rounded);
+    if (rc == RKH_ERR_NOMEM) {
+        // Memory pressure: give the domain's reclaim hook one chance to free idle allocations
+        // (reference src/rk_npu_core.cpp:195-240), then try once more.  The hook may free
+        // handles of this library (their release takes no lock held here) but must not allocate.
+        bool reclaimed = false;
+        {
+            std::lock_guard<std::mutex> lock(domain.reclaim_mutex);
+            if (domain.reclaim_epoch.load(std::memory_order_relaxed) != epoch) {
+                reclaimed = true; // another thread's failed allocation already ran the hook
+            } else if (domain.reclaim) {
+                domain.reclaim(domain.reclaim_cookie);
+                domain.reclaim_epoch.fetch_add(1, std::memory_order_relaxed);
+                reclaimed = true;
+            }
+        }
+        if (reclaimed) rc = rkh_malloc(owner.ctx->device, &p, rounded);
+    }
     if (rc) return map_error(rc);
     if (zero) {
         rc = rkh_fill32(owner.ctx->stream, p, 0u, rounded / 4);
@@ -168,9 +195,18 @@ bool consume_device_flag(rk_npu_ctx* ctx, int* flag) {
 }
 void note_pending_flag(rk_npu_ctx* ctx, int* flag) {
     std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+    if (ctx->capturing && std::find(ctx->capture_flags.begin(), ctx->capture_flags.end(), flag) == ctx->capture_flags.end())
+        ctx->capture_flags.push_back(flag);
     for (int* f : ctx->pending_flags)
         if (f == flag) return;
     ctx->pending_flags.push_back(flag);
+}
+void forget_pending_flag(rk_npu_ctx* ctx, int* flag) {
+    std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+    auto drop = [flag](std::vector<int*>& v) { v.erase(std::remove(v.begin(), v.end(), flag), v.end()); };
+    drop(ctx->pending_flags);
+    drop(ctx->capture_flags);
+    for (rk_npu_hip_graph* g : ctx->graphs) drop(g->flags);
 }
 
 int upload(const Owner& owner, DeviceBuffer& dst, const void* src, size_t bytes) {
@@ -181,6 +217,8 @@ int upload(const Owner& owner, DeviceBuffer& dst, const void* src, size_t bytes)
 }
 
 } // namespace rkhost
+
+static void abandon_profile(rk_npu_ctx* ctx); // (defined beside the profile entry points)
 
 extern "C" {
 
@@ -226,7 +264,16 @@ rk_npu_ctx* rk_npu_open(const char* dev) {
 
 void rk_npu_close(rk_npu_ctx* ctx) {
     if (!ctx) return;
+    abandon_profile(ctx); // (a context closed between profile_begin and profile_end)
     rkh_close(ctx->device, ctx->stream);
+    {
+        // graphs that outlive their context only keep their executable; graph_free releases it
+        std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+        for (rk_npu_hip_graph* g : ctx->graphs) {
+            g->ctx = nullptr;
+            g->flags.clear();
+        }
+    }
     delete ctx;
 }
 
@@ -259,6 +306,14 @@ void rk_npu_iommu_domain_free(rk_npu_iommu_domain* domain) { delete domain; }
 
 uint32_t rk_npu_iommu_domain_id(const rk_npu_iommu_domain* domain) {
     return domain ? domain->id : UINT32_MAX;
+}
+
+void rk_npu_iommu_domain_set_reclaim(rk_npu_iommu_domain* domain, rk_npu_reclaim_idle_fn reclaim, void* cookie) {
+    if (!domain || !domain->ctx) return;
+    auto& m = domain->ctx->memory[domain->id];
+    std::lock_guard<std::mutex> lock(m.reclaim_mutex);
+    m.reclaim = reclaim;
+    m.reclaim_cookie = reclaim ? cookie : nullptr;
 }
 
 int rk_npu_iommu_domain_memory_stats(const rk_npu_iommu_domain* domain,
@@ -390,6 +445,26 @@ void profile_marker(void* user, void* stream, const char* kernel) {
 }
 } // namespace
 
+} // extern "C"
+
+// Called by rk_npu_close: a context that is still the profile owner takes the marker down
+// (rkh_set_marker returns once no launch is inside the marker any more), gives the ownership
+// back and releases the events it recorded, so that nothing points at the context afterwards.
+static void abandon_profile(rk_npu_ctx* ctx) {
+    {
+        std::lock_guard<std::mutex> owner(g_profile_owner_mutex);
+        if (g_profile_owner != ctx) return;
+        rkh_set_marker(nullptr, nullptr);
+        g_profile_owner = nullptr;
+    }
+    std::lock_guard<std::mutex> lock(ctx->profile_mutex);
+    ctx->profiling = false;
+    for (auto& m : ctx->profile_marks) rkh_event_destroy(m.event);
+    ctx->profile_marks.clear();
+}
+
+extern "C" {
+
 int rk_npu_hip_profile_begin(rk_npu_ctx* ctx) {
     if (!ctx) return RK_NPU_ERR_PARAM;
     std::lock_guard<std::mutex> owner(g_profile_owner_mutex);
@@ -446,13 +521,16 @@ int rk_npu_hip_profile_end(rk_npu_ctx* ctx, char* names, size_t names_bytes, dou
 }
 
 /* ---- stream capture ---- */
-struct rk_npu_hip_graph {
-    void* exec = nullptr;
-};
 int rk_npu_hip_capture_begin(rk_npu_ctx* ctx) {
     if (!ctx) return RK_NPU_ERR_PARAM;
     std::lock_guard<std::mutex> submit(ctx->submit_mutex);
-    return rkhost::map_error(rkh_capture_begin(ctx->stream));
+    const int rc = rkhost::map_error(rkh_capture_begin(ctx->stream));
+    if (!rc) {
+        std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+        ctx->capturing = true;
+        ctx->capture_flags.clear();
+    }
+    return rc;
 }
 rk_npu_hip_graph* rk_npu_hip_capture_end(rk_npu_ctx* ctx) {
     if (!ctx) return nullptr;
@@ -460,21 +538,40 @@ rk_npu_hip_graph* rk_npu_hip_capture_end(rk_npu_ctx* ctx) {
     std::lock_guard<std::mutex> submit(ctx->submit_mutex);
     void* exec = nullptr;
     const int rc = rkh_capture_end(ctx->stream, &exec); // (always ends the capture, also when g is null)
+    std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+    ctx->capturing = false;
     if (rc || !g) {
+        ctx->capture_flags.clear();
         rkh_graph_destroy(exec);
         delete g;
         return nullptr;
     }
     g->exec = exec;
+    g->ctx = ctx;
+    g->flags.swap(ctx->capture_flags); // the workspaces whose kernels the graph replays
+    ctx->graphs.push_back(g);
     return g;
 }
 int rk_npu_hip_graph_launch(rk_npu_ctx* ctx, rk_npu_hip_graph* graph) {
-    if (!ctx || !graph || !graph->exec) return RK_NPU_ERR_PARAM;
+    if (!ctx || !graph || !graph->exec || graph->ctx != ctx) return RK_NPU_ERR_PARAM;
     std::lock_guard<std::mutex> submit(ctx->submit_mutex);
+    {
+        // A replay can reject input exactly like the eager calls it recorded: the next
+        // rk_npu_hip_sync has to look at the same flags (the sync before took them off the list).
+        std::lock_guard<std::mutex> lock(ctx->pending_mutex);
+        for (int* f : graph->flags)
+            if (std::find(ctx->pending_flags.begin(), ctx->pending_flags.end(), f) == ctx->pending_flags.end())
+                ctx->pending_flags.push_back(f);
+    }
     return rkhost::map_error(rkh_graph_launch(graph->exec, ctx->stream));
 }
 void rk_npu_hip_graph_free(rk_npu_hip_graph* graph) {
     if (!graph) return;
+    if (graph->ctx) {
+        std::lock_guard<std::mutex> lock(graph->ctx->pending_mutex);
+        auto& v = graph->ctx->graphs;
+        v.erase(std::remove(v.begin(), v.end(), graph), v.end());
+    }
     rkh_graph_destroy(graph->exec);
     delete graph;
 }

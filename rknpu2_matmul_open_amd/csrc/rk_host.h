@@ -30,6 +30,14 @@ struct rk_npu_ctx {
     size_t scratch_bytes = 0;
     struct DomainMemory {
         std::atomic<uint64_t> live_bytes{0}, peak_bytes{0}, creates{0}, destroys{0};
+        // Reclaim hook of the domain tag (rk_npu_iommu_domain_set_reclaim): called once when a
+        // device allocation for this tag reports out-of-memory, after which the allocation is
+        // tried once more.  `reclaim_epoch` counts completed calls, so that of several
+        // allocations failing together only the first one runs the hook.
+        std::mutex reclaim_mutex;
+        rk_npu_reclaim_idle_fn reclaim = nullptr;
+        void* reclaim_cookie = nullptr;
+        std::atomic<uint64_t> reclaim_epoch{0};
     } memory[RK_NPU_IOMMU_DOMAIN_COUNT];
     // Device work of one context is issued on one stream; submissions from
     // different workspaces are serialised here so stream order == call order.
@@ -47,6 +55,13 @@ struct rk_npu_ctx {
     // points since the last rk_npu_hip_sync().
     std::mutex pending_mutex;
     std::vector<int*> pending_flags;
+    // Stream capture (rk_npu_hip_capture_begin / _end): the flags noted while capturing are kept
+    // with the graph, whose every launch registers them again -- a replay runs the same kernels
+    // and can reject input like the eager call did.  `graphs` lists the live graphs of this
+    // context so that a workspace being freed can take its flag out of them.
+    bool capturing = false;
+    std::vector<int*> capture_flags;
+    std::vector<struct rk_npu_hip_graph*> graphs;
 };
 
 struct rk_npu_iommu_domain {
@@ -204,6 +219,8 @@ private:
 // Blocking check of one raw device flag (used by rk_npu_hip_sync).
 bool consume_device_flag(rk_npu_ctx* ctx, int* flag);
 void note_pending_flag(rk_npu_ctx* ctx, int* flag);
+// A workspace that owns `flag` is going away: no later sync or graph launch may read it.
+void forget_pending_flag(rk_npu_ctx* ctx, int* flag);
 
 // Raw upload of a host array into a fresh device buffer (used at weights_create).
 int upload(const Owner& owner, DeviceBuffer& dst, const void* src, size_t bytes);

@@ -25,7 +25,9 @@
 #include <float.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <atomic>
 #include <mutex>
+#include <shared_mutex>
 #include <type_traits>
 
 #include "rk_hip_shim.h"
@@ -46,9 +48,17 @@ namespace {
 // Stage marker (see rkh_set_marker): told the name of every kernel launched through this
 // file just before the launch, so that a caller can put stream events between the kernels
 // of a multi-kernel step.  Null unless a caller is profiling.
+// Launches come from any thread: the pair is read under a shared lock, which rkh_set_marker
+// takes exclusively -- so once it has returned, no thread is inside the old marker or about
+// to call it with the old user pointer.  `g_marker_on` keeps the lock off the path of every
+// launch while nobody profiles.
+std::shared_mutex g_marker_mutex;
+std::atomic<bool> g_marker_on{false};
 rkh_marker_fn g_marker = nullptr;
 void* g_marker_user = nullptr;
 inline void mark(hipStream_t stream, const char* kernel) {
+    if (!g_marker_on.load(std::memory_order_acquire)) return;
+    std::shared_lock<std::shared_mutex> lock(g_marker_mutex);
     if (g_marker) g_marker(g_marker_user, stream, kernel);
 }
 
@@ -2974,14 +2984,16 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
 #define RK_WK(W4, EPI)                                                                              \
     do {                                                                                            \
         /* the LDS opt-in is per function and per device: once for each device this process uses */ \
-        static bool opted_in[64] = {};                                                              \
+        /* (several threads may get here together: setting the attribute twice is harmless, and the  \
+           flag is only set once a call has succeeded) */                                           \
+        static std::atomic<bool> opted_in[64] = {};                                                 \
         int dev = 0;                                                                                \
         RKH_CHECK(hipGetDevice(&dev));                                                              \
         if (dev < 0 || dev >= 64) return RKH_ERR_RUNTIME;                                           \
-        if (!opted_in[dev]) {                                                                       \
+        if (!opted_in[dev].load(std::memory_order_acquire)) {                                       \
             RKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wk_kernel<TM, W4, EPI>), \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES)); \
-            opted_in[dev] = true;                                                                   \
+            opted_in[dev].store(true, std::memory_order_release);                                   \
         }                                                                                           \
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI>), grid, block, WK_LDS_BYTES, st,           \
                            g.A, g.W, g.M, g.K, mblocks, nblocks, ksplit, per, g);                   \
@@ -3029,6 +3041,9 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : fuse->in_dtype == RKH_F32 ? 2 : 3;
     if (qt == 3 && g.w_int4) return RKH_ERR_RUNTIME; // (gemv_can_fuse lets int8 rows through for int8 weights only)
+    // the instantiation that reads rows must have rows to read, the other one quantized rows
+    if (qt ? !q.src : !g.A) return RKH_ERR_RUNTIME;
+    if (!g.W || !g.C) return RKH_ERR_RUNTIME;
     const char* label = qt == 3 ? "gemv_kernel (int8 rows)" : qt ? "gemv_kernel (fused quantize)" : "gemv_kernel";
     if (MR == 1 && !g.w_int4 && cw == 32) { // (the burst variant, see gemv_kernel)
         mark(st, qt == 3 ? "gemv_kernel<burst> (int8 rows)" : qt ? "gemv_kernel<burst> (fused quantize)" : "gemv_kernel<burst>");
@@ -3063,6 +3078,8 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
     const dim3 grid(g.interleave_F / 32), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+    if (qt ? !q.src : !g.A) return RKH_ERR_RUNTIME; // (rows to read for the instantiation that is launched)
+    if (!g.W || !g.C) return RKH_ERR_RUNTIME;
     mark(st, qt ? "gemv_swiglu_kernel (fused quantize)" : "gemv_swiglu_kernel");
 #define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q)
     // (dense SwiGLU exists for int4 weights only, with rows as fp32 or already quantized:
@@ -3183,8 +3200,10 @@ int rkh_debug_set_ts(void* device_buffer) {
 #endif
 
 void rkh_set_marker(rkh_marker_fn fn, void* user) {
-    g_marker_user = user;
+    std::unique_lock<std::shared_mutex> lock(g_marker_mutex);
     g_marker = fn;
+    g_marker_user = fn ? user : nullptr;
+    g_marker_on.store(fn != nullptr, std::memory_order_release);
 }
 
 int rkh_malloc(int device, void** ptr, size_t bytes) {

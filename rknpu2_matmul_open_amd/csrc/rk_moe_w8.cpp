@@ -120,11 +120,7 @@ struct rk_npu_moe_w8_workspace {
                h_scale.bytes() + y.bytes() + out.bytes();
     }
     ~rk_npu_moe_w8_workspace() {
-        if (owner.ctx) {
-            std::lock_guard<std::mutex> lock(owner.ctx->pending_mutex);
-            auto& v = owner.ctx->pending_flags;
-            v.erase(std::remove(v.begin(), v.end(), flag.device()), v.end());
-        }
+        if (owner.ctx) rkhost::forget_pending_flag(owner.ctx, flag.device());
     }
 };
 
@@ -621,10 +617,19 @@ namespace {
 // this library and are not interchangeable with the reference's (its records
 // hold NPU tile images).  Every byte of an image is two valid codes, so a record
 // cannot smuggle a value outside [-8, 7] into a slot.
+// `layout` is this library's own revision of the image layout, beside the API's blob version:
+// it changes whenever the bytes of an image mean something else (revision 1 held the codes as
+// int8 tiles padded to 64 k, under the magic "RKHM" and a 16-byte header; revision 2 holds
+// packed nibbles padded to 256 k).  Every byte of an image is valid codes in any layout, so
+// nothing but the header can tell a record of another revision apart: import checks the magic,
+// both versions and the two image sizes before it touches a slot.
 struct RecordHeader {
     uint32_t magic, version, hidden, intermediate;
+    uint32_t layout, reserved;
+    uint64_t gate_bytes, down_bytes;
 };
-constexpr uint32_t kRecordMagic = 0x4d484b52u; // "RKHM"
+constexpr uint32_t kRecordMagic = 0x34484b52u; // "RKH4"
+constexpr uint32_t kRecordLayout = 2;
 
 uint64_t record_bytes(const rk_npu_moe_w8_weights* w) {
     return sizeof(RecordHeader) + w->gate_stride4 + w->down_stride4 +
@@ -649,7 +654,8 @@ int rk_npu_moe_quant_export_expert(const rk_npu_moe_w8_weights* w, int e, void* 
     const int H = w->config.hidden, I = w->config.intermediate;
     rk_npu_ctx* ctx = w->owner.ctx;
     uint8_t* p = static_cast<uint8_t*>(data);
-    const RecordHeader header{kRecordMagic, RK_NPU_MOE_QUANT_BLOB_VERSION, (uint32_t)H, (uint32_t)I};
+    const RecordHeader header{kRecordMagic, RK_NPU_MOE_QUANT_BLOB_VERSION, (uint32_t)H, (uint32_t)I,
+                              kRecordLayout, 0u, (uint64_t)w->gate_stride4, (uint64_t)w->down_stride4};
     std::memcpy(p, &header, sizeof(header));
     p += sizeof(header);
     std::lock_guard<std::mutex> lock(ctx->submit_mutex);
@@ -688,7 +694,9 @@ int rk_npu_moe_quant_import_expert_timed(rk_npu_moe_w8_weights* w, int slot, con
     const uint8_t* down_scales = gate_scales + (size_t)2 * I * sizeof(float);
     auto at = Clock::now();
     bool ok = header.magic == kRecordMagic && header.version == RK_NPU_MOE_QUANT_BLOB_VERSION &&
-              header.hidden == (uint32_t)H && header.intermediate == (uint32_t)I;
+              header.hidden == (uint32_t)H && header.intermediate == (uint32_t)I &&
+              header.layout == kRecordLayout && header.gate_bytes == (uint64_t)w->gate_stride4 &&
+              header.down_bytes == (uint64_t)w->down_stride4;
     if (ok) {
         std::vector<float> scales((size_t)2 * I + H); // the record need not be aligned for float access
         std::memcpy(scales.data(), gate_scales, scales.size() * sizeof(float));

@@ -406,8 +406,12 @@ int rk_npu_f16i8f16_run_dynamic_noalloc_device(const rk_npu_f16i8f16_weights* we
     auto round256 = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t scale_bytes = round256((size_t)rkh_align_up(M, RKH_ROW_ALIGN) * sizeof(float));
     const size_t tiled_bytes = round256(rkh_tiled_i8_bytes(M, w->K, RKH_ROW_ALIGN));
-    const size_t split_bytes = round256(splitk_scratch_bytes(M, w->N, w->K, false));
-    if (scale_bytes + tiled_bytes + split_bytes > ctx->scratch_bytes) return RK_NPU_ERR_NOMEM;
+    // The K split over workgroups is an optimisation, not a need: without room for its int32
+    // partial tiles the GEMM runs unsplit (integer sums: the same bits either way), so only rows
+    // that do not fit by themselves are refused.
+    size_t split_bytes = round256(splitk_scratch_bytes(M, w->N, w->K, false));
+    if (scale_bytes + tiled_bytes > ctx->scratch_bytes) return RK_NPU_ERR_NOMEM;
+    if (scale_bytes + tiled_bytes + split_bytes > ctx->scratch_bytes) split_bytes = 0;
     uint8_t* base = static_cast<uint8_t*>(ctx->scratch);
     rkh_quant_args q{};
     q.src = A;

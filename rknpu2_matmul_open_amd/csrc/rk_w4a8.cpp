@@ -238,11 +238,7 @@ struct rk_npu_w4a8_workspace {
     BadFlag flag;
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     ~rk_npu_w4a8_workspace() {
-        if (owner.ctx) {
-            std::lock_guard<std::mutex> lock(owner.ctx->pending_mutex);
-            auto& v = owner.ctx->pending_flags;
-            v.erase(std::remove(v.begin(), v.end(), flag.device()), v.end());
-        }
+        if (owner.ctx) rkhost::forget_pending_flag(owner.ctx, flag.device());
     }
 };
 

@@ -420,17 +420,23 @@ def test_i4_host_side(lib):
     lib.rk_npu_i4_workspace_free(None)
 
 
-def test_build_names_the_compiler_it_was_validated_with(tmp_path, capsys):
+def test_build_refuses_a_compiler_it_was_not_validated_with(tmp_path, capsys, monkeypatch):
     """The inline-assembly load kernels depend on how one hipcc schedules around hand-placed
-    waits: the build records that compiler's version and warns loudly about any other."""
+    waits: the build records that compiler's version, refuses any other, and only builds with
+    it -- warning loudly -- when the caller opts in through the environment."""
     from rknpu2_matmul_open_amd import build
+    monkeypatch.delenv(build.ALLOW_ENV, raising=False)
     line = build.check_toolchain(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"))
-    assert line.startswith("HIP version:")
-    quiet = capsys.readouterr().err
-    assert ("WARNING" in quiet) == (not line.startswith(build.VALIDATED_HIPCC))
+    assert line.startswith(build.VALIDATED_HIPCC)       # this image's compiler is the validated one
+    assert "WARNING" not in capsys.readouterr().err
     other = tmp_path / "hipcc"
     other.write_text("#!/bin/sh\necho 'HIP version: 9.9.99999-deadbeef'\n")
     other.chmod(0o755)
+    with pytest.raises(build.UnvalidatedToolchain) as refused:
+        build.check_toolchain(str(other))
+    assert "gemm_wk_kernel" in str(refused.value) and build.VALIDATED_HIPCC in str(refused.value)
+    assert build.ALLOW_ENV in str(refused.value)
+    monkeypatch.setenv(build.ALLOW_ENV, "1")
     assert build.check_toolchain(str(other)) == "HIP version: 9.9.99999-deadbeef"
     err = capsys.readouterr().err
     assert "WARNING" in err and "gemm_wk_kernel" in err and build.VALIDATED_HIPCC in err

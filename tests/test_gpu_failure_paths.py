@@ -50,6 +50,65 @@ def _drive(sess, create):
     raise AssertionError("constructor never succeeded")
 
 
+def test_reclaim_hook_runs_once_and_the_allocation_is_retried(sess, oracle):
+    """rk_npu_iommu_domain_set_reclaim (reference include/rk_npu_common.h:147-153): an allocation
+    that reports out-of-memory calls the domain's hook once -- which here frees an idle weights
+    handle -- and is tried again; the constructor then succeeds, and its result is exact.
+    Without a hook the same failure returns NULL."""
+    M, K, N = 3, 200, 96
+    c = workloads.w8a8_case(M, K, N, 0, 1)
+    lib = sess.lib
+    B = np.ascontiguousarray(c["B"], np.int8)
+    wscale = np.ascontiguousarray(c["w_scale"], np.float32)
+    wc = capi.MatmulWeightConfig(K, N, min(K, 2048))
+
+    def create():
+        return lib.rk_npu_f16i8f16_weights_create(sess.domain, C.byref(wc), capi.ptr(B), capi.ptr(wscale))
+
+    idle = create()
+    assert idle
+    base = _live_bytes(sess)
+    calls = []
+
+    def hook(cookie):
+        calls.append(cookie)
+        if idle_box[0]:
+            lib.rk_npu_f16i8f16_weights_free(idle_box[0])
+            idle_box[0] = None
+
+    idle_box = [idle]
+    cb = capi.ReclaimIdleFn(hook)
+    try:
+        lib.rk_npu_iommu_domain_set_reclaim(sess.domain, cb, C.c_void_p(1234))
+        lib.rk_npu_hip_fail_alloc_after(1)
+        w = create()
+        lib.rk_npu_hip_fail_alloc_after(0)
+        assert w, "the allocation was not retried after the hook"
+        assert calls == [1234] and idle_box[0] is None
+        assert _live_bytes(sess) == base   # one handle freed by the hook, one created
+        # a second failure with the hook cleared: plain NULL, no call
+        lib.rk_npu_iommu_domain_set_reclaim(sess.domain, None, None)
+        lib.rk_npu_hip_fail_alloc_after(1)
+        assert not create()
+        lib.rk_npu_hip_fail_alloc_after(0)
+        assert calls == [1234] and _live_bytes(sess) == base
+        # the handle made on the retried allocation computes exactly
+        strategy = ops.default_strategy(capi.F16I8F16_DYNAMIC, M, N, K)
+        ws = lib.rk_npu_matmul_workspace_create(sess.domain, C.byref(strategy))
+        assert ws
+        out = np.empty((M, N), np.uint16)
+        A = np.ascontiguousarray(c["A"])
+        assert lib.rk_npu_f16i8f16_run_dynamic(ws, w, capi.ptr(A), capi.ptr(out)) == 0
+        assert np.array_equal(out, oracle.w8a8(c["A"], c["B"], c["w_scale"])["C"])
+        lib.rk_npu_matmul_workspace_free(ws)
+        lib.rk_npu_f16i8f16_weights_free(w)
+    finally:
+        lib.rk_npu_hip_fail_alloc_after(0)
+        lib.rk_npu_iommu_domain_set_reclaim(sess.domain, None, None)
+        if idle_box[0]:
+            lib.rk_npu_f16i8f16_weights_free(idle_box[0])
+
+
 def test_w8a8_constructors_survive_every_allocation_failure(sess, oracle):
     M, K, N = 40, 300, 200
     c = workloads.w8a8_case(M, K, N, 0, 1)

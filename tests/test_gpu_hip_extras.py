@@ -178,3 +178,104 @@ def test_measurement_probes_run_and_validate_their_arguments(sess):
         assert lib.rk_npu_hip_probe_mfma_i8(sess.ctx, src, 0, C.byref(ops_count)) == capi.RK_NPU_ERR_PARAM
     finally:
         sess.free_device(src)
+
+
+def test_replay_reports_rejected_input_after_an_earlier_sync(sess, oracle):
+    """A decode loop is graph_launch + sync, again and again.  The sync takes the workspaces'
+    rejected-input flags off the context's list, so every launch of the graph has to put them
+    back: input that turns bad between two replays (a NaN token, an expert id out of range, a
+    negative coefficient) must surface as RK_NPU_ERR_PARAM at the sync behind THAT replay, and
+    the replay after it, on good input again, must be clean and exact."""
+    lib = sess.lib
+    T, H, E, top_k, I = 4, 128, 6, 2, 64
+    mc = workloads.moe_case(T, H, E, top_k, I)
+    moe = ops.MoeW8(sess, H, I, E, 0, top_k, 32, mc["experts"])
+    M, K, N = 1, 320, 200
+    rng = np.random.default_rng(5)
+    B4 = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    s4 = (rng.random(N).astype(np.float32) + 0.5) * 0.02
+    w4, ws4 = ops.W4A8Weights(sess, B4, s4), ops.W4A8Workspace(sess, M, N, K)
+    x = np.ascontiguousarray(mc["x"], np.float32)
+    ids, routes = np.ascontiguousarray(mc["ids"], np.int32), np.ascontiguousarray(mc["routes"], np.float32)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    dx, dids, drt, dout = sess.to_device(x), sess.to_device(ids), sess.to_device(routes), sess.empty_device(T * H * 4)
+    dA, dC = sess.to_device(a), sess.empty_device(M * N * 4)
+
+    def enqueue():
+        assert lib.rk_npu_moe_w8_run_f32_device(moe.ws, moe.w, T, dx, dids, drt, dout) == 0
+        assert lib.rk_npu_w4a8_run_f32_device(ws4.h, w4.h, dA, dC) == 0
+
+    def good():
+        _upload(sess, dx, x)
+        _upload(sess, dids, ids)
+        _upload(sess, drt, routes)
+        _upload(sess, dA, a)
+
+    graph = None
+    try:
+        enqueue()
+        assert sess.sync() == 0
+        assert lib.rk_npu_hip_capture_begin(sess.ctx) == 0
+        enqueue()
+        graph = lib.rk_npu_hip_capture_end(sess.ctx)
+        assert graph
+        rc, want = oracle.moe_w8(mc["experts"], H, I, E, 0, top_k, ids, routes, input_f32=x)
+        want4 = oracle.w4a8(a, B4, s4)["C"]
+        assert lib.rk_npu_hip_graph_launch(sess.ctx, graph) == 0
+        assert sess.sync() == 0            # <- from here on no flag is registered by an eager call
+        bad_x = x.copy(); bad_x[2, 7] = np.nan
+        bad_ids = ids.copy(); bad_ids[1, 0] = E + 3
+        bad_routes = routes.copy(); bad_routes[3, 1] = -0.25
+        bad_a = a.copy(); bad_a[0, 11] = np.inf
+        for what, dst, bad in (("NaN token", dx, bad_x), ("expert id", dids, bad_ids),
+                               ("negative coefficient", drt, bad_routes), ("Inf row (w4a8)", dA, bad_a)):
+            _upload(sess, dst, bad)
+            assert lib.rk_npu_hip_graph_launch(sess.ctx, graph) == 0
+            assert sess.sync() == capi.RK_NPU_ERR_PARAM, what
+            good()
+            assert lib.rk_npu_hip_graph_launch(sess.ctx, graph) == 0
+            assert sess.sync() == 0, "clean replay after " + what
+            assert np.array_equal(sess.from_device(dout, (T, H), np.float32).view(np.uint32), want.view(np.uint32))
+            assert np.array_equal(sess.from_device(dC, (M, N), np.float32).view(np.uint32), want4.view(np.uint32))
+        # a workspace freed while the graph lives takes its flag with it: a later sync must not
+        # read freed memory (the graph itself is not launched again)
+        ws4.close()
+        assert sess.sync() == 0
+    finally:
+        if graph:
+            lib.rk_npu_hip_graph_free(graph)
+        for d in (dx, dids, drt, dout, dA, dC):
+            sess.free_device(d)
+        moe.close()
+        ws4.close()
+        w4.close()
+
+
+def test_closing_a_context_that_is_profiling_releases_the_marker(sess):
+    """rk_npu_close between profile_begin and profile_end: the process-wide marker and the
+    profile ownership go with the context, so launches on other contexts do not touch freed
+    memory and another context can profile afterwards."""
+    lib = sess.lib
+    other = ops.Session()
+    M, K, N = 2, 256, 128
+    c = workloads.w8a8_case(M, K, N, 0, 1)
+    lin_other = ops.W8A8Linear(other, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    dA = other.to_device(c["A"])
+    dC = other.empty_device(M * N * 2)
+    assert lib.rk_npu_hip_profile_begin(other.ctx) == 0
+    assert lin_other.run_device(dA, dC) == 0        # records an event owned by `other`
+    other.free_device(dA)
+    other.free_device(dC)
+    lin_other.close()
+    other.close()                                    # still profiling
+    lin = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    dA, dC = sess.to_device(c["A"]), sess.empty_device(M * N * 2)
+    try:
+        assert lin.run_device(dA, dC) == 0           # would call the stale marker
+        assert sess.sync() == 0
+        prof = ops.profile_kernels(sess, lambda: lin.run_device(dA, dC), iters=3)   # not BUSY
+        assert len(prof) == 1
+    finally:
+        sess.free_device(dA)
+        sess.free_device(dC)
+        lin.close()

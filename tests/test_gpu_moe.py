@@ -429,6 +429,16 @@ def test_slot_banks_records_and_slot_exchange(sess, oracle):
         bad = records[0].copy()
         bad[:4] = 0
         assert lib.rk_npu_moe_quant_import_expert(bank.w, slot_of[0], capi.ptr(bad), need) == capi.RK_NPU_ERR_PARAM
+        # a record of the library's earlier layout (magic "RKHM", 16-byte header, int8 tiles): larger
+        # than today's record for the same geometry, so only the header can give it away
+        old = np.zeros(2 * need, np.uint8)
+        old[:16] = np.frombuffer(np.array([0x4d484b52, 3, H, I], np.uint32).tobytes(), np.uint8)
+        old[16:] = 0x11
+        assert lib.rk_npu_moe_quant_import_expert(bank.w, slot_of[0], capi.ptr(old), 2 * need) == capi.RK_NPU_ERR_PARAM
+        for field, value in ((4, 1), (6, 12345), (8, 7)):   # layout revision, gate/up image bytes, down image bytes
+            bad = records[0].copy()
+            bad[4 * field:4 * field + 4] = np.frombuffer(np.uint32(value).tobytes(), np.uint8)
+            assert lib.rk_npu_moe_quant_import_expert(bank.w, slot_of[0], capi.ptr(bad), need) == capi.RK_NPU_ERR_PARAM
         bad = records[0].copy()
         bad[need - 4:need] = np.frombuffer(np.float32(-1.0).tobytes(), np.uint8)   # a negative down scale
         assert lib.rk_npu_moe_quant_import_expert(bank.w, slot_of[0], capi.ptr(bad), need) == capi.RK_NPU_ERR_PARAM

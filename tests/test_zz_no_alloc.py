@@ -41,10 +41,13 @@ def _run_both(sess, oracle, M, N, K, seed):
 
 # (first call, second smaller call): the MFMA kernel with K split over workgroups (partial tiles in
 # the scratch) then a ragged streaming-kernel shape; the large-tile kernel then the fused decode
-# GEMV; a decode GEMV of the benchmark's shape then a ragged two-row one
+# GEMV; a decode GEMV of the benchmark's shape then a ragged two-row one; a shape whose rows fit
+# the array but whose K-split partial tiles would not (12.6 MB of them: the call runs the GEMM
+# unsplit instead of refusing, same bits) then a small one
 PAIRS = [((200, 1024, 4096), (17, 300, 200)),
          ((700, 6900, 1100), (1, 520, 1000)),
-         ((1, 14336, 4096), (2, 700, 3000))]
+         ((1, 14336, 4096), (2, 700, 3000)),
+         ((192, 4096, 4096), (5, 200, 300))]
 
 
 @pytest.mark.parametrize("first,second", PAIRS)
