@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "librk_npu_matmul.so")
-SOURCES = ["rk_kernels.hip", "rk_core.cpp", "rk_quant_matmul.cpp", "rk_autotune.cpp", "rk_w4a8.cpp", "rk_w4a8_tune.cpp", "rk_i4.cpp",
+SOURCES = ["rk_kernels.hip", "rk_kernels_gemv.hip", "rk_kernels_gemm.hip", "rk_kernels_stream.hip", "rk_core.cpp", "rk_quant_matmul.cpp", "rk_autotune.cpp", "rk_w4a8.cpp", "rk_w4a8_tune.cpp", "rk_i4.cpp",
            "rk_moe_w8.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

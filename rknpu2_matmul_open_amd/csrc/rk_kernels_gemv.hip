@@ -1,0 +1,748 @@
+// Decode-sized rows (M <= 8): dot-product kernels, no MFMA.  gemv_kernel (optionally with the
+// per-token quantization in its prologue), gemv_swiglu_kernel (gate/up + SwiGLU of one or two
+// rows) and their launchers.  Bound by HBM.
+#include "rk_kernels_common.h"
+
+namespace {
+
+// ------------------------------------------------------------------ GEMV
+// One workgroup per physical 32-column block; the waves of the group split K
+// (k-tiles interleaved across waves so that neighbouring loads are adjacent in
+// memory); activations sit in LDS; lanes l and l+32 hold the two 16-byte
+// halves of a k-tile for column l%32, so the cross-lane reduction is one xor
+// shuffle, followed by a small LDS reduction across waves.
+#ifndef RK_GEMV_WAVES
+#define RK_GEMV_WAVES 8
+#endif
+#ifndef RK_GEMV_UNROLL
+#define RK_GEMV_UNROLL 8
+#endif
+constexpr int GEMV_WAVES = RK_GEMV_WAVES;
+constexpr int GEMV_UNROLL = RK_GEMV_UNROLL;
+constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
+
+constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
+
+// QT: 0 = activations come quantized from the tiled buffer g.A;
+//     3 = int8 rows as the caller holds them (row-major q.src): staged from there, no launch of
+//     the re-tiling kernel in front;
+//     1 / 2 = fused per-token quantization of fp16 / fp32 rows q.src (every
+//     workgroup quantizes the few rows itself -- they are L2 hits after the first
+//     -- which saves a kernel launch per decode step; workgroup 0 also writes the
+//     scales and the tiled int8 copy that the two-kernel path would have left).
+// Two workgroups must fit a compute unit (a grid of a few hundred workgroups
+// otherwise runs in two rounds), i.e. four waves per SIMD and at most 128
+// vector registers: stated as a requirement, because the int4 variants with the
+// fused quantization would otherwise be allocated more.
+// CW < 32 (narrow matrices, where one workgroup per 32-column block leaves compute
+// units without work -- 128 workgroups for a 4096-column projection): 32 / CW
+// workgroups share a column block, CW = 16 or 8 columns each.  A load instruction
+// then covers the workgroup's part of 32 / CW consecutive k-tiles (pieces of
+// 16 * CW bytes): lane = column % CW + CW * k-half + 2 * CW * (tile of the group),
+// and the cross-lane reduction takes two or three xor-shuffles instead of one.
+//
+// BURST (one int8 row of a wide matrix, more than 256 column blocks -- the decode shape of the
+// benchmark): the loads past the end of K are skipped by branches instead of being sent through
+// the bounds-checked descriptor.  With the branches the compiler no longer counts the
+// outstanding loads exactly and waits for ALL of a wave's loads wherever it needs one of them --
+// so every wave of a workgroup has its whole group of tiles before the quantization prologue
+// starts, passes the prologue's barriers with nothing outstanding, uses the group at once and
+// asks for the next group in one burst together with the other seven waves.  For a matrix that
+// is bound by memory throughput that is the faster order, measured on one box for 4096 x 14336:
+// 11.05 us against 11.5 us with exact waits (11.4 with an explicit wait for the whole group in
+// front of the prologue or of the K loop).  Int4 matrices of the same shape are faster with
+// exact waits (7.8 against 8.3 us).  Since the prologue waits for everything anyway, the weight
+// tiles are requested ahead of the activation rows, a dozen instructions from the kernel's
+// entry instead of behind the row loader's code (in-kernel time stamps: 2.4 us from a wave's
+// start until its weight requests were out; 10.9 -> 10.6 us).  Tried on this variant and slower,
+// same box, against 10.6 us: a second group of tiles requested before the prologue (11.0 us; all
+// 16 loads of a wave requested at the start: 12.2), the wave index read into a scalar register
+// (10.85: the branches around the loads become scalar and the compiler counts the loads exactly
+// again), the column scales of the epilogue fetched with the first loads (10.7), a first group
+// of 4 / 6 / 10 / 12 tiles per wave with the rest in one group behind the prologue (11.8 / 11.1 /
+// 11.0 / 11.6), four tiles per group throughout (11.4), the exact-wait kernel with four loads
+// per wave in flight (10.7), 28 instead of 32 columns per workgroup (512 workgroups, two for
+// every compute unit, instead of 448 -- 11.85 us; the per-lane addresses this needs cost 0.4 us
+// already with 32 columns).
+template <int MR, bool W4, int QT, int CW, bool BURST = false>
+__global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
+void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
+    RK_GEMV_HEAD_APPLY(g, q);
+    RK_TS(0);
+    static_assert(CW == 32 || CW == 16 || CW == 8, "columns per workgroup");
+    constexpr bool FUSEQ = QT == 1 || QT == 2; // the kernel quantizes the rows itself
+    static_assert(QT != 3 || !W4, "int8 rows as given: the exact int8 x int8 product only");
+    // Load instructions of a wave in flight.  One row, exact waits: four -- the quantization
+    // prologue and the first dot products start after half as many bytes, and nothing is gained
+    // by queueing more in front of the memory system (4096 x 14336 int4: 7.25 -> 6.8 us; int4
+    // 4096 x 4096 4.9 -> 4.1, 4096 x 11008 7.0 -> 6.6, 8192 x 1024 5.1 -> 4.5; int8 2048 x 2048
+    // 4.2 -> 3.6, 14336 x 4096 12.8 -> 12.5, the other int8 shapes within 1 %).  Several rows
+    // and the burst variant are faster with eight (two rows lose 2 - 9 % with four on most
+    // shapes; the burst variant 10.6 -> 11.4 us).
+    constexpr int UNR = (MR == 1 && !BURST) ? 4 : GEMV_UNROLL;
+    static_assert(!BURST || (MR == 1 && !W4 && CW == 32), "the burst variant serves one int8 row, whole column blocks");
+    constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
+    // (padding for the single-row variants of narrow matrices: their look-ahead of UNR loads per wave, and
+    // one more step for the activations, runs up to that many load instructions past the end
+    // of a chunk, 32 / CW tiles of 32 -- int4: 64 -- staged bytes each)
+    constexpr bool ROLLING = MR == 1 && CW < 32; // see the K loop
+    constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
+    __shared__ int red[GEMV_WAVES][MR][CW];
+    __shared__ uint32_t row_max[MR];
+    __shared__ float row_scale[MR];
+    const int lane = lane_id(), wave = wave_id();
+    const int half = (lane / CW) & 1;                       // which 16 k of a 32-k tile
+    const int sub = lane / (2 * CW);                        // which tile of the group one load covers
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int p = (int)blockIdx.x / TPL;
+    const int col0 = ((int)blockIdx.x % TPL) * CW;          // first column of the block this workgroup owns
+    const bool first_wg = blockIdx.x == 0;
+    // byte of this lane inside a 1 KiB tile
+    const unsigned lane_byte = (unsigned)((col0 + lane % CW) + 32 * half) * 16u;
+    // chunk of K staged in LDS at a time (multiple of 64)
+    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
+    int acc[MR], acc_lo[MR]; // (int4 weights: the sums of the high and of the low activation digits)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = acc_lo[m] = 0;
+
+    const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
+    const uint8_t* wbase = g.W + (size_t)p * block_bytes;
+    // Weight loads go through a buffer descriptor over this column block: a load whose offset
+    // lies beyond it returns zeros without touching memory, so the loop below needs no branch
+    // around the loads past the end of K -- and without branches the compiler counts the
+    // outstanding loads exactly (it waits for the one it needs, not for all of them).
+    const __amdgpu_buffer_rsrc_t wrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)block_bytes, 0x00020000);
+    auto load_tile = [&](int unit, int units, int first_tile) -> v4i { // `unit` counts this wave's load instructions
+        if constexpr (BURST) {
+            return unit < units ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+                                      wbase + (size_t)(first_tile + unit) * 1024 + lane * 16))
+                                : v4i{0, 0, 0, 0};
+        } else {
+            const unsigned off = unit < units ? (unsigned)(first_tile + unit * TPL + sub) * 1024u + lane_byte : 0xFFFFFFF0u;
+            return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+        }
+    };
+
+    // Fused path: put the first batch of weight loads in flight before the
+    // quantization prologue so that its latency hides behind them.
+    // The activation rows are requested FIRST: loads return in issue order, so
+    // behind the weight loads they would arrive with the last of those, and the
+    // prologue (and with it the second batch of weight loads) would start only
+    // then.  Fetched first they are back after one L2 round trip and the whole
+    // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
+    v4i wpre[UNR];
+    using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
+    typename RowLoader<QT_T>::Raw araw[FUSEQ ? GEMV_QCHUNKS : 1];
+    if constexpr (FUSEQ) {
+        const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
+        if constexpr (BURST) {
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = (int)threadIdx.x + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const QT_T* row = static_cast<const QT_T*>(q.src) + (size_t)m * K;
+                araw[i] = RowLoader<QT_T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!BURST) {
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        RK_TS(4);
+    }
+    if constexpr (FUSEQ) {
+        using T = QT_T;
+        const int t = threadIdx.x;
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+        if (t < MR) row_max[t] = 0u;
+        __syncthreads();
+        RK_TS(5);
+        // (the rows stay in registers as fetched and are converted once per pass:
+        // holding them as floats across the barriers costs the int4 variants their
+        // second workgroup per compute unit)
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                float mx = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    mx = fmaxf(mx, fabsf(v[j]));
+                    bad |= not_finite(v[j]);
+                }
+                // (non-negative floats order like their bits.  For one row, a shuffle reduction per wave
+                // and one atomic per wave instead of 64 on the same address measured slower: 4096 x 14336
+                // int8 10.65 -> 10.7 us, int4 6.8 -> 7.2 us)
+                atomicMax(&row_max[m], __float_as_uint(mx));
+            }
+        }
+        __syncthreads();
+        if (t < g.M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            if (first_wg && q.scale) q.scale[t] = sc;
+        }
+        if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
+        // zero the K padding of the staged rows
+        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) {
+            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
+                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            }
+        }
+        // a_scale of the epilogue comes from LDS in this path
+        RK_TS(1);
+    }
+
+    for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
+        const int kc = min(kc_max, Kp - kc0);
+        // stage activations: row-major [MR][kc] in LDS from the tiled buffer
+        const int chunks = kc >> 4;
+        if (kc0) __syncthreads();
+        if constexpr (QT == 0) {
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks;
+                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
+            }
+        } else if constexpr (QT == 3) {
+            // int8 rows as the caller holds them (row-major, any alignment, K not padded); the first
+            // workgroup also leaves the tiled copy a launch of the re-tiling kernel would have left
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks, gc = (kc0 >> 4) + c;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (m < g.M) {
+                    const int8_t* src = static_cast<const int8_t*>(q.src) + (size_t)m * g.K + (size_t)gc * 16;
+                    if (gc * 16 + 16 <= g.K && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+                        v = *reinterpret_cast<const uint4*>(src);
+                    } else {
+                        uint32_t w[4] = {0, 0, 0, 0};
+                        for (int j = 0; j < 16; ++j)
+                            if (gc * 16 + j < g.K) w[j >> 2] |= (uint32_t)(uint8_t)src[j] << ((j & 3) * 8);
+                        v = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                    if (first_wg && q.dst) store_codes(q.dst + tiled_chunk_offset(m, gc, KB), v);
+                }
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
+            }
+        }
+        __syncthreads();
+
+        // One group = UNR tiles per wave.  Int4: a tile is a 64-deep super-tile.
+        // (counted in load instructions: one of them spans 32 / CW tiles; K is padded to 256 and a
+        // chunk but the last holds a multiple of 4096 k, so the tile count is a multiple of that)
+        const int tiles = (W4 ? kc >> 6 : kc >> 5) / TPL, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
+        auto load_unit = [&](int unit) -> v4i { return load_tile(unit, tiles, tile0); };
+        auto consume_unit = [&](const v4i& wu, int unit) {
+            {
+                // This lane's tile within the chunk.  Past the end of the chunk the weights are
+                // zeros, so whatever the activation read returns does not matter: it lands in the
+                // next row or in the padding behind the last one.
+                const int tt = unit * TPL + sub;
+                if constexpr (!W4) {
+#pragma unroll
+                    for (int m = 0; m < MR; ++m) {
+                        const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                        acc[m] = __builtin_amdgcn_sdot4(av.x, wu.x, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.y, wu.y, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.z, wu.z, acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4(av.w, wu.w, acc[m], false);
+                    }
+                } else {
+                    // (the staged activations of the lane's 16 k of each 32-deep half: digits, see above)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        const int w0 = s ? wu.z : wu.x, w1 = s ? wu.w : wu.y;
+#pragma unroll
+                        for (int m = 0; m < MR; ++m) {
+                            const v4i av = *reinterpret_cast<const v4i*>(
+                                a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                            dot_digits(av, w0, w1, acc[m], acc_lo[m]);
+                        }
+                    }
+                }
+            }
+        };
+        if constexpr (ROLLING) {
+            // A rolling window of UNR loads per wave: as soon as a tile is used, the
+            // register it sat in takes the load of the tile UNR places further on, so the
+            // number of loads in flight does not drain between groups (a workgroup of a narrow
+            // matrix walks a long K alone on its compute unit).  The fused path starts from the
+            // group fetched ahead of the prologue (it has a single K chunk).
+            // The staged activations of a tile are read one step ahead of its use, so that
+            // their LDS latency does not sit between the arrival of a tile and the next load.
+            struct ActTile { v4i a[W4 ? 2 : 1]; };
+            auto read_act = [&](int unit) {
+                const int tt = unit * TPL + sub; // (past the end of the chunk: the next row or the padding)
+                ActTile r;
+                if constexpr (!W4) {
+                    r.a[0] = *reinterpret_cast<const v4i*>(a_lds + (size_t)(tt * 2 + half) * 16);
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        r.a[s] = *reinterpret_cast<const v4i*>(a_lds + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                }
+                return r;
+            };
+            auto dot_tile = [&](const v4i& wu, const ActTile& t) {
+                if constexpr (!W4) {
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].x, wu.x, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].y, wu.y, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].z, wu.z, acc[0], false);
+                    acc[0] = __builtin_amdgcn_sdot4(t.a[0].w, wu.w, acc[0], false);
+                } else {
+                    dot_digits(t.a[0], wu.x, wu.y, acc[0], acc_lo[0]);
+                    dot_digits(t.a[1], wu.z, wu.w, acc[0], acc_lo[0]);
+                }
+            };
+            v4i w[UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                if constexpr (FUSEQ) w[u] = wpre[u];
+                else w[u] = load_unit(wave + u * GEMV_WAVES);
+            }
+            ActTile cur = read_act(wave);
+            for (int tb = wave; tb < tiles; tb += GEMV_WAVES * UNR) {
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    const ActTile nxt = read_act(tb + (u + 1) * GEMV_WAVES);
+                    dot_tile(w[u], cur);
+                    w[u] = load_unit(tb + (UNR + u) * GEMV_WAVES);
+                    // (each load stays behind the use of its register; gathered at the end of the
+                    // iteration, as the scheduler would have them, the window drains every time)
+                    __builtin_amdgcn_sched_barrier(0);
+                    cur = nxt;
+                }
+            }
+        } else {
+            // A group of UNR loads at a time.  Several rows: the rolling window above costs
+            // those variants more registers than two workgroups per compute unit leave.  Wide
+            // matrices: they are bound by memory throughput, not by a workgroup's own latency, and
+            // a workgroup that asks for its next 64 KiB in one go is served faster than one that
+            // trickles the requests out a tile at a time (4096 x 14336, int8: 11.5 against 11.9 us).
+            int tb = wave;
+            if constexpr (FUSEQ) {
+#pragma unroll
+                for (int u = 0; u < UNR; ++u)
+                    if (tb + u * GEMV_WAVES < tiles) consume_unit(wpre[u], tb + u * GEMV_WAVES);
+                tb += GEMV_WAVES * UNR;
+            }
+            for (; tb < tiles; tb += GEMV_WAVES * UNR) {
+                v4i w[UNR];
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) w[u] = load_unit(tb + u * GEMV_WAVES);
+#pragma unroll
+                for (int u = 0; u < UNR; ++u)
+                    if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
+            }
+        }
+    }
+
+    RK_TS(2);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        int v = W4 ? 16 * acc[m] + acc_lo[m] : acc[m];
+        v += __shfl_xor(v, 32);
+        if (CW <= 16) v += __shfl_xor(v, 16);
+        if (CW <= 8) v += __shfl_xor(v, 8);
+        if (lane < CW) red[wave][m][lane] = v;
+    }
+    __syncthreads();
+    static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
+    if ((int)threadIdx.x < MR * CW) {
+        const int m = (int)threadIdx.x / CW, j = (int)threadIdx.x % CW;
+        if (m >= g.M) return;
+        RK_TS(3);
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
+        const int n = block_first_col(p, g.interleave_F) + col0 + j;
+        if (W4 && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
+        if (n < g.N)
+            store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
+                      FUSEQ ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
+                      g.w_scale ? g.w_scale[n] : 1.0f);
+    }
+}
+
+
+// ---- gate/up GEMV with the SwiGLU epilogue (one or two rows, quantized rows in g.A) ----
+// One workgroup per 32 columns of the middle: its gate block (physical block 2j)
+// and its up block (2j + 1) are neighbours in the weight buffer, so the eight
+// waves stream both over their interleaved k-tiles exactly as gemv_kernel streams
+// one, with two accumulators per row.  The epilogue is the one of the GEMM
+// kernels: middle = silu_poly(gate) * up per element, one partial row maximum
+// per (row, 32 columns).  With few rows the SwiGLU GEMM is a weight stream like
+// any decode GEMV; on the MFMA kernel (one 32-row tile, 31 of them padding) the
+// gate/up projection of a 4096 -> 14336 FFN took 14.9 us.
+constexpr int GEMV_SWIGLU_UNROLL = 4; // load instructions per wave and block in flight (two blocks)
+
+// QT as in gemv_kernel: 0 = quantized rows in g.A, 1 / 2 = the kernel quantizes the fp16 / fp32
+// rows q.src itself (same prologue: rows requested first, then the first group of weights).
+template <int MR, bool W4, int QT>
+__global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
+void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
+    RK_GEMV_HEAD_APPLY(g, q);
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES];
+    __shared__ int red[2][GEMV_WAVES][MR][32];
+    __shared__ uint32_t row_max[MR];
+    __shared__ float row_scale[MR];
+    const int lane = lane_id(), wave = wave_id();
+    const int half = lane >> 5;
+    const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
+    const int KB = Kp / 32;
+    const int F = g.interleave_F;
+    const int j = blockIdx.x; // 32-column block of the middle
+    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
+    int acc[2][MR], acc_lo[2][MR]; // (int4 weights: sums of the high / low activation digits, see split_digits)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[b][m] = acc_lo[b][m] = 0;
+
+    const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
+    const uint8_t* wbase = g.W + (size_t)(2 * j) * block_bytes;    // gate block, the up block right behind it
+    // (bounds-checked descriptor over the two blocks: see gemv_kernel)
+    const __amdgpu_buffer_rsrc_t wrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)(2 * block_bytes), 0x00020000);
+    v4i w[2][GEMV_SWIGLU_UNROLL];
+    auto load_group = [&](int tb, int tiles, int tile0) {
+#pragma unroll
+        for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int tt = tb + u * GEMV_WAVES;
+                const unsigned off = tt < tiles ? (unsigned)(b * block_bytes) + (unsigned)(tile0 + tt) * 1024u + (unsigned)lane * 16u
+                                                : 0xFFFFFFF0u;
+                w[b][u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+            }
+    };
+
+    if constexpr (QT != 0) { // (the fused path has a single K chunk: rows fit the staging area)
+        using T = typename std::conditional<QT == 2, float, uint16_t>::type;
+        const int t = threadIdx.x;
+        const bool first_wg = blockIdx.x == 0;
+        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
+        typename RowLoader<T>::Raw araw[GEMV_QCHUNKS];
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                const T* row = static_cast<const T*>(q.src) + (size_t)m * K;
+                araw[i] = RowLoader<T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_group(wave, W4 ? Kp >> 6 : Kp >> 5, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t < MR) row_max[t] = 0u;
+        __syncthreads();
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                float mx = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    mx = fmaxf(mx, fabsf(v[e]));
+                    bad |= not_finite(v[e]);
+                }
+                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
+            }
+        }
+        __syncthreads();
+        if (t < g.M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            if (first_wg && q.scale) q.scale[t] = sc;
+        }
+        if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
+        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) { // zero the K padding
+            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            const int pidx = t + i * GEMV_WAVES * 64;
+            if (pidx < total) {
+                const int m = pidx / nchunks, c = pidx - m * nchunks;
+                float v[16];
+                RowLoader<T>::unpack(araw[i], v);
+                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
+                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
+            }
+        }
+    }
+
+    for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
+        const int kc = min(kc_max, Kp - kc0);
+        const int chunks = kc >> 4;
+        if (kc0) __syncthreads();
+        if constexpr (QT == 0) {
+            for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
+                const int m = idx / chunks, c = idx - m * chunks;
+                const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
+            }
+        }
+        __syncthreads();
+
+        const int tiles = W4 ? kc >> 6 : kc >> 5, tile0 = W4 ? kc0 >> 6 : kc0 >> 5;
+        for (int tb = wave; tb < tiles; tb += GEMV_WAVES * GEMV_SWIGLU_UNROLL) {
+            if (QT == 0 || tb != wave) load_group(tb, tiles, tile0); // (fused: the first group is on its way)
+#pragma unroll
+            for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u) {
+                const int tt = tb + u * GEMV_WAVES;
+                if (tt >= tiles) continue;
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    if constexpr (!W4) {
+#pragma unroll
+                        for (int m = 0; m < MR; ++m) {
+                            const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
+                            acc[b][m] = __builtin_amdgcn_sdot4(av.x, w[b][u].x, acc[b][m], false);
+                            acc[b][m] = __builtin_amdgcn_sdot4(av.y, w[b][u].y, acc[b][m], false);
+                            acc[b][m] = __builtin_amdgcn_sdot4(av.z, w[b][u].z, acc[b][m], false);
+                            acc[b][m] = __builtin_amdgcn_sdot4(av.w, w[b][u].w, acc[b][m], false);
+                        }
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {
+                            const int w0 = s ? w[b][u].z : w[b][u].x, w1 = s ? w[b][u].w : w[b][u].y;
+#pragma unroll
+                            for (int m = 0; m < MR; ++m) {
+                                const v4i av = *reinterpret_cast<const v4i*>(
+                                    a_lds + (size_t)m * kc + (size_t)((tt * 2 + s) * 2 + half) * 16);
+                                dot_digits(av, w0, w1, acc[b][m], acc_lo[b][m]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            int v = W4 ? 16 * acc[b][m] + acc_lo[b][m] : acc[b][m];
+            v += __shfl_xor(v, 32);
+            if (lane < 32) red[b][wave][m][lane] = v;
+        }
+    __syncthreads();
+    static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
+    if ((int)threadIdx.x < MR * 32) { // a row of 32 columns per half wave
+        const int m = (int)threadIdx.x >> 5, c = (int)threadIdx.x & 31;
+        const int n = j * 32 + c;
+        const bool live = m < g.M && n < F;
+        int gate = 0, up = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) {
+            gate += red[0][w][m][c];
+            up += red[1][w][m][c];
+        }
+        uint32_t bits = 0;
+        if (live) {
+            if (W4) { // (the constant term of the digit split)
+                gate += 8 * g.w_colsum[n];
+                up += 8 * g.w_colsum[F + n];
+            }
+            const float as = QT != 0 ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f);
+            const float gf = dequant(gate, as, g.w_scale ? g.w_scale[n] : 1.0f);
+            const float uf = dequant(up, as, g.w_scale ? g.w_scale[F + n] : 1.0f);
+            const float y = __fmul_rn(silu_poly(gf), uf);
+            static_cast<float*>(g.C)[(size_t)m * g.ldc + n] = y;
+            bits = __float_as_uint(y) & 0x7fffffffu;
+        }
+#pragma unroll
+        for (int d = 16; d > 0; d >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, d));
+        if (g.row_max_bits && c == 0 && m < g.M) g.row_max_bits[(size_t)m * (F / 32) + j] = bits;
+    }
+}
+
+
+template <int MR>
+int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    const int pblocks = (int)(rkh_align_up(g.N, 32) / 32);
+    // Narrow matrices: several workgroups per column block (16 columns each up to 256 blocks =
+    // 8192 columns, 8 columns each up to 64 blocks), so that a 4096-column projection has a
+    // workgroup for every compute unit; all of them still run at once.  (Measured per shape on
+    // one box, M = 1, int8 / int4 us: 4096 x 4096: 7.7 / 6.1 with 32 columns, 6.6 / 5.5 with 16,
+    // 6.9 / 6.0 with 8; 14336 x 4096: 16.6 / 12.3, 14.5 / 10.5, 13.7 / 11.3; 8192 x 1024:
+    // 10.6 / 8.1, 7.9 / 6.4, 6.4 / 5.7; a 14336-column matrix loses a quarter with 16.)
+    // (RK_NPU_HIP_GEMV_COLS = 8 / 16 / 32 forces the choice: tuning aid)
+    static const char* forced = getenv("RK_NPU_HIP_GEMV_COLS");
+    const int want = forced ? atoi(forced) : 0;
+    // Beyond 256 blocks: whole blocks -- unless the rows come as int8 (no quantization prologue that every
+    // workgroup repeats) and halves leave the fullest compute unit with fewer columns: 344 blocks, an
+    // 11008-column projection, 2 x 32 against 3 x 16 columns, one row 10.1 -> 9.3 us, four rows
+    // 12.3 -> 10.9.  (448 blocks: 2 x 32 = 4 x 16, and whole blocks are a quarter faster.  With the
+    // quantization fused, halves cost the same 344-block matrix 6 % to 18 % for 2 to 8 rows.)
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    const bool halves = fuse && fuse->in_dtype == RKH_I8 &&
+                        ((2 * pblocks + cus - 1) / cus) * 16 < ((pblocks + cus - 1) / cus) * 32;
+    const int cw = want == 8 || want == 16 || want == 32 ? want : pblocks <= 64 ? 8 : pblocks <= 256 || halves ? 16 : 32;
+    const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);
+    const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
+    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : fuse->in_dtype == RKH_F32 ? 2 : 3;
+    if (qt == 3 && g.w_int4) return RKH_ERR_RUNTIME; // (gemv_can_fuse lets int8 rows through for int8 weights only)
+    // the instantiation that reads rows must have rows to read, the other one quantized rows
+    if (qt ? !q.src : !g.A) return RKH_ERR_RUNTIME;
+    if (!g.W || !g.C) return RKH_ERR_RUNTIME;
+    const char* label = qt == 3 ? "gemv_kernel (int8 rows)" : qt ? "gemv_kernel (fused quantize)" : "gemv_kernel";
+    if (MR == 1 && !g.w_int4 && cw == 32) { // (the burst variant, see gemv_kernel)
+        mark(st, qt == 3 ? "gemv_kernel<burst> (int8 rows)" : qt ? "gemv_kernel<burst> (fused quantize)" : "gemv_kernel<burst>");
+        if (qt == 0) hipLaunchKernelGGL((gemv_kernel<1, false, 0, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else if (qt == 1) hipLaunchKernelGGL((gemv_kernel<1, false, 1, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else if (qt == 2) hipLaunchKernelGGL((gemv_kernel<1, false, 2, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        else hipLaunchKernelGGL((gemv_kernel<1, false, 3, 32, true>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);
+        RKH_CHECK(hipGetLastError());
+        return RKH_OK;
+    }
+    mark(st, label);
+#define RK_GEMV(W4, QT)                                                                        \
+    do {                                                                                       \
+        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
+        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q); \
+        else if constexpr (!(MR == 1 && !W4)) /* (one int8 row, 32 columns: the burst variant above) */   \
+            hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
+    } while (0)
+    if (g.w_int4) {
+        if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
+    } else {
+        if (qt == 0) RK_GEMV(false, 0); else if (qt == 1) RK_GEMV(false, 1); else if (qt == 2) RK_GEMV(false, 2);
+        else RK_GEMV(false, 3);
+    }
+#undef RK_GEMV
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+template <int MR>
+int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    const dim3 grid(g.interleave_F / 32), block(GEMV_WAVES * 64);
+    const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
+    const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : 2;
+    if (qt ? !q.src : !g.A) return RKH_ERR_RUNTIME; // (rows to read for the instantiation that is launched)
+    if (!g.W || !g.C) return RKH_ERR_RUNTIME;
+    mark(st, qt ? "gemv_swiglu_kernel (fused quantize)" : "gemv_swiglu_kernel");
+#define RK_SWI(W4, QT) hipLaunchKernelGGL((gemv_swiglu_kernel<MR, W4, QT>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q)
+    // (dense SwiGLU exists for int4 weights only, with rows as fp32 or already quantized:
+    // the w4a8 interface has no other call, and gemv_swiglu_applies lets nothing else through)
+    if (!g.w_int4 || qt == 1) return RKH_ERR_RUNTIME;
+    if (qt == 0) RK_SWI(true, 0); else RK_SWI(true, 2);
+#undef RK_SWI
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
+// gate/up + SwiGLU of one or two rows as a GEMV (columns gate/up interleaved in blocks of 32,
+// F a multiple of 32, both blocks of a workgroup within the 4 GiB reach of its descriptor).
+// Measured for 4096 -> 2 x 14336 int4 against 14.9 us on the MFMA kernel: 12.8 us for one row,
+// 13.8 for two, 15.1 for four, 20.1 for eight -- so from three rows on the MFMA kernel keeps it
+// (also when the GEMV could quantize the rows itself and save that launch: a whole 4096 -> 14336
+// -> 4096 FFN of three / four rows took 33.6 / 34.8 us that way against 34.6 / 34.5).
+bool gemv_swiglu_applies(const rkh_gemm_args& g) {
+    return !g.blk_expert && g.w_int4 && g.M <= 2 && g.epilogue == RKH_EPI_SWIGLU && g.interleave_F >= 32 &&
+           g.interleave_F % 32 == 0 && g.N == 2 * g.interleave_F && g.K <= (1 << 24);
+}
+
+int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    if (g.M == 1) return launch_gemv_swiglu<1>(st, g, fuse);
+    return launch_gemv_swiglu<2>(st, g, fuse);
+}
+
+int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
+    if (g.M == 1) return launch_gemv<1>(st, g, fuse);
+    if (g.M == 2) return launch_gemv<2>(st, g, fuse);
+    if (g.M <= 4) return launch_gemv<4>(st, g, fuse);
+    return launch_gemv<8>(st, g, fuse);
+}
+
+// The decode path can quantize inside the GEMV when the rows fit the kernel's
+// LDS staging and per-thread register cache.
+// Whether the streaming MFMA kernel can take this dense GEMM at all (int4 codes ride as 16 * code).
+bool dense_stream_fits(const rkh_gemm_args& g) { return !g.w_int4 || g.K <= 131072; }
+
+// Most rows the dot-product kernels take for this matrix: eight, but four on a matrix of more than
+// 256 column blocks, where five to eight rows are faster as one 32-row block of the streaming MFMA
+// kernel behind a quantization launch (fp16 rows, every step from HBM, dot products against
+// stream, us: 4096 x 11008 int8 17.2 - 20.5 against 15.3 - 15.5, int4 15.5 - 18.9 against 12.3 - 12.5;
+// 4096 x 14336 18.8 - 21.9 against 16.2 - 16.5, int4 16.1 - 19.3 against 12.8 - 12.9; on narrower
+// matrices the dot products win: 4096 x 4096 9.5 - 11.6 against 13.6, 11008 x 4096 22.6 against 27.3;
+// up to four rows they win everywhere).  RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
+int gemv_max_rows(const rkh_gemm_args& g) {
+    static const int rows = [] {
+        const char* e = getenv("RK_NPU_HIP_GEMV_MAX_ROWS");
+        const int v = e ? atoi(e) : 8;
+        return v >= 1 && v <= 8 ? v : 8;
+    }();
+    const bool wide = (g.N + 31) / 32 > 256;
+    return wide && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
+}
+
+bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
+    if (g.w_int4 && !g.w_colsum) return false;
+    if (g.blk_expert || g.M > gemv_max_rows(g) || (g.epilogue == RKH_EPI_SWIGLU) != swiglu || q.src_is_host) return false;
+    // int8 rows as given (the exact int8 x int8 product): staged by the kernel in K chunks, any K
+    if (q.in_dtype == RKH_I8) return q.mode == RKH_Q_COPY_I8 && !g.w_int4 && !swiglu;
+    if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
+    if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
+    const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
+    const long kp = (long)rkh_align_up(g.K, RKH_K_ALIGN);
+    if (kp * mr > GEMV_LDS_BYTES) return false;
+    const long chunks = (long)g.M * ((g.K + 15) / 16);
+    return chunks <= (long)GEMV_QCHUNKS * GEMV_WAVES * 64;
+}
+
+} // namespace
+
+namespace rkk {
+bool gemv_swiglu_applies(const rkh_gemm_args& g) { return ::gemv_swiglu_applies(g); }
+int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) { return ::dispatch_gemv_swiglu(st, g, fuse); }
+int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) { return ::dispatch_gemv(st, g, fuse); }
+bool dense_stream_fits(const rkh_gemm_args& g) { return ::dense_stream_fits(g); }
+int gemv_max_rows(const rkh_gemm_args& g) { return ::gemv_max_rows(g); }
+bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu) { return ::gemv_can_fuse(q, g, swiglu); }
+#ifdef RK_DEBUG_TS
+void set_ts_gemv(unsigned long long* p) { (void)hipMemcpyToSymbol(HIP_SYMBOL(rk_dbg_ts), &p, sizeof(p)); }
+#endif
+} // namespace rkk
