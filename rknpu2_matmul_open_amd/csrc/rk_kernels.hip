@@ -181,16 +181,31 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
         // int8 input is re-tiled byte for byte (the full range -128..127 is legal
         // for the raw integer operator)
         const int8_t* brow = reinterpret_cast<const int8_t*>(row);
-        for (int c = chunk0 + t; c < nchunks; c += 256) {
-            uint32_t w[4] = {0, 0, 0, 0};
-            if (vec && c * 16 + 16 <= K) {
-                const uint4 v4 = *reinterpret_cast<const uint4*>(brow + c * 16);
-                w[0] = v4.x; w[1] = v4.y; w[2] = v4.z; w[3] = v4.w;
-            } else {
-                for (int j = 0; j < 16; ++j)
-                    if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
+        // (four chunks are fetched before the first is stored: the store is an asm statement the
+        // compiler keeps every load behind, and a thread that alternates load and store pays one
+        // memory latency per chunk)
+        for (int c0 = chunk0 + t; c0 < nchunks; c0 += 4 * 256) {
+            uint4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = c0 + i * 256;
+                uint32_t w[4] = {0, 0, 0, 0};
+                if (c < nchunks) {
+                    if (vec && c * 16 + 16 <= K) {
+                        const uint4 v4 = *reinterpret_cast<const uint4*>(brow + c * 16);
+                        w[0] = v4.x; w[1] = v4.y; w[2] = v4.z; w[3] = v4.w;
+                    } else {
+                        for (int j = 0; j < 16; ++j)
+                            if (c * 16 + j < K) w[j >> 2] |= (uint32_t)(uint8_t)brow[c * 16 + j] << ((j & 3) * 8);
+                    }
+                }
+                v[i] = make_uint4(w[0], w[1], w[2], w[3]);
             }
-            store_codes(a.dst + tiled_chunk_offset(m, c, KB), make_uint4(w[0], w[1], w[2], w[3]));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = c0 + i * 256;
+                if (c < nchunks) store_codes(a.dst + tiled_chunk_offset(m, c, KB), v[i]);
+            }
         }
         return;
     }

@@ -265,18 +265,14 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         if constexpr ((SLOT + 1) % G == 0) asm volatile("s_barrier" ::: "memory");
     };
 
-    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
-#pragma unroll
-    for (int t = -D; t < 0; ++t) {
-        copy_a(t + D);
-        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
-    }
-    RK_TS(1);
-    // The tile's scales are fetched now, behind the prologue's loads, and handed
+    // The tile's scales are requested now, ahead of the prologue's loads, and handed
     // to the epilogue through LDS after the loop, so the epilogue does not start
     // with a round trip to memory: thread t holds the row scale of row t
-    // (t < BM) and the column scale of physical column t (t < 256).  (Two more
-    // loads in the queue only make the first sub-steps' waits stricter.)
+    // (t < BM) and the column scale of physical column t (t < 256).  They are the
+    // oldest loads of the wave, so the first wait below covers them (loads return
+    // in issue order) -- and only behind that wait do the two values become, for
+    // the compiler, the long-lived values the epilogue uses: whatever it does with
+    // them from there on (a copy, a spill) moves data that has arrived.
     float my_as = 0.0f, my_ws = 0.0f;
     bool as_valid = false, ws_valid = false;
     if constexpr (EPI != RKH_EPI_I32) {
@@ -301,7 +297,15 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
     }
+    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
+#pragma unroll
+    for (int t = -D; t < 0; ++t) {
+        copy_a(t + D);
+        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
+    }
+    RK_TS(1);
     w_wait(wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
+    asm volatile("" : "+v"(my_as), "+v"(my_ws)); // (landed: see above)
     asm volatile("s_barrier" ::: "memory");
     static_for<4>([&](auto f_tag) { read_frag(afr[0][decltype(f_tag)::value], std::integral_constant<int, 0>{}, f_tag); });
     static_for<NWREG>([&](auto e_tag) { unpack_item(wop[0], wring[0], e_tag); });

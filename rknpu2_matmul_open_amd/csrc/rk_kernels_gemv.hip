@@ -86,6 +86,11 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // one more step for the activations, runs up to that many load instructions past the end
     // of a chunk, 32 / CW tiles of 32 -- int4: 64 -- staged bytes each)
     constexpr bool ROLLING = MR == 1 && CW < 32; // see the K loop
+    // Several rows, int8 weights: the group of loads is kept as two halves, see the K loop.  (Measured
+    // per shape against the whole group at a time, fp16 rows, us: 4096 x 14336 two / four rows 11.85 ->
+    // 11.7 / 13.85 -> 13.2; 14336 x 4096 16.1 -> 14.9 / 22.9 -> 21.4; 4096 x 4096 within 1 %; int4
+    // weights lose with two rows, 8.5 -> 9.3 and 5.35 -> 5.6, and keep the whole group.)
+    constexpr bool PINGPONG = MR > 1 && !W4;
     constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
     __shared__ int red[GEMV_WAVES][MR][CW];
@@ -234,8 +239,14 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
             }
         } else if constexpr (QT == 3) {
-            // int8 rows as the caller holds them (row-major, any alignment, K not padded); the first
-            // workgroup also leaves the tiled copy a launch of the re-tiling kernel would have left
+            // int8 rows as the caller holds them (row-major, any alignment, K not padded).  The tiled
+            // copy a launch of the re-tiling kernel would have left is written on the side, every
+            // workgroup storing an equal contiguous share of its chunks: when the first
+            // workgroup wrote all of it (write-through stores between its loads), that workgroup
+            // finished 2 - 4 us after the others and the launch with it -- four rows took 7.4 us
+            // where one took 5.2 (4096 x 4096) and 15.1 where one took 10.0 (11008 x 4096).
+            const unsigned copy_share = ((unsigned)g.M * (unsigned)(Kp >> 4) + gridDim.x - 1) / gridDim.x;
+            const unsigned copy_lo = blockIdx.x * copy_share; // this workgroup's chunks of the tiled copy
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
                 const int m = idx / chunks, c = idx - m * chunks, gc = (kc0 >> 4) + c;
                 uint4 v = make_uint4(0, 0, 0, 0);
@@ -249,12 +260,14 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                             if (gc * 16 + j < g.K) w[j >> 2] |= (uint32_t)(uint8_t)src[j] << ((j & 3) * 8);
                         v = make_uint4(w[0], w[1], w[2], w[3]);
                     }
-                    if (first_wg && q.dst) store_codes(q.dst + tiled_chunk_offset(m, gc, KB), v);
+                    if (q.dst && (unsigned)(m * (Kp >> 4) + gc) - copy_lo < copy_share)
+                        *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, gc, KB)) = v;
                 }
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = v;
             }
         }
         __syncthreads();
+        RK_TS(6);
 
         // One group = UNR tiles per wave.  Int4: a tile is a 64-deep super-tile.
         // (counted in load instructions: one of them spans 32 / CW tiles; K is padded to 256 and a
@@ -349,6 +362,43 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             // a workgroup that asks for its next 64 KiB in one go is served faster than one that
             // trickles the requests out a tile at a time (4096 x 14336, int8: 11.5 against 11.9 us).
             int tb = wave;
+            if constexpr (PINGPONG) {
+                // Several rows: the group is kept as two halves.  While one half is multiplied
+                // with the rows (MR LDS reads and 4 * MR dot products per tile) the other half is
+                // in flight, and a half's registers are asked for again as soon as it is used --
+                // the loads of a wave never drain, in the registers the whole group took before.
+                constexpr int H = UNR / 2;
+                v4i wa[H], wb[H];
+#pragma unroll
+                for (int u = 0; u < H; ++u) {
+                    if constexpr (FUSEQ) {
+                        wa[u] = wpre[u];
+                        wb[u] = wpre[H + u];
+                    } else {
+                        wa[u] = load_unit(tb + u * GEMV_WAVES);
+                    }
+                }
+                if constexpr (!FUSEQ) {
+#pragma unroll
+                    for (int u = 0; u < H; ++u) wb[u] = load_unit(tb + (H + u) * GEMV_WAVES);
+                }
+                for (; tb < tiles; tb += GEMV_WAVES * UNR) {
+#pragma unroll
+                    for (int u = 0; u < H; ++u)
+                        if (tb + u * GEMV_WAVES < tiles) consume_unit(wa[u], tb + u * GEMV_WAVES);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < H; ++u) wa[u] = load_unit(tb + (UNR + u) * GEMV_WAVES); // (past the end: zeros, no access)
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < H; ++u)
+                        if (tb + (H + u) * GEMV_WAVES < tiles) consume_unit(wb[u], tb + (H + u) * GEMV_WAVES);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < H; ++u) wb[u] = load_unit(tb + (UNR + H + u) * GEMV_WAVES);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
             if constexpr (FUSEQ) {
 #pragma unroll
                 for (int u = 0; u < UNR; ++u)
@@ -362,6 +412,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
                 for (int u = 0; u < UNR; ++u)
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
+            }
             }
         }
     }

@@ -151,6 +151,10 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RING - 1) * LPS) : "memory");
 #pragma unroll
         for (int l = 0; l < LPS; ++l) asm volatile("" : "+v"(regs[l]));
+        // (the scale loads are older than every load of the ring: landed too.  From here on the
+        // two values are, for the compiler, defined behind a wait -- a copy or a spill of them
+        // moves data that has arrived)
+        asm volatile("" : "+v"(my_as), "+v"(my_ws));
     };
 
 #pragma unroll
