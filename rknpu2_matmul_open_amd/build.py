@@ -64,9 +64,19 @@ def check_toolchain(hipcc):
     return line
 
 
-def build(verbose=True):
+def build(verbose=True, audit=True):
+    """Compiles and links the library.  audit: also compile the two inline-assembly load units to
+    device assembly (alongside the objects) and check the hand-placed waits in it, see
+    audit_waits.py; a violation fails the build (RK_NPU_HIP_SKIP_WAIT_AUDIT=1 skips the check)."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     check_toolchain(hipcc)
+    audit = audit and os.environ.get("RK_NPU_HIP_SKIP_WAIT_AUDIT") != "1"
+    audit_pool = audit_jobs = None
+    if audit:
+        from concurrent.futures import ThreadPoolExecutor
+        from . import audit_waits
+        audit_pool = ThreadPoolExecutor(len(audit_waits.UNITS))
+        audit_jobs = [audit_pool.submit(audit_waits.device_assembly, u, hipcc, FLAGS) for u in audit_waits.UNITS]
     objs = []
     procs = []
     for src in SOURCES:
@@ -88,6 +98,21 @@ def build(verbose=True):
             sys.stderr.write("[build] %s\n%s\n" % (src, out))
     if failed:
         raise RuntimeError("hipcc failed")
+    if audit:
+        violations, checked = [], 0
+        for job in audit_jobs:
+            v, c = audit_waits.audit_text(job.result())
+            violations += v
+            checked += c
+        audit_pool.shutdown()
+        if violations or not checked:
+            for line in violations[:20]:
+                sys.stderr.write("[build] wait audit: %s\n" % line)
+            raise RuntimeError("wait audit: %d violations in %d kernels (hand-placed waits of the inline-assembly "
+                               "load kernels no longer cover their loads in the code this compiler produced)"
+                               % (len(violations), checked))
+        if verbose:
+            sys.stderr.write("[build] wait audit: %d kernels, no violation\n" % checked)
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lpthread"]
     subprocess.check_call(cmd)
     return LIB

@@ -84,6 +84,16 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// Compile-time chain: f(<0>) and, while it returns true, f(<1>) ... f(<N-1>).  Unlike N
+// independent `if`s the generated control flow has no path that skips a step and runs a later
+// one, which is what a sequence "the first n of N steps" means.
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_while(F&& f) {
+    if constexpr (I < N) {
+        if (f(std::integral_constant<int, I>{})) static_while<N, I + 1>(f);
+    }
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 

@@ -265,14 +265,23 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         if constexpr ((SLOT + 1) % G == 0) asm volatile("s_barrier" ::: "memory");
     };
 
-    // The tile's scales are requested now, ahead of the prologue's loads, and handed
+    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
+#pragma unroll
+    for (int t = -D; t < 0; ++t) {
+        copy_a(t + D);
+        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
+    }
+    RK_TS(1);
+    // The tile's scales are fetched now, behind the prologue's loads, and handed
     // to the epilogue through LDS after the loop, so the epilogue does not start
     // with a round trip to memory: thread t holds the row scale of row t
-    // (t < BM) and the column scale of physical column t (t < 256).  They are the
-    // oldest loads of the wave, so the first wait below covers them (loads return
-    // in issue order) -- and only behind that wait do the two values become, for
-    // the compiler, the long-lived values the epilogue uses: whatever it does with
-    // them from there on (a copy, a spill) moves data that has arrived.
+    // (t < BM) and the column scale of physical column t (t < 256).  (Two more
+    // loads in the queue only make the first sub-steps' waits stricter.  Ahead of
+    // the prologue's loads they cost the 128-row tile 0.2 us: the first copies
+    // leave later.)  They are in flight until the wait of the loop's third
+    // sub-step, or the closing wait; like every register an asm load writes they
+    // must not be touched before -- which the build verifies in the compiled code
+    // (audit_waits.py) rather than trusting the allocator.
     float my_as = 0.0f, my_ws = 0.0f;
     bool as_valid = false, ws_valid = false;
     if constexpr (EPI != RKH_EPI_I32) {
@@ -297,15 +306,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_as) : "v"(pa));
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
     }
-    // prologue: the same issue order as if the loop had run for sub-steps -D..-1
-#pragma unroll
-    for (int t = -D; t < 0; ++t) {
-        copy_a(t + D);
-        if (t + NSW - 1 >= 0) load_w(wring[t + NSW - 1]);
-    }
-    RK_TS(1);
     w_wait(wring[0]); // weights of sub-step 0 and the copies of sub-steps 0..D-NSW+1 have landed
-    asm volatile("" : "+v"(my_as), "+v"(my_ws)); // (landed: see above)
     asm volatile("s_barrier" ::: "memory");
     static_for<4>([&](auto f_tag) { read_frag(afr[0][decltype(f_tag)::value], std::integral_constant<int, 0>{}, f_tag); });
     static_for<NWREG>([&](auto e_tag) { unpack_item(wop[0], wring[0], e_tag); });
@@ -314,10 +315,14 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
 
     int s = 0;
     for (; s + UNR <= ksteps; s += UNR) static_for<UNR>([&](auto slot) { k_step(slot); });
-    if (s < ksteps)
-        static_for<UNR>([&](auto slot) {
-            if (s + decltype(slot)::value < ksteps) k_step(slot);
-        });
+    // (the remaining sub-steps as a chain that ends at the first one beyond K: the control flow
+    // then only holds the sequences of sub-steps that can happen, which is what the static check
+    // of the waits, audit_waits.py, walks)
+    static_while<UNR>([&](auto slot) {
+        if (s + decltype(slot)::value >= ksteps) return false;
+        k_step(slot);
+        return true;
+    });
     __builtin_amdgcn_s_setprio(0);
     RK_TS(3);
 
