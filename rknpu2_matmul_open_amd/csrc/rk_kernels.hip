@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
 
     float v[QR_CACHE][16];
     float mx = 0.0f;
-    bool bad = false;
+    float taint = 0.0f; // (NaN once an Inf or a NaN was seen, see absmax16)
     if (cached) {
 #pragma unroll
         for (int i = 0; i < QR_CACHE; ++i) {
@@ -222,11 +222,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
             if (c < nchunks) {
                 RowLoader<T>::load16(row, c * 16, K, vec, v[i]);
                 if (need_max) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        mx = fmaxf(mx, fabsf(v[i][j]));
-                        bad |= not_finite(v[i][j]);
-                    }
+                    absmax16(v[i], mx, taint);
                 }
             }
         }
@@ -234,11 +230,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
         for (int c = chunk0 + t; c < nchunks; c += 256) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                mx = fmaxf(mx, fabsf(tmp[j]));
-                bad |= not_finite(tmp[j]);
-            }
+            absmax16(tmp, mx, taint);
         }
     }
 
@@ -246,7 +238,7 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
     if (need_max) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-        const unsigned long long bad_mask = __ballot(bad && check);
+        const unsigned long long bad_mask = __ballot(tainted(taint) && check);
         if (lane_id() == 0) {
             wave_max[wave_id()] = mx;
             wave_bad[wave_id()] = bad_mask != 0ull;
@@ -565,31 +557,23 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const int32_t* h_ids, 
         }
     } else {
         float mx = 0.0f;
-        bool bad = false;
+        float taint = 0.0f; // (NaN once an Inf or a NaN was seen, see absmax16)
         if (cached) {
 #pragma unroll
             for (int i = 0; i < QR_CACHE; ++i)
                 if (t + i * 256 < nchunks) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        mx = fmaxf(mx, fabsf(v[i][j]));
-                        bad |= not_finite(v[i][j]);
-                    }
+                    absmax16(v[i], mx, taint);
                 }
         } else {
             for (int c = t; c < nchunks; c += 256) {
                 float tmp[16];
                 RowLoader<T>::load16(row, c * 16, K, vec, tmp);
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    mx = fmaxf(mx, fabsf(tmp[j]));
-                    bad |= not_finite(tmp[j]);
-                }
+                absmax16(tmp, mx, taint);
             }
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-        const unsigned long long bad_mask = __ballot(bad);
+        const unsigned long long bad_mask = __ballot(tainted(taint));
         if (lane == 0) {
             wave_max[wave] = mx;
             wave_bad[wave] = bad_mask != 0ull;
@@ -738,22 +722,18 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(rkh_moe_decode_arg
     constexpr int CACHE = MOE_DECODE_MAX_K / 16 / 512; // chunks per thread
     float v[CACHE][16];
     float mx = 0.0f;
-    bool bad = false;
+    float taint = 0.0f; // (NaN once an Inf or a NaN was seen, see absmax16)
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
         const int c = tid + i * 512;
         if (c < nchunks) {
             RowLoader<float>::load16(row, c * 16, H, vec, v[i]);
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                mx = fmaxf(mx, fabsf(v[i][q]));
-                bad |= not_finite(v[i][q]);
-            }
+            absmax16(v[i], mx, taint);
         }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    const unsigned long long bad_mask = __ballot(bad);
+    const unsigned long long bad_mask = __ballot(tainted(taint));
     if (lane == 0) {
         wave_max[wave] = mx;
         wave_bad[wave] = bad_mask != 0ull;

@@ -188,9 +188,40 @@ template <> struct RowLoader<int8_t> {
     }
 };
 
+// The largest magnitude bit pattern among the 16 elements of a chunk as fetched (sign bits
+// cleared).  Magnitudes of finite values order like their patterns, and a pattern of 0x7c00
+// (fp16) / 0x7f800000 (fp32) or more says that the chunk holds an Inf or a NaN.
+typedef unsigned short rk_us2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t chunk_top_magnitude(const RowLoader<uint16_t>::Raw& r) {
+    rk_us2 top = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        top = __builtin_elementwise_max(top, __builtin_bit_cast(rk_us2, r.w[j] & 0x7fff7fffu));
+    return top.x > top.y ? top.x : top.y;
+}
+__device__ __forceinline__ uint32_t chunk_top_magnitude(const RowLoader<float>::Raw& r) {
+    uint32_t top = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) top = max(top, __float_as_uint(r.v[j]) & 0x7fffffffu);
+    return top;
+}
+
 __device__ __forceinline__ bool not_finite(float x) {
     return (__float_as_uint(x) & 0x7f800000u) == 0x7f800000u;
 }
+
+// Running largest magnitude of 16 values and a watch for an Inf or a NaN among them: x * 0 is NaN
+// for an Inf or a NaN and a zero otherwise, so one fma per element leaves `taint` (started at 0)
+// NaN iff one was seen -- a comparison of the exponent bits costs three instructions per element,
+// and the quantizers are bound by their vector instructions as much as by memory.
+__device__ __forceinline__ void absmax16(const float* v, float& mx, float& taint) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        mx = fmaxf(mx, fabsf(v[j]));
+        taint = fmaf(v[j], 0.0f, taint);
+    }
+}
+__device__ __forceinline__ bool tainted(float taint) { return taint != taint; }
 
 // Byte offset of the 16-byte chunk (row, chunk c = k/16) in a tiled int8 matrix.
 __device__ __forceinline__ size_t tiled_chunk_offset(int row, int c, int KB) {
@@ -382,7 +413,7 @@ __device__ __forceinline__ void quant_rows_group(const rkh_quant_args& a, int fi
 
     float v[CACHE][16];
     float mx = 0.0f;
-    bool bad = false;
+    float taint = 0.0f; // (NaN once an Inf or a NaN was seen, see absmax16)
     if (cached) {
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
@@ -393,11 +424,7 @@ __device__ __forceinline__ void quant_rows_group(const rkh_quant_args& a, int fi
 #pragma unroll
             for (int i = 0; i < CACHE; ++i) {
                 if (cl + CSTEP * i < nchunks) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        mx = fmaxf(mx, fabsf(v[i][j]));
-                        bad |= not_finite(v[i][j]);
-                    }
+                    absmax16(v[i], mx, taint);
                 }
             }
         }
@@ -405,18 +432,14 @@ __device__ __forceinline__ void quant_rows_group(const rkh_quant_args& a, int fi
         for (int c = cl; c < nchunks; c += CSTEP) {
             float tmp[16];
             RowLoader<T>::load16(row, c * 16, K, vec, tmp);
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                mx = fmaxf(mx, fabsf(tmp[j]));
-                bad |= not_finite(tmp[j]);
-            }
+            absmax16(tmp, mx, taint);
         }
     }
     float scale = 1.0f;
     if (need_max) {
 #pragma unroll
         for (int off = ROWS; off < 64; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-        const unsigned long long bad_mask = __ballot(bad && check && live);
+        const unsigned long long bad_mask = __ballot(tainted(taint) && check && live);
         if (lane < ROWS) part_max[wave * ROWS + lane] = mx;
         if (lane == 0) part_bad[wave] = bad_mask != 0ull;
         __syncthreads();

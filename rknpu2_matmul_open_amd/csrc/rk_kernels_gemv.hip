@@ -21,7 +21,142 @@ constexpr int GEMV_WAVES = RK_GEMV_WAVES;
 constexpr int GEMV_UNROLL = RK_GEMV_UNROLL;
 constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
 
+#ifndef RK_GEMV_MFMA_ROWS
+#define RK_GEMV_MFMA_ROWS 4
+#endif
+constexpr int GEMV_MFMA_ROWS = RK_GEMV_MFMA_ROWS; // from this many rows on the products go through the matrix cores
 constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
+
+// The per-token quantization that both dot-product kernels can run in their prologue: every
+// workgroup quantizes the few rows itself into its LDS staging area (they are L2 hits after the
+// first workgroup), which saves a launch per decode step.  Every instruction here is executed by
+// every workgroup, ahead of its first dot product -- for several rows this prologue, not the
+// weight stream, is what a 4096 x 4096 call waits for (in-kernel time stamps, eight rows: 3.8 of
+// 9.4 us) -- so it is kept lean:
+//   * chunk i of 16 elements of thread t is number t + i * (threads) of the rows laid end to end;
+//     its row and its place in the row are stepped from chunk to chunk (one division per thread,
+//     none for a single row), and each pass steps again from the first chunk's place, which is all
+//     that stays in registers between the passes (the empty asm keeps the compiler from holding
+//     all eight indices instead);
+//   * the largest magnitude of a chunk is taken from the bit patterns as fetched: magnitudes of
+//     finite values order like their patterns, so no element is converted for this pass (fp16: two
+//     per instruction), and a chunk that holds an Inf or a NaN -- its largest pattern says so --
+//     takes the float comparisons, which skip NaNs;
+//   * 1 / scale is divided once per row, not once per chunk.
+// The rows stay in registers as fetched and are converted once, for the codes: holding them as
+// floats across the barriers costs the int4 variants their second workgroup per compute unit.
+template <typename T, int MR>
+struct FusedRows {
+    static constexpr int THREADS = GEMV_WAVES * 64;
+    typename RowLoader<T>::Raw raw[GEMV_QCHUNKS];
+    int m0, c0; // row and place in the row of this thread's first chunk
+
+    __device__ __forceinline__ void index(int nchunks, int (&m)[GEMV_QCHUNKS], int (&c)[GEMV_QCHUNKS]) {
+        if constexpr (MR == 1) {
+#pragma unroll
+            for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+                c[i] = (int)threadIdx.x + i * THREADS;
+                m[i] = c[i] < nchunks ? 0 : 1;
+            }
+        } else {
+            const int step_m = THREADS / nchunks, step_c = THREADS - step_m * nchunks; // (uniform)
+            asm volatile("" : "+v"(m0), "+v"(c0));
+            m[0] = m0;
+            c[0] = c0;
+#pragma unroll
+            for (int i = 1; i < GEMV_QCHUNKS; ++i) {
+                const int cc = c[i - 1] + step_c;
+                const bool wrap = cc >= nchunks;
+                c[i] = wrap ? cc - nchunks : cc;
+                m[i] = m[i - 1] + step_m + (wrap ? 1 : 0);
+            }
+        }
+    }
+    // requests this thread's chunks of the M rows of K elements at src
+    __device__ __forceinline__ void fetch(const void* src, int M, int K) {
+        const int nchunks = (K + 15) >> 4;
+        m0 = MR == 1 ? 0 : (int)threadIdx.x / nchunks;
+        c0 = (int)threadIdx.x - m0 * nchunks;
+        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        index(nchunks, m, c);
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            if (m[i] < M) {
+                const T* row = static_cast<const T*>(src) + (size_t)m[i] * K;
+                raw[i] = RowLoader<T>::load16_raw(row, c[i] * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            }
+        }
+    }
+    // row maxima (as float bits, into the zeroed row_max[] in LDS); true if a chunk of this thread
+    // holds an Inf or a NaN
+    __device__ __forceinline__ bool maxima(int M, int K, uint32_t* row_max) {
+        const int nchunks = (K + 15) >> 4;
+        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        index(nchunks, m, c);
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            if (m[i] < M) {
+                uint32_t top = chunk_top_magnitude(raw[i]);
+                if (top >= (sizeof(T) == 2 ? 0x7c00u : 0x7f800000u)) {
+                    bad = true;
+                    float v[16];
+                    RowLoader<T>::unpack(raw[i], v);
+                    float mx = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, fabsf(v[j]));
+                    top = __float_as_uint(mx);
+                } else if (sizeof(T) == 2) {
+                    top = __float_as_uint(half_bits_to_float((uint16_t)top));
+                }
+                // (non-negative floats order like their bits.  For one row, a shuffle reduction per wave
+                // and one atomic per wave instead of 64 on the same address measured slower: 4096 x 14336
+                // int8 10.65 -> 10.7 us, int4 6.8 -> 7.2 us)
+                atomicMax(&row_max[m[i]], top);
+            }
+        }
+        return bad;
+    }
+    // scale and 1 / scale of row threadIdx.x (threads below M), by the rule of the mode
+    static __device__ __forceinline__ void scales(int M, int mode, const uint32_t* row_max, float* row_scale,
+                                                  float* row_inv, float* out_scale) {
+        const int t = threadIdx.x;
+        if (t < M) {
+            const float mx = __uint_as_float(row_max[t]);
+            const float sc = mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
+                                                : (mx > 0.0f ? mx / 127.0f : 1.0f);
+            row_scale[t] = sc;
+            row_inv[t] = 1.0f / sc;
+            if (out_scale) out_scale[t] = sc;
+        }
+    }
+    // zeroes the K padding of the staged rows (row-major [M][Kp] at a_lds)
+    static __device__ __forceinline__ void zero_padding(int M, int K, int Kp, uint8_t* a_lds) {
+        const int nchunks = (K + 15) >> 4, pad = (Kp >> 4) - nchunks;
+        for (int idx = threadIdx.x; idx < M * pad; idx += THREADS) {
+            const int m = idx / pad, c = nchunks + idx % pad;
+            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+        }
+    }
+    // codes into the staged rows (as their two signed digits if DIGITS) and, where dst is given,
+    // into the tiled copy the separate quantization launch would have left
+    template <bool DIGITS>
+    __device__ __forceinline__ void quantize(int M, int K, int Kp, const float* row_inv, uint8_t* a_lds, uint8_t* dst) {
+        const int nchunks = (K + 15) >> 4, KB = Kp / 32;
+        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        index(nchunks, m, c);
+#pragma unroll
+        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            if (m[i] < M) {
+                float v[16];
+                RowLoader<T>::unpack(raw[i], v);
+                const uint4 packed = quantize16<false>(v, row_inv[m[i]]);
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m[i] * Kp + (size_t)c[i] * 16) = DIGITS ? digits16(packed) : packed;
+                if (dst) *reinterpret_cast<uint4*>(dst + tiled_chunk_offset(m[i], c[i], KB)) = packed;
+            }
+        }
+    }
+};
 
 // QT: 0 = activations come quantized from the tiled buffer g.A;
 //     3 = int8 rows as the caller holds them (row-major q.src): staged from there, no launch of
@@ -91,11 +226,23 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // 11.7 / 13.85 -> 13.2; 14336 x 4096 16.1 -> 14.9 / 22.9 -> 21.4; 4096 x 4096 within 1 %; int4
     // weights lose with two rows, 8.5 -> 9.3 and 5.35 -> 5.6, and keep the whole group.)
     constexpr bool PINGPONG = MR > 1 && !W4;
+    // Several rows on the matrix cores: with dot products every staged row costs a 16-byte LDS read
+    // per lane and tile, and a compute unit's LDS serves one such read per 8 clocks while HBM
+    // delivers it a tile every ~40 -- from four rows on the LDS, not the memory, sets the pace.
+    // A weight tile as a lane holds it IS the first operand of v_mfma_i32_32x32x32_i8 (32 columns x
+    // 32 k; the 16-column workgroups' piece of two consecutive tiles is the first operand of
+    // v_mfma_i32_16x16x64_i8), and the staged rows are the second one: lane l reads the 16 bytes
+    // of row l % CW at its k-half -- one LDS read and one MFMA per tile however many rows.  Rows
+    // past MR read row MR - 1 again: column j of the product depends on column j of the second
+    // operand only, and those columns are never stored.
+    constexpr bool MATRIX = MR >= GEMV_MFMA_ROWS && CW >= 16 && !(W4 && CW == 32);
+    constexpr int CREGS = CW == 32 ? 16 : 4;                // accumulator registers of the matrix path
     constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
     __shared__ int red[GEMV_WAVES][MR][CW];
     __shared__ uint32_t row_max[MR];
     __shared__ float row_scale[MR];
+    __shared__ float row_inv[MR];
     const int lane = lane_id(), wave = wave_id();
     const int half = (lane / CW) & 1;                       // which 16 k of a 32-k tile
     const int sub = lane / (2 * CW);                        // which tile of the group one load covers
@@ -111,6 +258,12 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     int acc[MR], acc_lo[MR]; // (int4 weights: the sums of the high and of the low activation digits)
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[m] = acc_lo[m] = 0;
+    // matrix path: the 32 x 32 (16 x 16) tile of sums, lane l = row l % CW; int4 weights ride as
+    // 16 x code, taken off per K chunk into `ctot` so that no K can wrap the factor
+    typename std::conditional<CW == 32, v16i, v4i>::type cacc, ctot;
+#pragma unroll
+    for (int r = 0; r < CREGS; ++r) cacc[r] = ctot[r] = 0;
+    const int mrow = min(lane % (CW < 16 ? 16 : CW), MR - 1);
 
     const size_t block_bytes = (size_t)(W4 ? Kp / 64 : KB) * 1024; // one column block over all of K
     const uint8_t* wbase = g.W + (size_t)p * block_bytes;
@@ -140,7 +293,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
     v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
-    typename RowLoader<QT_T>::Raw araw[FUSEQ ? GEMV_QCHUNKS : 1];
+    FusedRows<QT_T, MR> rows;
     if constexpr (FUSEQ) {
         const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
         if constexpr (BURST) {
@@ -148,16 +301,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = (int)threadIdx.x + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                const QT_T* row = static_cast<const QT_T*>(q.src) + (size_t)m * K;
-                araw[i] = RowLoader<QT_T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
-            }
-        }
+        rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!BURST) {
 #pragma unroll
@@ -167,62 +311,16 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         RK_TS(4);
     }
     if constexpr (FUSEQ) {
-        using T = QT_T;
-        const int t = threadIdx.x;
-        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
-        if (t < MR) row_max[t] = 0u;
+        if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
         __syncthreads();
         RK_TS(5);
-        // (the rows stay in registers as fetched and are converted once per pass:
-        // holding them as floats across the barriers costs the int4 variants their
-        // second workgroup per compute unit)
-        bool bad = false;
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                float mx = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    mx = fmaxf(mx, fabsf(v[j]));
-                    bad |= not_finite(v[j]);
-                }
-                // (non-negative floats order like their bits.  For one row, a shuffle reduction per wave
-                // and one atomic per wave instead of 64 on the same address measured slower: 4096 x 14336
-                // int8 10.65 -> 10.7 us, int4 6.8 -> 7.2 us)
-                atomicMax(&row_max[m], __float_as_uint(mx));
-            }
-        }
+        const bool bad = rows.maxima(g.M, g.K, row_max);
         __syncthreads();
-        if (t < g.M) {
-            const float mx = __uint_as_float(row_max[t]);
-            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
-                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
-            row_scale[t] = sc;
-            if (first_wg && q.scale) q.scale[t] = sc;
-        }
+        rows.scales(g.M, q.mode, row_max, row_scale, row_inv, first_wg ? q.scale : nullptr);
         if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
-        // zero the K padding of the staged rows
-        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) {
-            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
-            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
-        }
+        rows.zero_padding(g.M, g.K, Kp, a_lds);
         __syncthreads();
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
-                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
-            }
-        }
+        rows.template quantize<W4 && !MATRIX>(g.M, g.K, Kp, row_inv, a_lds, first_wg ? q.dst : nullptr);
         // a_scale of the epilogue comes from LDS in this path
         RK_TS(1);
     }
@@ -236,7 +334,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
                 const int m = idx / chunks, c = idx - m * chunks;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
+                *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = (W4 && !MATRIX) ? digits16(v) : v;
             }
         } else if constexpr (QT == 3) {
             // int8 rows as the caller holds them (row-major, any alignment, K not padded).  The tiled
@@ -280,7 +378,23 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                 // zeros, so whatever the activation read returns does not matter: it lands in the
                 // next row or in the padding behind the last one.
                 const int tt = unit * TPL + sub;
-                if constexpr (!W4) {
+                if constexpr (MATRIX) {
+                    auto mma = [&](const v4i& wop, const v4i& aop) {
+                        if constexpr (CW == 32) cacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, aop, cacc, 0, 0, 0);
+                        else cacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, aop, cacc, 0, 0, 0);
+                    };
+                    if constexpr (!W4) {
+                        mma(wu, *reinterpret_cast<const v4i*>(a_lds + (size_t)mrow * kc + (size_t)(tt * 2 + half) * 16));
+                    } else {
+                        // (a super-tile: the lane's 8 bytes of each 32-deep half, unpacked as 16 x code)
+                        const v4i lo = v4i{(wu.x << 4) & (int)0xF0F0F0F0, wu.x & (int)0xF0F0F0F0,
+                                           (wu.y << 4) & (int)0xF0F0F0F0, wu.y & (int)0xF0F0F0F0};
+                        const v4i hi = v4i{(wu.z << 4) & (int)0xF0F0F0F0, wu.z & (int)0xF0F0F0F0,
+                                           (wu.w << 4) & (int)0xF0F0F0F0, wu.w & (int)0xF0F0F0F0};
+                        mma(lo, *reinterpret_cast<const v4i*>(a_lds + (size_t)mrow * kc + (size_t)((tt * 2 + 0) * 2 + half) * 16));
+                        mma(hi, *reinterpret_cast<const v4i*>(a_lds + (size_t)mrow * kc + (size_t)((tt * 2 + 1) * 2 + half) * 16));
+                    }
+                } else if constexpr (!W4) {
 #pragma unroll
                     for (int m = 0; m < MR; ++m) {
                         const v4i av = *reinterpret_cast<const v4i*>(a_lds + (size_t)m * kc + (size_t)(tt * 2 + half) * 16);
@@ -415,9 +529,29 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
             }
             }
         }
+        if constexpr (MATRIX && W4 && !FUSEQ) {
+            // (a wave's share of a chunk is at most 512 k per row: 16 x code sums stay far inside int32;
+            // the fused path has a single chunk and shifts in the epilogue)
+#pragma unroll
+            for (int r = 0; r < CREGS; ++r) {
+                ctot[r] += cacc[r] >> 4;
+                cacc[r] = 0;
+            }
+        }
     }
 
     RK_TS(2);
+    if constexpr (MATRIX) {
+        // lane l holds row l % CW of the tile: 16 columns 8 * (r / 4) + 4 * (l / 32) + r % 4 of 32, or 4
+        // columns 4 * (l / 16) + r of 16; the MFMA has already summed over the lanes' k-halves
+        if (lane % CW < MR) {
+#pragma unroll
+            for (int r = 0; r < CREGS; ++r) {
+                const int col = CW == 32 ? 8 * (r / 4) + 4 * (lane / 32) + r % 4 : 4 * (lane / 16) + r;
+                red[wave][lane % CW][col] = !W4 ? cacc[r] : FUSEQ ? cacc[r] >> 4 : ctot[r];
+            }
+        }
+    } else {
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         int v = W4 ? 16 * acc[m] + acc_lo[m] : acc[m];
@@ -425,6 +559,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         if (CW <= 16) v += __shfl_xor(v, 16);
         if (CW <= 8) v += __shfl_xor(v, 8);
         if (lane < CW) red[wave][m][lane] = v;
+    }
     }
     __syncthreads();
     static_assert(MR * 32 <= GEMV_WAVES * 64, "one output element per thread");
@@ -436,7 +571,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
         const int n = block_first_col(p, g.interleave_F) + col0 + j;
-        if (W4 && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
+        if (W4 && !MATRIX && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
         if (n < g.N)
             store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
                       FUSEQ ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
@@ -466,6 +601,7 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
     __shared__ int red[2][GEMV_WAVES][MR][32];
     __shared__ uint32_t row_max[MR];
     __shared__ float row_scale[MR];
+    __shared__ float row_inv[MR];
     const int lane = lane_id(), wave = wave_id();
     const int half = lane >> 5;
     const int Kp = (int)rkh_align_up(g.K, RKH_K_ALIGN);
@@ -499,67 +635,21 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
 
     if constexpr (QT != 0) { // (the fused path has a single K chunk: rows fit the staging area)
         using T = typename std::conditional<QT == 2, float, uint16_t>::type;
-        const int t = threadIdx.x;
         const bool first_wg = blockIdx.x == 0;
-        const int K = g.K, nchunks = (K + 15) >> 4, total = g.M * nchunks;
-        typename RowLoader<T>::Raw araw[GEMV_QCHUNKS];
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                const T* row = static_cast<const T*>(q.src) + (size_t)m * K;
-                araw[i] = RowLoader<T>::load16_raw(row, c * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
-            }
-        }
+        FusedRows<T, MR> rows;
+        rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
         load_group(wave, W4 ? Kp >> 6 : Kp >> 5, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (t < MR) row_max[t] = 0u;
+        if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
         __syncthreads();
-        bool bad = false;
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                float mx = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    mx = fmaxf(mx, fabsf(v[e]));
-                    bad |= not_finite(v[e]);
-                }
-                atomicMax(&row_max[m], __float_as_uint(mx)); // non-negative floats order like their bits
-            }
-        }
+        const bool bad = rows.maxima(g.M, g.K, row_max);
         __syncthreads();
-        if (t < g.M) {
-            const float mx = __uint_as_float(row_max[t]);
-            const float sc = q.mode == RKH_Q_W4A8 ? (mx == 0.0f ? 1.0f : fmaxf(mx / 127.0f, FLT_MIN))
-                                                  : (mx > 0.0f ? mx / 127.0f : 1.0f);
-            row_scale[t] = sc;
-            if (first_wg && q.scale) q.scale[t] = sc;
-        }
+        rows.scales(g.M, q.mode, row_max, row_scale, row_inv, first_wg ? q.scale : nullptr);
         if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
-        for (int idx = t; idx < g.M * ((Kp >> 4) - nchunks); idx += GEMV_WAVES * 64) { // zero the K padding
-            const int m = idx / ((Kp >> 4) - nchunks), c = nchunks + idx % ((Kp >> 4) - nchunks);
-            *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
-        }
+        rows.zero_padding(g.M, g.K, Kp, a_lds);
         __syncthreads();
-#pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
-            const int pidx = t + i * GEMV_WAVES * 64;
-            if (pidx < total) {
-                const int m = pidx / nchunks, c = pidx - m * nchunks;
-                float v[16];
-                RowLoader<T>::unpack(araw[i], v);
-                const uint4 packed = quantize16<false>(v, 1.0f / row_scale[m]);
-                *reinterpret_cast<uint4*>(a_lds + (size_t)m * Kp + (size_t)c * 16) = W4 ? digits16(packed) : packed;
-                if (first_wg && q.dst) *reinterpret_cast<uint4*>(q.dst + tiled_chunk_offset(m, c, KB)) = packed;
-            }
-        }
+        rows.template quantize<W4>(g.M, g.K, Kp, row_inv, a_lds, first_wg ? q.dst : nullptr);
     }
 
     for (int kc0 = 0; kc0 < Kp; kc0 += kc_max) {
