@@ -19,13 +19,26 @@ namespace {
 #endif
 constexpr int GEMV_WAVES = RK_GEMV_WAVES;
 constexpr int GEMV_UNROLL = RK_GEMV_UNROLL;
-constexpr int GEMV_LDS_BYTES = 32768; // activation bytes staged per K chunk
+// Activation bytes staged per K chunk: 32 KiB; 64 KiB in the BIG variants (two workgroups of 64 KiB +
+// their reduction area still fit a compute unit's 160 KiB), which take four to eight rows of a long
+// K on int8 weights, so that four rows of a 14336-deep projection are one chunk -- and can be
+// quantized by the kernel itself instead of a launch in front (21.6 -> 18.0 us).  Shapes that fit
+// the small area keep the small kernel: with room for eight chunks a thread, four rows of
+// 4096 x 4096 took 7.1 instead of 6.65 us.  (The int4 variants have no registers to spare for it.)
+constexpr int GEMV_LDS_BYTES = 32768;
+__host__ __device__ constexpr int gemv_lds_bytes(bool big) { return big ? 2 * GEMV_LDS_BYTES : GEMV_LDS_BYTES; }
+__host__ __device__ constexpr bool gemv_big_applies(int mr, bool w4, long padded_k) {
+    return mr >= 4 && !w4 && padded_k * mr > GEMV_LDS_BYTES;
+}
 
 #ifndef RK_GEMV_MFMA_ROWS
 #define RK_GEMV_MFMA_ROWS 4
 #endif
 constexpr int GEMV_MFMA_ROWS = RK_GEMV_MFMA_ROWS; // from this many rows on the products go through the matrix cores
-constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may quantize in the fused path
+// 16-element activation chunks a thread may quantize in the fused path: four; eight for fp16 rows
+// (8 registers a chunk as fetched) in the BIG variants, which fills their staging area
+constexpr int GEMV_QCHUNKS = 4;
+__host__ __device__ constexpr int gemv_qchunks(bool big, int elem_bytes) { return big && elem_bytes == 2 ? 2 * GEMV_QCHUNKS : GEMV_QCHUNKS; }
 
 // The per-token quantization that both dot-product kernels can run in their prologue: every
 // workgroup quantizes the few rows itself into its LDS staging area (they are L2 hits after the
@@ -45,16 +58,17 @@ constexpr int GEMV_QCHUNKS = 4; // 16-element activation chunks a thread may qua
 //   * 1 / scale is divided once per row, not once per chunk.
 // The rows stay in registers as fetched and are converted once, for the codes: holding them as
 // floats across the barriers costs the int4 variants their second workgroup per compute unit.
-template <typename T, int MR>
+template <typename T, int MR, bool BIG>
 struct FusedRows {
     static constexpr int THREADS = GEMV_WAVES * 64;
-    typename RowLoader<T>::Raw raw[GEMV_QCHUNKS];
+    static constexpr int QCH = gemv_qchunks(BIG, (int)sizeof(T));
+    typename RowLoader<T>::Raw raw[QCH];
     int m0, c0; // row and place in the row of this thread's first chunk
 
-    __device__ __forceinline__ void index(int nchunks, int (&m)[GEMV_QCHUNKS], int (&c)[GEMV_QCHUNKS]) {
+    __device__ __forceinline__ void index(int nchunks, int (&m)[QCH], int (&c)[QCH]) {
         if constexpr (MR == 1) {
 #pragma unroll
-            for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+            for (int i = 0; i < QCH; ++i) {
                 c[i] = (int)threadIdx.x + i * THREADS;
                 m[i] = c[i] < nchunks ? 0 : 1;
             }
@@ -64,7 +78,7 @@ struct FusedRows {
             m[0] = m0;
             c[0] = c0;
 #pragma unroll
-            for (int i = 1; i < GEMV_QCHUNKS; ++i) {
+            for (int i = 1; i < QCH; ++i) {
                 const int cc = c[i - 1] + step_c;
                 const bool wrap = cc >= nchunks;
                 c[i] = wrap ? cc - nchunks : cc;
@@ -77,10 +91,10 @@ struct FusedRows {
         const int nchunks = (K + 15) >> 4;
         m0 = MR == 1 ? 0 : (int)threadIdx.x / nchunks;
         c0 = (int)threadIdx.x - m0 * nchunks;
-        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        int m[QCH], c[QCH];
         index(nchunks, m, c);
 #pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+        for (int i = 0; i < QCH; ++i) {
             if (m[i] < M) {
                 const T* row = static_cast<const T*>(src) + (size_t)m[i] * K;
                 raw[i] = RowLoader<T>::load16_raw(row, c[i] * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
@@ -91,11 +105,11 @@ struct FusedRows {
     // holds an Inf or a NaN
     __device__ __forceinline__ bool maxima(int M, int K, uint32_t* row_max) {
         const int nchunks = (K + 15) >> 4;
-        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        int m[QCH], c[QCH];
         index(nchunks, m, c);
         bool bad = false;
 #pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+        for (int i = 0; i < QCH; ++i) {
             if (m[i] < M) {
                 uint32_t top = chunk_top_magnitude(raw[i]);
                 if (top >= (sizeof(T) == 2 ? 0x7c00u : 0x7f800000u)) {
@@ -143,10 +157,10 @@ struct FusedRows {
     template <bool DIGITS>
     __device__ __forceinline__ void quantize(int M, int K, int Kp, const float* row_inv, uint8_t* a_lds, uint8_t* dst) {
         const int nchunks = (K + 15) >> 4, KB = Kp / 32;
-        int m[GEMV_QCHUNKS], c[GEMV_QCHUNKS];
+        int m[QCH], c[QCH];
         index(nchunks, m, c);
 #pragma unroll
-        for (int i = 0; i < GEMV_QCHUNKS; ++i) {
+        for (int i = 0; i < QCH; ++i) {
             if (m[i] < M) {
                 float v[16];
                 RowLoader<T>::unpack(raw[i], v);
@@ -199,7 +213,7 @@ struct FusedRows {
 // per wave in flight (10.7), 28 instead of 32 columns per workgroup (512 workgroups, two for
 // every compute unit, instead of 448 -- 11.85 us; the per-lane addresses this needs cost 0.4 us
 // already with 32 columns).
-template <int MR, bool W4, int QT, int CW, bool BURST = false>
+template <int MR, bool W4, int QT, int CW, bool BURST = false, bool BIG = false>
 __global__ __launch_bounds__(GEMV_WAVES * 64) __attribute__((amdgpu_waves_per_eu(GEMV_WAVES / 2)))
 void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     RK_GEMV_HEAD_APPLY(g, q);
@@ -216,6 +230,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // shapes; the burst variant 10.6 -> 11.4 us).
     constexpr int UNR = (MR == 1 && !BURST) ? 4 : GEMV_UNROLL;
     static_assert(!BURST || (MR == 1 && !W4 && CW == 32), "the burst variant serves one int8 row, whole column blocks");
+    static_assert(!BIG || (MR >= 4 && !W4), "the larger staging area: four to eight rows, int8 weights");
     constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
     // (padding for the single-row variants of narrow matrices: their look-ahead of UNR loads per wave, and
     // one more step for the activations, runs up to that many load instructions past the end
@@ -238,7 +253,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     constexpr bool MATRIX = MR >= GEMV_MFMA_ROWS && CW >= 16 && !(W4 && CW == 32);
     constexpr int CREGS = CW == 32 ? 16 : 4;                // accumulator registers of the matrix path
     constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
-    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GEMV_LDS_BYTES + A_PAD];
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[gemv_lds_bytes(BIG) + A_PAD];
     __shared__ int red[GEMV_WAVES][MR][CW];
     __shared__ uint32_t row_max[MR];
     __shared__ float row_scale[MR];
@@ -254,7 +269,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // byte of this lane inside a 1 KiB tile
     const unsigned lane_byte = (unsigned)((col0 + lane % CW) + 32 * half) * 16u;
     // chunk of K staged in LDS at a time (multiple of 64)
-    const int kc_max = (GEMV_LDS_BYTES / MR) & ~63;
+    const int kc_max = (gemv_lds_bytes(BIG) / MR) & ~63;
     int acc[MR], acc_lo[MR]; // (int4 weights: the sums of the high and of the low activation digits)
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[m] = acc_lo[m] = 0;
@@ -293,7 +308,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // quantization runs under the weight loads' latency.  (BURST: the other way round, see above.)
     v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
-    FusedRows<QT_T, MR> rows;
+    FusedRows<QT_T, MR, BIG> rows;
     if constexpr (FUSEQ) {
         const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
         if constexpr (BURST) {
@@ -636,7 +651,7 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
     if constexpr (QT != 0) { // (the fused path has a single K chunk: rows fit the staging area)
         using T = typename std::conditional<QT == 2, float, uint16_t>::type;
         const bool first_wg = blockIdx.x == 0;
-        FusedRows<T, MR> rows;
+        FusedRows<T, MR, false> rows;
         rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
         load_group(wave, W4 ? Kp >> 6 : Kp >> 5, 0);
@@ -779,12 +794,21 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
         return RKH_OK;
     }
     mark(st, label);
+#define RK_GEMV_CW(W4, QT, BIG)                                                                \
+    do {                                                                                       \
+        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8, false, BIG>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
+        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16, false, BIG>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q); \
+        else if constexpr (!(MR == 1 && !W4)) /* (one int8 row, 32 columns: the burst variant above) */   \
+            hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32, false, BIG>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
+    } while (0)
+    // (the larger staging area where the rows do not fit the small one, see gemv_lds_bytes)
+    const bool big = gemv_big_applies(MR, g.w_int4 != 0, (long)rkh_align_up(g.K, RKH_K_ALIGN));
 #define RK_GEMV(W4, QT)                                                                        \
     do {                                                                                       \
-        if (cw == 8) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 8>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);        \
-        else if (cw == 16) hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 16>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q); \
-        else if constexpr (!(MR == 1 && !W4)) /* (one int8 row, 32 columns: the burst variant above) */   \
-            hipLaunchKernelGGL((gemv_kernel<MR, W4, QT, 32>), grid, block, 0, st, RK_GEMV_HEAD(g, q), g, q);               \
+        if constexpr (MR >= 4 && !W4) {                                                        \
+            if (big) { RK_GEMV_CW(W4, QT, true); break; }                                      \
+        }                                                                                      \
+        RK_GEMV_CW(W4, QT, false);                                                             \
     } while (0)
     if (g.w_int4) {
         if (qt == 0) RK_GEMV(true, 0); else if (qt == 1) RK_GEMV(true, 1); else RK_GEMV(true, 2);
@@ -793,6 +817,7 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
         else RK_GEMV(false, 3);
     }
 #undef RK_GEMV
+#undef RK_GEMV_CW
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
@@ -869,9 +894,10 @@ bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu 
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
     const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
     const long kp = (long)rkh_align_up(g.K, RKH_K_ALIGN);
-    if (kp * mr > GEMV_LDS_BYTES) return false;
+    const bool big = !swiglu && gemv_big_applies(mr, g.w_int4 != 0, kp); // (the SwiGLU kernel keeps the small area)
+    if (kp * mr > gemv_lds_bytes(big)) return false;
     const long chunks = (long)g.M * ((g.K + 15) / 16);
-    return chunks <= (long)GEMV_QCHUNKS * GEMV_WAVES * 64;
+    return chunks <= (long)gemv_qchunks(big, q.in_dtype == RKH_F16 ? 2 : 4) * GEMV_WAVES * 64;
 }
 
 } // namespace
