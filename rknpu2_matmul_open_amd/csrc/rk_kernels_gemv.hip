@@ -58,6 +58,12 @@ __host__ __device__ constexpr int gemv_qchunks(bool big, int elem_bytes) { retur
 //   * 1 / scale is divided once per row, not once per chunk.
 // The rows stay in registers as fetched and are converted once, for the codes: holding them as
 // floats across the barriers costs the int4 variants their second workgroup per compute unit.
+// (One fp16 row in pieces of 8 elements, so that a row of 4096 gives every one of the 512 threads a
+// piece instead of half of them a chunk, was built and measured: 10.9 against 10.75 us for
+// 4096 x 14336, 5.35 against 5.15 for 4096 x 4096 -- twice the lanes on the one LDS maximum and
+// twice the slots of straight-line code cost more than the idle waves.  Note for anyone who tries
+// again: an LDS atomic whose address the compiler can prove uniform is replaced by a scalar loop
+// over the 64 lanes, 1.5 us per use here; keep the index in a vector register.)
 template <typename T, int MR, bool BIG>
 struct FusedRows {
     static constexpr int THREADS = GEMV_WAVES * 64;
@@ -87,17 +93,36 @@ struct FusedRows {
         }
     }
     // requests this thread's chunks of the M rows of K elements at src
+    // (Whole chunks with vector loads, whatever the row's alignment: this target reads under-aligned
+    // vectors, the compiler itself emits them for a 16-byte copy from a 2-byte-aligned address.  The
+    // ragged last chunk of a row -- one per row -- is read element by element in a loop of its own
+    // and placed into its owner's slot: inlined into every slot, that path tripled the code between
+    // the top of the kernel and the first dot product.)
     __device__ __forceinline__ void fetch(const void* src, int M, int K) {
-        const int nchunks = (K + 15) >> 4;
+        const int nchunks = (K + 15) >> 4, whole = K >> 4;
         m0 = MR == 1 ? 0 : (int)threadIdx.x / nchunks;
         c0 = (int)threadIdx.x - m0 * nchunks;
         int m[QCH], c[QCH];
         index(nchunks, m, c);
+        // (zeros first, loads behind them: a register cleared after a load into it was issued makes
+        // the compiler wait for every load in flight, the weight tiles requested ahead included)
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) __builtin_memset(&raw[i], 0, sizeof(raw[i]));
 #pragma unroll
         for (int i = 0; i < QCH; ++i) {
-            if (m[i] < M) {
-                const T* row = static_cast<const T*>(src) + (size_t)m[i] * K;
-                raw[i] = RowLoader<T>::load16_raw(row, c[i] * 16, K, (reinterpret_cast<uintptr_t>(row) & 15) == 0);
+            if (m[i] < M && c[i] < whole)
+                __builtin_memcpy(&raw[i], static_cast<const T*>(src) + (size_t)m[i] * K + (size_t)c[i] * 16, sizeof(raw[i]));
+        }
+        if (K & 15) {
+#pragma nounroll
+            for (int mm = 0; mm < M; ++mm) {
+                const int pidx = mm * nchunks + whole; // (uniform: the tail chunk of row mm, its owner and slot)
+                if ((int)threadIdx.x != pidx % THREADS) continue;
+                const typename RowLoader<T>::Raw tail =
+                    RowLoader<T>::load16_raw(static_cast<const T*>(src) + (size_t)mm * K, whole * 16, K, false);
+#pragma unroll
+                for (int i = 0; i < QCH; ++i)
+                    if (i == pidx / THREADS) raw[i] = tail;
             }
         }
     }
