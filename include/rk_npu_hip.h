@@ -88,10 +88,11 @@ int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* workspace,
  * and without any allocation, for callers that cannot allocate: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  The scratch the kernels need (the
  * quantized rows, their scales, K-split partial tiles) lies in a static device array of
- * 12 MiB that each GPU the library runs on holds until the process ends; a shape needing more
- * (roughly align128(M) * align256(K) + 4 * align128(M) + the partial tiles, e.g. M = 2048
+ * 12 MiB that each GPU the library runs on holds until the process ends; a shape whose rows
+ * and scales need more (roughly align128(M) * align256(K) + 4 * align128(M), e.g. M = 2048
  * with K = 4096 fits, M = 4096 with K = 4096 does not) is rejected with RK_NPU_ERR_NOMEM
- * before any device work.  Device pointers in and out, work enqueued on the stream of the
+ * before any device work, and a shape whose partial tiles would not fit beside them runs
+ * without the K split.  Device pointers in and out, work enqueued on the stream of the
  * context the weights belong to, nothing waited for; results are bit-identical to
  * rk_npu_f16i8f16_run_dynamic_device.  All calls on one GPU share the one array: calls
  * through the same context are ordered on its stream, calls that overlap on one GPU through
