@@ -1,6 +1,8 @@
-"""Child process of tests/test_gpu_plan_override.py: decode-sized calls (1, 2, 4 and 8 rows) of every
+"""Child process of tests/test_gpu_plan_override.py: decode-sized calls (1 to 8 rows) of every
 operator with the columns per workgroup of the dot-product kernels forced by RK_NPU_HIP_GEMV_COLS
-(read once per process), checked against the oracle.  Prints OK <columns> on success."""
+(read once per process), checked against the oracle -- short rows, and rows long enough for the
+larger staging area, for several K chunks and for the chunk-wise scaling of int4 sums.  Prints
+OK <columns> on success."""
 import os
 import sys
 
@@ -69,6 +71,45 @@ def main():
         assert rc == 0 and np.array_equal(bits32(got), bits32(want32)), ("w4a8 host", M)
         for d in (dA32, dA16, dC):
             sess.free_device(d)
+        wsp.close()
+        w.close()
+    # Long rows: several rows that fill the larger staging area of the int8-weight kernels (one chunk,
+    # quantized by the kernel), rows beyond it (several chunks behind a quantization launch), fewer rows
+    # than the kernel's row count, and int4 weights over enough K chunks that the 16 x code sums are
+    # taken off chunk by chunk.
+    N = 72                                # 3 column blocks, the last one ragged
+    for M, K in ((4, 9000), (3, 12000), (8, 5000), (5, 20000), (7, 3000)):
+        A8 = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        B8 = rng.integers(-128, 128, (K, N)).astype(np.int8)
+        op = ops.W8A8Linear(sess, capi.I8I8I32, M, B8)
+        dA, dC = sess.to_device(A8), sess.empty_device(M * N * 4)
+        assert op.run_device(dA, dC) == 0 and sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.int32), oracle.gemm_i8(A8, B8)), ("long i8 device", M, K)
+        sess.free_device(dA)
+        sess.free_device(dC)
+        op.close()
+        c = workloads.w8a8_case(M, K, N, 11 + M, 12)
+        op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+        want = oracle.w8a8(c["A"], c["B"], c["w_scale"])["C"]
+        dA, dC = sess.to_device(c["A"]), sess.empty_device(M * N * 2)
+        assert op.run_device(dA, dC) == 0 and sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.uint16), want), ("long w8a8 device", M, K)
+        sess.free_device(dA)
+        sess.free_device(dC)
+        op.close()
+    for M, K in ((4, 70000), (6, 33000)):
+        B4 = np.full((K, N), -8, np.int8)
+        B4[::3] = 7
+        s4 = (rng.random(N).astype(np.float32) + 0.5) * np.float32(0.01)
+        w = ops.W4A8Weights(sess, B4, s4)
+        wsp = ops.W4A8Workspace(sess, M, N, K)
+        A16 = np.where(rng.random((M, K)) < 0.5, -1000.0, 1000.0).astype(np.float16).view(np.uint16)  # every code +-127
+        want16 = oracle.w4a8(A16, B4, s4)["C"]
+        dA16, dC = sess.to_device(A16), sess.empty_device(M * N * 2)
+        assert lib.rk_npu_w4a8_run_f16_device(wsp.h, w.h, dA16, dC) == 0 and sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.uint16), want16), ("long w4a8 f16 device", M, K)
+        sess.free_device(dA16)
+        sess.free_device(dC)
         wsp.close()
         w.close()
     sess.close()
