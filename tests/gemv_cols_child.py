@@ -78,7 +78,7 @@ def main():
     # than the kernel's row count, and int4 weights over enough K chunks that the 16 x code sums are
     # taken off chunk by chunk.
     N = 72                                # 3 column blocks, the last one ragged
-    for M, K in ((4, 9000), (3, 12000), (8, 5000), (5, 20000), (7, 3000)):
+    for M, K in ((4, 9000), (3, 10000), (8, 5000), (5, 6000), (5, 20000), (7, 3000)):
         A8 = rng.integers(-128, 128, (M, K)).astype(np.int8)
         B8 = rng.integers(-128, 128, (K, N)).astype(np.int8)
         op = ops.W8A8Linear(sess, capi.I8I8I32, M, B8)
@@ -89,14 +89,19 @@ def main():
         sess.free_device(dC)
         op.close()
         c = workloads.w8a8_case(M, K, N, 11 + M, 12)
-        op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
-        want = oracle.w8a8(c["A"], c["B"], c["w_scale"])["C"]
-        dA, dC = sess.to_device(c["A"]), sess.empty_device(M * N * 2)
-        assert op.run_device(dA, dC) == 0 and sess.sync() == 0
-        assert np.array_equal(sess.from_device(dC, (M, N), np.uint16), want), ("long w8a8 device", M, K)
-        sess.free_device(dA)
-        sess.free_device(dC)
-        op.close()
+        for kind, A, dtype in ((capi.F16I8F16_DYNAMIC, c["A"], np.uint16),
+                               (capi.F32I8F32_DYNAMIC, (rng.standard_normal((M, K)) * 2).astype(np.float32), np.float32)):
+            op = ops.W8A8Linear(sess, kind, M, c["B"], c["w_scale"])
+            want = oracle.w8a8(A, c["B"], c["w_scale"])["C"]
+            dA, dC = sess.to_device(A), sess.empty_device(M * N * 4)
+            assert op.run_device(dA, dC) == 0 and sess.sync() == 0
+            got = sess.from_device(dC, (M, N), dtype)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), ("long w8a8 device", kind, M, K)
+            rc, got = op.run(A)          # (host call: rows quantized by a launch of their own)
+            assert rc == 0 and np.array_equal(got.view(np.uint8), want.view(np.uint8)), ("long w8a8 host", kind, M, K)
+            sess.free_device(dA)
+            sess.free_device(dC)
+            op.close()
     for M, K in ((4, 70000), (6, 33000)):
         B4 = np.full((K, N), -8, np.int8)
         B4[::3] = 7
