@@ -35,6 +35,12 @@ __host__ __device__ constexpr bool gemv_big_applies(int mr, bool w4, long padded
 #define RK_GEMV_MFMA_ROWS 4
 #endif
 constexpr int GEMV_MFMA_ROWS = RK_GEMV_MFMA_ROWS; // from this many rows on the products go through the matrix cores
+#ifndef RK_GEMV_MFMA_ROWS_I8
+#define RK_GEMV_MFMA_ROWS_I8 2
+#endif
+// (the same for int8 weights: two rows already -- 4096 x 4096 6.2 -> 5.85 us, 14336 x 4096 14.3 -> 13.9; int4
+// weights pay for the unpacking, two rows 5.3 -> 6.4 us)
+constexpr int GEMV_MFMA_ROWS_I8 = RK_GEMV_MFMA_ROWS_I8;
 // 16-element activation chunks a thread may quantize in the fused path: four; eight for fp16 rows
 // (8 registers a chunk as fetched) in the BIG variants, which fills their staging area
 constexpr int GEMV_QCHUNKS = 4;
@@ -275,7 +281,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // of row l % CW at its k-half -- one LDS read and one MFMA per tile however many rows.  Rows
     // past MR read row MR - 1 again: column j of the product depends on column j of the second
     // operand only, and those columns are never stored.
-    constexpr bool MATRIX = MR >= GEMV_MFMA_ROWS && CW >= 16 && !(W4 && CW == 32);
+    constexpr bool MATRIX = MR >= (W4 ? GEMV_MFMA_ROWS : GEMV_MFMA_ROWS_I8) && CW >= 16 && !(W4 && CW == 32);
     constexpr int CREGS = CW == 32 ? 16 : 4;                // accumulator registers of the matrix path
     constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[gemv_lds_bytes(BIG) + A_PAD];
