@@ -62,15 +62,18 @@ typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 // Row / column block of logical dense tile `tile`: column sweeps over groups of
 // 4 row blocks, so that concurrently running tiles share weight columns in L2.
-__device__ __forceinline__ void wk_tile_coords(int tile, int mblocks, int nblocks, int& mblk, int& nblk) {
-    constexpr int GM = 4;
-    const int per_group = GM * nblocks;
-    const int group = tile / per_group;
-    const int first_m = group * GM;
-    const int gm = min(mblocks - first_m, GM);
-    const int in_group = tile - group * per_group;
-    mblk = first_m + in_group % gm;
-    nblk = in_group / gm;
+// (unsigned arithmetic: these divisions stand between a wave's start and its first load, and a
+// signed division by a run-time value is half as long again)
+__device__ __forceinline__ void wk_tile_coords(unsigned tile, unsigned mblocks, unsigned nblocks, int& mblk, int& nblk) {
+    constexpr unsigned GM = 4;
+    const unsigned per_group = GM * nblocks;
+    const unsigned group = tile / per_group;
+    const unsigned first_m = group * GM;
+    const unsigned gm = min(mblocks - first_m, GM);
+    const unsigned in_group = tile - group * per_group;
+    const unsigned col = in_group / gm;
+    mblk = (int)(first_m + in_group - col * gm);
+    nblk = (int)col;
 }
 
 #pragma clang diagnostic push
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
     // ---- tile assignment: XCD-contiguous ranges, 4 row blocks per column sweep
     const int tiles = mblocks * nblocks;
     const int logical = xcd_remap(blockIdx.x, tiles * ksplit);
-    const int kpart = logical / tiles;
+    const int kpart = ksplit > 1 ? (int)((unsigned)logical / (unsigned)tiles) : 0;
     const int tile = logical - kpart * tiles;
     int mblk, nblk;
     wk_tile_coords(tile, mblocks, nblocks, mblk, nblk);

@@ -64,6 +64,15 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
 
     [[maybe_unused]] constexpr int TSB = EPI == RKH_EPI_SWIGLU ? 4 : 0; // (debug stamps: the SwiGLU launch keeps its own slots)
     RK_TS(TSB + 0);
+    // Grouped: the block -> expert table (up to 64 row blocks, one entry per lane) is requested
+    // together with the number of live blocks, so that a wave knows its unit's expert one round trip
+    // after its start: read entry by entry, the expert waited for the block count and the first
+    // weight tile for the expert -- three dependent round trips ahead of the first data (3.7 us from
+    // a wave's start in the MoE layer of 256 tokens, against 2.6 us in a dense launch).  Entries of
+    // blocks that are not live hold whatever the last call left; they are never used.
+    int expert_of_lane = 0;
+    const bool table_in_lanes = g.blk_expert && mblocks <= 64;
+    if (table_in_lanes) expert_of_lane = g.blk_expert[min(lane, mblocks - 1)];
     // dense use (no block -> expert table): one weight matrix, every row block live
     const int live_blocks = g.blk_expert ? g.num_blocks[0] : mblocks;
 
@@ -71,7 +80,7 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // pair_pb0 (BAL) or the wave's pair of column tile nblk (otherwise).
     auto run_unit = [&](int mblk, int nblk, int pair_pb0) {
     if (mblk >= live_blocks) return;
-    const int e = g.blk_expert ? g.blk_expert[mblk] : 0;
+    const int e = !g.blk_expert ? 0 : table_in_lanes ? __builtin_amdgcn_readlane(expert_of_lane, mblk) : g.blk_expert[mblk];
     // grouped: this launch serves the experts held in its own format (int4 images come first in a bank)
     if (g.blk_expert && (e < g.int4_experts) != W4) return;
     const uint8_t* Wb = !g.blk_expert ? g.W
@@ -257,8 +266,9 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     }; // run_unit
 
     if constexpr (!BAL) {
-        const int logical = xcd_remap(blockIdx.x, mblocks * nblocks);
-        run_unit(logical % mblocks, logical / mblocks, 0);
+        const unsigned logical = (unsigned)xcd_remap(blockIdx.x, mblocks * nblocks);
+        const unsigned col_tile = logical / (unsigned)mblocks; // (one unsigned division ahead of the first load)
+        run_unit((int)(logical - col_tile * (unsigned)mblocks), (int)col_tile, 0);
     } else {
         // Balanced launch: one workgroup of eight waves per compute unit, the units (live row
         // block, column pair) dealt out in equal contiguous shares -- first to the dies (a
@@ -266,12 +276,14 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
         // by its workgroup's waves in turn.  Consecutive units are column pairs of one row block,
         // so the waves of a workgroup share the activation tiles through the L1, and the row
         // blocks of one expert meet in one die's L2.
-        const int pairs = (g.N + 63) / 64;
-        const long units = (long)live_blocks * pairs;
-        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = (int)(gridDim.x + 7 - xcd) >> 3;
-        const long die0 = units * xcd / 8, die1 = units * (xcd + 1) / 8;
-        const long first = die0 + (die1 - die0) * slot / slots, last = die0 + (die1 - die0) * (slot + 1) / slots;
-        for (long u = first + wave; u < last; u += WAVES) run_unit((int)(u / pairs), 0, (int)(u % pairs) * TN);
+        // (32-bit arithmetic: the launcher uses this variant only while 8 x the units fit; 64-bit
+        // divisions are a few hundred instructions between a wave's start and its first load)
+        const unsigned pairs = (unsigned)(g.N + 63) / 64;
+        const unsigned units = (unsigned)live_blocks * pairs;
+        const unsigned xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = (gridDim.x + 7 - xcd) >> 3;
+        const unsigned die0 = units * xcd / 8, die1 = units * (xcd + 1) / 8;
+        const unsigned first = die0 + (die1 - die0) * slot / slots, last = die0 + (die1 - die0) * (slot + 1) / slots;
+        for (unsigned u = first + wave; u < last; u += WAVES) run_unit((int)(u / pairs), 0, (int)(u % pairs) * TN);
     }
 }
 
@@ -316,6 +328,7 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     static const char* forced = getenv("RK_NPU_HIP_GROUPED");
     if (forced && forced[0] == 'b') balanced = grouped && moe_epilogue && cus > 0;
     if (forced && forced[0] == 't') balanced = false;
+    if ((long)mblocks * ((g.N + 63) / 64) > 0x0fffffffL) balanced = false; // (the kernel deals the units in 32-bit arithmetic)
     if (balanced) {
         mark(st, "gemm_stream_kernel<balanced>");
         const dim3 grid(cus), block(512);
