@@ -307,7 +307,12 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(RK_QUANT_HEAD_PARAMS, i
 __global__ __launch_bounds__(256) void requant_rows_wave_kernel(RK_QUANT_HEAD_PARAMS, rkh_quant_args a) {
     RK_QUANT_HEAD_APPLY(a);
     const int lane = lane_id(), m = blockIdx.x * 4 + wave_id();
-    if (m >= a.M || (a.active_blocks && m >= a.active_blocks[0] * 32)) return;
+    if (m >= a.M) return;
+    // (The count of live row blocks is requested with the row, not ahead of it: rows beyond the
+    // live blocks exist -- the buffers are sized for the most blocks a call can have -- so reading
+    // one is harmless, and the wave leaves before it writes anything.  Asked for first, the count
+    // cost every wave a round trip before its first row load.)
+    const int live_rows = a.active_blocks ? a.active_blocks[0] * 32 : a.M;
     const int K = a.K, KB = (int)(rkh_align_up(K, RKH_K_ALIGN) / 32);
     const int nchunks = (K + 15) >> 4;
     const float* row = static_cast<const float*>(a.src) + (size_t)m * K;
@@ -318,6 +323,7 @@ __global__ __launch_bounds__(256) void requant_rows_wave_kernel(RK_QUANT_HEAD_PA
         if (lane + 64 * i < nchunks) RowLoader<float>::load16(row, (lane + 64 * i) * 16, K, vec, v[i]);
     uint32_t bits = 0; // unsigned compare of |x| bit patterns
     for (int i = lane; i < a.row_max_parts; i += 64) bits = max(bits, a.row_max_bits[(size_t)m * a.row_max_parts + i]);
+    if (m >= live_rows) return;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
     const float mx = __uint_as_float(bits);
@@ -620,15 +626,34 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* h_Y, cons
     if (n >= a.H) return;
     const int slots = a.top_k + a.shared;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < slots; ++s) {
-        const int d = a.dest_rows[(size_t)tkn * slots + s];
-        if (d < 0) continue;
-        const float w = s < a.top_k ? a.routes[(size_t)tkn * a.top_k + s] : 1.0f;
-        const float4 y = *reinterpret_cast<const float4*>(a.Y + (size_t)d * a.H + n);
-        sum.x = fmaf(y.x, w, sum.x);
-        sum.y = fmaf(y.y, w, sum.y);
-        sum.z = fmaf(y.z, w, sum.z);
-        sum.w = fmaf(y.w, w, sum.w);
+    // Eight slots at a time: their destination rows and coefficients first, then the rows they name,
+    // then the sums in slot order.  Slot by slot the loop was a chain of two dependent round trips
+    // per slot (row index, then the row), 2.7 us for the four slots of a top-4 layer in a kernel
+    // that moves a few MB.
+    constexpr int B = 8;
+    for (int s0 = 0; s0 < slots; s0 += B) {
+        int d[B];
+        float w[B];
+        float4 y[B];
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            const int s = s0 + j;
+            d[j] = s < slots ? a.dest_rows[(size_t)tkn * slots + s] : -1;
+            w[j] = s < a.top_k ? a.routes[(size_t)tkn * a.top_k + s] : 1.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            y[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (d[j] >= 0) y[j] = *reinterpret_cast<const float4*>(a.Y + (size_t)d[j] * a.H + n);
+        }
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            if (d[j] < 0) continue;
+            sum.x = fmaf(y[j].x, w[j], sum.x);
+            sum.y = fmaf(y[j].y, w[j], sum.y);
+            sum.z = fmaf(y[j].z, w[j], sum.z);
+            sum.w = fmaf(y[j].w, w[j], sum.w);
+        }
     }
     *reinterpret_cast<float4*>(a.out + (size_t)tkn * a.H + n) = sum;
 }
