@@ -714,7 +714,21 @@ __device__ __forceinline__ v4i moe_load_tile(const uint8_t* block, int idx, int 
 
 constexpr int MOE_DECODE_PREFETCH = 4; // tiles per wave and column block requested ahead of the quantization
 
-__global__ __launch_bounds__(512) void moe_decode_gate_kernel(rkh_moe_decode_args a) {
+// (Leading scalar arguments, in registers when a wave starts: what the first loads of both kernels
+// depend on -- the routing arrays, the token rows, the middle rows.  Read from the argument
+// structure they cost every wave a round trip to memory ahead of the routing entries.)
+#define RK_MOE_DECODE_HEAD_PARAMS                                                                       \
+    const float* h_x, const int32_t* h_ids, const float* h_routes, int h_top_k, int h_experts, int h_shared, int h_H, \
+        int h_I, float* h_hidden, uint32_t* h_row_max_bits
+#define RK_MOE_DECODE_HEAD(a) (a).x, (a).ids, (a).routes, (a).top_k, (a).experts, (a).shared, (a).H, (a).I, (a).hidden, (a).row_max_bits
+#define RK_MOE_DECODE_HEAD_APPLY(a)                                                                     \
+    do {                                                                                                \
+        (a).x = h_x; (a).ids = h_ids; (a).routes = h_routes; (a).top_k = h_top_k; (a).experts = h_experts; \
+        (a).shared = h_shared; (a).H = h_H; (a).I = h_I; (a).hidden = h_hidden; (a).row_max_bits = h_row_max_bits; \
+    } while (0)
+
+__global__ __launch_bounds__(512) void moe_decode_gate_kernel(RK_MOE_DECODE_HEAD_PARAMS, rkh_moe_decode_args a) {
+    RK_MOE_DECODE_HEAD_APPLY(a);
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[MOE_DECODE_MAX_K];
     __shared__ int red[2][8][32];
     __shared__ float wave_max[8];
@@ -837,7 +851,8 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(rkh_moe_decode_arg
 constexpr int MOE_DECODE_SLOTS = ROUTE_MAX_TOPK + 1;
 constexpr int MOE_DECODE_DOWN_K = 3584; // longest middle row (padded): nine of them fit the staging area
 static_assert(MOE_DECODE_SLOTS * MOE_DECODE_DOWN_K <= MOE_DECODE_MAX_K, "staging area");
-__global__ __launch_bounds__(512) void moe_decode_down_kernel(rkh_moe_decode_args a) {
+__global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD_PARAMS, rkh_moe_decode_args a) {
+    RK_MOE_DECODE_HEAD_APPLY(a);
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[MOE_DECODE_MAX_K]; // live slot i at i * Ip
     __shared__ int red[MOE_DECODE_SLOTS][8][32];
     __shared__ float live_scale[MOE_DECODE_SLOTS], live_coeff[MOE_DECODE_SLOTS];
@@ -847,18 +862,18 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(rkh_moe_decode_arg
     const int pb = blockIdx.x, t = blockIdx.y;
     const int tid = threadIdx.x, lane = lane_id(), wave = wave_id(), half = lane >> 5;
     const int I = a.I, Ip = (int)rkh_align_up(I, RKH_K_ALIGN), nchunks = I >> 4, parts = I / 32;
-    if (tid == 0) { // the live slots in slot order
-        int n = 0;
-        for (int s = 0; s < slots; ++s) {
-            const MoeSlot slot = moe_slot(a, t, s);
-            if (slot.live) {
-                live_expert[n] = slot.expert;
-                live_coeff[n] = slot.coeff;
-                live_slot[n] = s;
-                ++n;
-            }
+    if (wave == 0) { // the live slots in slot order: lane s reads slot s, a live slot's place is its rank among them
+        // (one thread walking the slots was a chain of as many round trips to the routing arrays)
+        MoeSlot slot = {0, 0.0f, false, false};
+        if (lane < slots) slot = moe_slot(a, t, lane);
+        const unsigned long long live_mask = __ballot(slot.live);
+        if (slot.live) {
+            const int n = __popcll(live_mask & ((1ull << lane) - 1ull));
+            live_expert[n] = slot.expert;
+            live_coeff[n] = slot.coeff;
+            live_slot[n] = lane;
         }
-        live_count = n;
+        if (lane == 0) live_count = __popcll(live_mask);
     }
     __syncthreads();
     const int nlive = live_count;
@@ -1407,9 +1422,11 @@ int rkh_moe_decode(void* stream, const rkh_moe_decode_args* args) {
     if (!rkh_moe_decode_applies(a.rows, a.H, a.I) || a.top_k < 1) return RKH_ERR_RUNTIME;
     const int slots = a.top_k + (a.shared ? 1 : 0);
     mark((hipStream_t)stream, "moe_decode_gate_kernel");
-    hipLaunchKernelGGL(moe_decode_gate_kernel, dim3(a.I / 32, a.rows * slots), dim3(512), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(moe_decode_gate_kernel, dim3(a.I / 32, a.rows * slots), dim3(512), 0, (hipStream_t)stream,
+                       RK_MOE_DECODE_HEAD(a), a);
     mark((hipStream_t)stream, "moe_decode_down_kernel");
-    hipLaunchKernelGGL(moe_decode_down_kernel, dim3(a.H / 32, a.rows), dim3(512), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(moe_decode_down_kernel, dim3(a.H / 32, a.rows), dim3(512), 0, (hipStream_t)stream,
+                       RK_MOE_DECODE_HEAD(a), a);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
