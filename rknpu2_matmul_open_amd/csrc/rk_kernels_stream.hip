@@ -31,11 +31,14 @@ namespace {
 // bank may hold int4 and int8 experts (routed INT4, shared int8): each format
 // has its launch over the same grid, and a workgroup whose row block belongs to
 // an expert of the other format exits at once.
-template <int EPI, int KS, bool W4, bool BAL = false>
+template <int EPI, int KS, bool W4, bool BAL = false, int TN = 2>
 __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HEAD_PARAMS, int mblocks, int nblocks,
                                                                       rkh_gemm_args g) {
     RK_GEMM_HEAD_APPLY(g);
-    constexpr int TN = 2, WAVES = BAL ? 8 : 4;
+    constexpr int WAVES = BAL ? 8 : 4;
+    // TN: 32-column blocks per wave.  Two; one for small launches whose K is split over the waves
+    // (32-column tiles: twice the workgroups where 64-column tiles leave most compute units idle).
+    static_assert(TN == 2 || (TN == 1 && KS > 1 && !BAL && EPI != RKH_EPI_SWIGLU), "one column block per wave: small K-split launches");
     constexpr bool KSPLIT = KS > 1;
     static_assert(!BAL || !KSPLIT, "the balanced variant does not split K");
     constexpr int CG = WAVES / KS; // column pairs per workgroup
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
         } else {
             const bool live = g.interleave_F ? pb < g.N / 32 : pb * 32 < g.N;
             n = block_first_col(pb, g.interleave_F) + (lane & 31);
-            ws_ok = live && n < g.N;
+            ws_ok = live && n < g.N && (lane >> 5) < TN;
         }
         as_ok = m < m_limit;
         const float* pa = g.a_scale + (as_ok ? m : 0);
@@ -256,7 +259,7 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // loop takes 14 us, 1.9 us for the plain fp32 tile pair.  A dry pass through the same code
     // while the first loads were in flight, to have it in the instruction cache, changed nothing.)
     if constexpr (EPI == RKH_EPI_SWIGLU) {
-        epilogue_swiglu_scaled(g, acc[0], acc[1], m0, pb0, lane, as, ws[0], ws[1], m_limit, stage_lds);
+        epilogue_swiglu_scaled(g, acc[0], acc[TN - 1], m0, pb0, lane, as, ws[0], ws[TN - 1], m_limit, stage_lds);
     } else {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -313,7 +316,14 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     const int mblocks = grouped ? g.max_blocks : (g.M + 31) / 32;
     const long wide = (long)mblocks * ((g.N + 255) / 256);
     const int ks = wide < (grouped ? GROUPED_KS4_BELOW : DENSE_KS4_BELOW) ? 4 : 1;
-    const int cols = 256 / ks;
+    // 64-column tiles with K split over the waves; 32-column tiles while even twice as many workgroups
+    // leave compute units without one (a compute unit draws 55 GB/s however few of them work: 64 rows of
+    // 2048 x 2048 are 64 workgroups of 192 KB or 128 of 128 KB).  RK_NPU_HIP_STREAM_NARROW=0 switches it off
+    // (tuning aid).
+    static const char* narrow_env = getenv("RK_NPU_HIP_STREAM_NARROW");
+    const bool narrow = ks == 4 && g.epilogue != RKH_EPI_SWIGLU && !(narrow_env && narrow_env[0] == '0') &&
+                        compute_units() > 0 && 2L * mblocks * ((g.N + 63) / 64) <= compute_units();
+    const int cols = narrow ? 32 : 256 / ks;
     const int nblocks = (g.N + cols - 1) / cols;
     // Many row blocks (a prefill-sized MoE call): the balanced launch, one workgroup per compute
     // unit.  With a workgroup per (row block, column tile) the 392 workgroups of a 256-token,
@@ -347,9 +357,16 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
         return RKH_OK;
     }
     const dim3 grid(mblocks * nblocks), block(256);
-    mark(st, ks == 4 ? "gemm_stream_kernel<KS=4>" : "gemm_stream_kernel");
+    mark(st, narrow ? "gemm_stream_kernel<KS=4, 32 columns>" : ks == 4 ? "gemm_stream_kernel<KS=4>" : "gemm_stream_kernel");
 #define RK_LAUNCH(EPI)                                                                                         \
     do {                                                                                                       \
+        if constexpr (EPI != RKH_EPI_SWIGLU) {                                                                 \
+            if (narrow) {                                                                                      \
+                if (any_int4) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true, false, 1>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);  \
+                if (any_int8) hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, false, false, 1>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); \
+                break;                                                                                         \
+            }                                                                                                  \
+        }                                                                                                      \
         if (any_int4 && ks == 4)                                                                               \
             hipLaunchKernelGGL((gemm_stream_kernel<EPI, 4, true>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g);   \
         else if (any_int4)                                                                                     \
