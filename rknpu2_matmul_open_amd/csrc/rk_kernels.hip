@@ -361,6 +361,10 @@ __global__ __launch_bounds__(256) void requant_rows_wave_kernel(RK_QUANT_HEAD_PA
 // it holds several workgroups: 4 rows are used while 8 would leave fewer than
 // two workgroups per compute unit.
 // Modes: dynamic W8 / W4A8 maxima or a given static scale; rows written in place.
+// (Holding fp16 rows as fetched -- 8 registers a chunk, twice the reach -- with the maxima taken
+// from the bit patterns was built and measured: rows of 11008 at 1024 rows 19.7 -> 15.7 us, but at
+// 256 / 512 rows slower than a workgroup per row, 12.7 / 15.1 against 9.9 / 13.3 us, and the
+// 2048 x 4096 case 0.5 us slower, so rows are held as floats.)
 constexpr int Q8_CACHE = 8;
 
 template <typename T, int ROWS>
@@ -1208,9 +1212,14 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     if (args->M <= 0) return RKH_OK;
     const dim3 block(256);
     const int mode = args->mode;
-    if (args->M >= 256 && !args->active_blocks && args->in_dtype != RKH_I8 &&
+    // Several rows per workgroup only while a row fits the registers its threads hold it in (8 rows:
+    // 4096 elements, 4 rows: 8192): longer rows are read twice in a loop, and 256 rows of 11008 then
+    // took 15 us where a workgroup per row takes 6.5.
+    const int row_chunks = (args->K + 15) / 16;
+    const bool fits8 = row_chunks <= (256 / 8) * Q8_CACHE, fits4 = row_chunks <= (256 / 4) * Q8_CACHE;
+    if (args->M >= 256 && !args->active_blocks && args->in_dtype != RKH_I8 && fits4 &&
         (mode == RKH_Q_W8_DYNAMIC || mode == RKH_Q_W4A8 || mode == RKH_Q_W8_STATIC)) {
-        const bool rows4 = args->M < 8 * 2 * 256; // 8 rows would give fewer than two workgroups per compute unit
+        const bool rows4 = !fits8 || args->M < 8 * 2 * 256; // 8 rows would give fewer than two workgroups per compute unit
         const dim3 grid(rows4 ? (args->M + 3) / 4 : (args->M + 7) / 8);
         const hipStream_t st = (hipStream_t)stream;
         mark(st, "quant_rows8_kernel");
@@ -1236,7 +1245,6 @@ int rkh_quant_rows(void* stream, const rkh_quant_args* args) {
     // each, until the grid has a few hundred workgroups.
     int split = 1;
     if (reuse) {
-        const int row_chunks = (args->K + 15) / 16;
         while (split < 8 && args->M * split < 512 && row_chunks / (split * 2) >= 128) split *= 2;
     }
     const dim3 grid(args->M * split);
