@@ -855,16 +855,23 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(RK_MOE_DECODE_HEAD
 constexpr int MOE_DECODE_SLOTS = ROUTE_MAX_TOPK + 1;
 constexpr int MOE_DECODE_DOWN_K = 3584; // longest middle row (padded): nine of them fit the staging area
 static_assert(MOE_DECODE_SLOTS * MOE_DECODE_DOWN_K <= MOE_DECODE_MAX_K, "staging area");
+// CW = output columns per workgroup: 32, or 16 / 8 while that many workgroups still leave compute
+// units without one (one token of a 2048-wide layer: 64 workgroups of 32 columns) -- a load then
+// covers the workgroup's part of 32 / CW consecutive tiles, as in the decode GEMV.
+template <int CW>
 __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD_PARAMS, rkh_moe_decode_args a) {
     RK_MOE_DECODE_HEAD_APPLY(a);
+    constexpr int TPL = 32 / CW; // tiles covered by one load instruction
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[MOE_DECODE_MAX_K]; // live slot i at i * Ip
-    __shared__ int red[MOE_DECODE_SLOTS][8][32];
+    __shared__ int red[MOE_DECODE_SLOTS][8][CW];
     __shared__ float live_scale[MOE_DECODE_SLOTS], live_coeff[MOE_DECODE_SLOTS];
     __shared__ int live_expert[MOE_DECODE_SLOTS], live_slot[MOE_DECODE_SLOTS];
     __shared__ int live_count;
     const int slots = a.top_k + a.shared;
-    const int pb = blockIdx.x, t = blockIdx.y;
-    const int tid = threadIdx.x, lane = lane_id(), wave = wave_id(), half = lane >> 5;
+    const int pb = blockIdx.x / TPL, col0 = ((int)blockIdx.x % TPL) * CW, t = blockIdx.y;
+    const int tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+    const int half = (lane / CW) & 1, sub = lane / (2 * CW); // k-half of a tile, tile of the load
+    const unsigned lane_byte = (unsigned)((col0 + lane % CW) + 32 * half) * 16u;
     const int I = a.I, Ip = (int)rkh_align_up(I, RKH_K_ALIGN), nchunks = I >> 4, parts = I / 32;
     if (wave == 0) { // the live slots in slot order: lane s reads slot s, a live slot's place is its rank among them
         // (one thread walking the slots was a chain of as many round trips to the routing arrays)
@@ -895,7 +902,11 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
         int tiles;
         const uint8_t* wb = block_of(li, int4, tiles);
 #pragma unroll
-        for (int u = 0; u < PF; ++u) regs[u] = moe_load_tile(wb, (grp * PF + u) * 8 + wave, tiles, lane);
+        for (int u = 0; u < PF; ++u) {
+            const int tile = ((grp * PF + u) * 8 + wave) * TPL + sub;
+            regs[u] = tile < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + (size_t)tile * 1024 + lane_byte))
+                                   : v4i{0, 0, 0, 0};
+        }
     };
     v4i cur[PF], nxt[PF];
     if (nlive > 0) load_group(0, 0, cur);
@@ -940,7 +951,7 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
         bool int4;
         int tiles;
         block_of(li, int4, tiles);
-        const int groups = (tiles + 8 * PF - 1) / (8 * PF);
+        const int groups = ((tiles + TPL - 1) / TPL + 8 * PF - 1) / (8 * PF);
         const uint8_t* codes = a_lds + (size_t)li * Ip;
         int acc = 0;
         for (int grp = 0; grp < groups; ++grp) {
@@ -949,18 +960,20 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
             else if (li + 1 < nlive) load_group(li + 1, 0, nxt);
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
-                const int idx = (grp * PF + u) * 8 + wave;
-                if (idx < tiles) moe_dot_tile(int4, codes, idx, half, cur[u], acc);
+                const int tile = ((grp * PF + u) * 8 + wave) * TPL + sub;
+                if (tile < tiles) moe_dot_tile(int4, codes, tile, half, cur[u], acc);
             }
 #pragma unroll
             for (int u = 0; u < PF; ++u) cur[u] = nxt[u];
         }
         acc += __shfl_xor(acc, 32);
-        if (lane < 32) red[li][wave][lane] = acc;
+        if (CW <= 16) acc += __shfl_xor(acc, 16);
+        if (CW <= 8) acc += __shfl_xor(acc, 8);
+        if (lane < CW) red[li][wave][lane] = acc;
     }
     __syncthreads();
-    if (tid < 32) {
-        const int n = pb * 32 + tid; // (H is a multiple of 32)
+    if (tid < CW) {
+        const int n = pb * 32 + col0 + tid; // (H is a multiple of 32)
         float sum = 0.0f;
         for (int li = 0; li < nlive; ++li) {
             int acc = 0;
@@ -1433,8 +1446,14 @@ int rkh_moe_decode(void* stream, const rkh_moe_decode_args* args) {
     hipLaunchKernelGGL(moe_decode_gate_kernel, dim3(a.I / 32, a.rows * slots), dim3(512), 0, (hipStream_t)stream,
                        RK_MOE_DECODE_HEAD(a), a);
     mark((hipStream_t)stream, "moe_decode_down_kernel");
-    hipLaunchKernelGGL(moe_decode_down_kernel, dim3(a.H / 32, a.rows), dim3(512), 0, (hipStream_t)stream,
-                       RK_MOE_DECODE_HEAD(a), a);
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    const long down_wgs = (long)(a.H / 32) * a.rows; // (with 32 columns each)
+    if (down_wgs * 4 <= cus)
+        hipLaunchKernelGGL(moe_decode_down_kernel<8>, dim3(a.H / 8, a.rows), dim3(512), 0, (hipStream_t)stream, RK_MOE_DECODE_HEAD(a), a);
+    else if (down_wgs * 2 <= cus)
+        hipLaunchKernelGGL(moe_decode_down_kernel<16>, dim3(a.H / 16, a.rows), dim3(512), 0, (hipStream_t)stream, RK_MOE_DECODE_HEAD(a), a);
+    else
+        hipLaunchKernelGGL(moe_decode_down_kernel<32>, dim3(a.H / 32, a.rows), dim3(512), 0, (hipStream_t)stream, RK_MOE_DECODE_HEAD(a), a);
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
 }
