@@ -320,6 +320,10 @@ def bench_c1w4(sess, ops, capi, workloads, steps, warmup):
            "weight_GBps": weight_bytes / step_us / 1e3, "ms_per_step": step_us / 1e3,
            "roofline": _hbm("gemv_kernel<1,true,1,32> (fused per-token quantize + int4 GEMV)", algo_bytes, step_us,
                             "gemv_c1w4", kernel_us=step_us)}
+    # the timed call against the CPU oracle: all 14336 fp16 outputs
+    step()
+    out["parity_vs_oracle"] = bool(np.array_equal(sess.from_device(dC, (M, N), np.uint16),
+                                                  _oracle().w4a8(c["A"], c["B"], c["w_scale"])["C"]))
     sess.free_device(dA)
     sess.free_device(dC)
     ws.close()

@@ -72,6 +72,7 @@ using rkk::gemv_can_fuse;
 using rkk::gemv_max_rows;
 using rkk::gemv_swiglu_applies;
 using rkk::launch_gemm_grouped;
+using rkk::launch_gemm_rows64;
 using rkk::wk_scratch_bytes;
 
 // ------------------------------------------------------------------ fill
@@ -1358,6 +1359,28 @@ static bool dense_streams(const rkh_gemm_args& g) {
     return !g.w_int4 || g.K <= 131072;
 }
 
+// A few hundred rows on int8 weights, while tiles of 64 rows x 128 columns still give every compute
+// unit at most one: the streaming kernel with two row blocks per wave (K split over two waves, no
+// second launch) instead of the LDS-ring kernel with its K split over workgroups and the reduce
+// launch behind it.  Measured, fp16 in / out, quantization included, us: 4096 x 4096 at 192 / 256 /
+// 384 / 512 rows 25.1 / 28.4 / 28.2 / 28.4 -> 23.0 / 23.1 / 24.1 / 24.9; 4096 x 11008 at 192 rows 31.1 ->
+// 27.7.  It loses where the tiles outnumber the compute units (4096 x 4096 at 768 rows 30.8 -> 35.8:
+// operands straight to registers are 1 KiB through the compute unit's 64 B / clock memory path per
+// MFMA, twice what the matrix pipes can wait for), for a long K (11008 x 4096 at 192 rows 33.4 -> 48.3:
+// there the other kernel's K split pays) and with int4 weights (everywhere by 1 - 10 us).
+// RK_NPU_HIP_ROWS64 = 0 switches it off, 1 forces it for every dense int8 GEMM beyond the streaming
+// kernel's rows (tuning aid).
+static bool dense_rows64(const rkh_gemm_args& g) {
+    if (g.blk_expert || g.w_int4 || g.epilogue == RKH_EPI_SWIGLU) return false;
+    static const char* forced = getenv("RK_NPU_HIP_ROWS64");
+    if (forced && forced[0]) return forced[0] == '1';
+    static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the LDS-ring kernel)
+    if (plan && plan[0]) return false;
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    const long tiles = (long)((g.M + 63) / 64) * ((g.N + 127) / 128);
+    return g.K <= 6144 && tiles <= cus + cus / 50;
+}
+
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
     if (M <= 8) return 0;
     const DensePlan plan = effective_plan(M, N, K, w_int4);
@@ -1373,6 +1396,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     if (gemv_swiglu_applies(g) && gemv_ok) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
+    if (dense_rows64(g)) return launch_gemm_rows64(st, g);
     const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {

@@ -31,11 +31,16 @@ namespace {
 // bank may hold int4 and int8 experts (routed INT4, shared int8): each format
 // has its launch over the same grid, and a workgroup whose row block belongs to
 // an expert of the other format exits at once.
-template <int EPI, int KS, bool W4, bool BAL = false, int TN = 2>
+template <int EPI, int KS, bool W4, bool BAL = false, int TN = 2, int TM = 1>
 __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HEAD_PARAMS, int mblocks, int nblocks,
                                                                       rkh_gemm_args g) {
     RK_GEMM_HEAD_APPLY(g);
     constexpr int WAVES = BAL ? 8 : 4;
+    // TM: 32-row blocks per wave.  One; two for dense GEMMs of a few hundred rows (`mblocks` then
+    // counts units of TM row blocks): a weight tile in registers is multiplied with both blocks'
+    // activation tiles, so a workgroup pulls K x (64 rows + its columns) bytes through its compute
+    // unit for twice the products -- tiles of 64 x 128, K split over two waves.
+    static_assert(TM == 1 || (TM == 2 && !BAL && TN == 2 && EPI != RKH_EPI_SWIGLU), "two row blocks per wave: dense launches");
     // TN: 32-column blocks per wave.  Two; one for small launches whose K is split over the waves
     // (32-column tiles: twice the workgroups where 64-column tiles leave most compute units idle).
     static_assert(TN == 2 || (TN == 1 && KS > 1 && !BAL && EPI != RKH_EPI_SWIGLU), "one column block per wave: small K-split launches");
@@ -52,12 +57,13 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // grouped calls): four -- a wave walks the whole K alone, 128 steps for K = 4096, and with two
     // it waits out a full memory latency per step: int8 128 x 4096 x 11008 took 37.9 us with 2,
     // 25.5 with 4, 25.9 with 8 (x 14336: 39.1 / 27.2 / 28.3).
+    // (two row blocks per wave: four as well -- six and eight steps measured the same or slower)
     constexpr int RING = KSPLIT ? 4 : BAL ? 2 : 4;
     constexpr int AT = W4 ? 2 : 1;   // activation tiles per step
-    constexpr int LPS = AT + TN;
+    constexpr int LPS = AT * TM + TN; // loads per step: TM activation tiles (int4: pairs), TN weight tiles
     static_assert((RING - 1) * LPS <= 63, "vmcnt field");
     constexpr int STAGE_BYTES = WAVES * 32 * (32 * 4 + 8);
-    constexpr int XCH_BYTES = KSPLIT ? CG * (KS - 1) * TN * 16 * 64 * 4 : 0;
+    constexpr int XCH_BYTES = KSPLIT ? CG * (KS - 1) * TM * TN * 16 * 64 * 4 : 0;
     __shared__ __attribute__((aligned(16))) uint8_t stage_raw[STAGE_BYTES + XCH_BYTES];
 
     const int lane = lane_id();
@@ -100,7 +106,8 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // interleave 6.4)
     const int kts = KB > kq ? (KB - kq + KS - 1) / KS : 0;
     const int kt0 = min(kq, KB - 1); // (a wave without a share still loads in bounds)
-    const uint8_t* asrc = g.A + ((size_t)mblk * KB + kt0) * (1024 * AT);
+    const size_t rb_stride = (size_t)KB * (1024 * AT); // bytes from a row block of the activations to the next
+    const uint8_t* asrc = g.A + ((size_t)mblk * TM * KB + kt0) * (1024 * AT);
     const uint8_t* wsrc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) wsrc[j] = Wb + ((size_t)(pb0 + j) * KB + kt0) * 1024;
@@ -113,12 +120,12 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // it a round trip to memory (an epilogue of 2.8 us instead of 1.4, of a kernel whose loop
     // takes 7).  Lane l holds the row scale of row l % 32 and the column scale of column l % 32
     // of column block l / 32 of the pair.
-    const int m0 = mblk * 32;
+    const int m0 = mblk * TM * 32;
     const int m_limit = g.blk_expert ? live_blocks * 32 : g.M;
     float my_as = 0.0f, my_ws = 0.0f;
     bool as_ok = false, ws_ok = false;
     if constexpr (EPI != RKH_EPI_I32) {
-        const int m = m0 + (lane & 31);
+        const int m = m0 + (TM == 2 ? lane : (lane & 31)); // (two row blocks: lanes 32.. hold the second one's)
         const int pb = pb0 + (lane >> 5);
         int n;
         if constexpr (EPI == RKH_EPI_SWIGLU) { // pb0 is even: the gate block, its up block right behind it
@@ -137,18 +144,20 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
         asm volatile("global_load_dword %0, %1, off" : "=v"(my_ws) : "v"(pw));
     }
 
-    v16i acc[TN];
+    v16i acc[TM][TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
-    v4i ring[RING][LPS]; // [0 .. AT) = activation tiles, [AT + j] = weights of column block j
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    v4i ring[RING][LPS]; // [i * AT .. (i + 1) * AT) = activation tiles of row block i, [AT * TM + j] = weights of column block j
 
     auto issue = [&](v4i* regs) {
         static_for<LPS>([&](auto l_tag) {
             constexpr int L = decltype(l_tag)::value;
             const unsigned off = lane_off; // (locals: asm operands cannot name captures of an enclosing lambda)
-            const uint8_t* base = L < AT ? asrc + L * 1024 : wsrc[L < AT ? 0 : L - AT];
+            const uint8_t* base = L < AT * TM ? asrc + (L / AT) * rb_stride + (L % AT) * 1024 : wsrc[L < AT * TM ? 0 : L - AT * TM];
             v4i r;
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
             regs[L] = r;
@@ -182,15 +191,20 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     if constexpr (W4) {
-                        const v4i raw = ring[SLOT][AT + j];
+                        const v4i raw = ring[SLOT][AT * TM + j];
                         const v4i lo = v4i{(raw.x << 4) & (int)0xF0F0F0F0, raw.x & (int)0xF0F0F0F0,
                                            (raw.y << 4) & (int)0xF0F0F0F0, raw.y & (int)0xF0F0F0F0};
                         const v4i hi = v4i{(raw.z << 4) & (int)0xF0F0F0F0, raw.z & (int)0xF0F0F0F0,
                                            (raw.w << 4) & (int)0xF0F0F0F0, raw.w & (int)0xF0F0F0F0};
-                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, ring[SLOT][0], acc[j], 0, 0, 0);
-                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, ring[SLOT][AT - 1], acc[j], 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < TM; ++i) {
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, ring[SLOT][i * AT], acc[i][j], 0, 0, 0);
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, ring[SLOT][i * AT + AT - 1], acc[i][j], 0, 0, 0);
+                        }
                     } else {
-                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][AT + j], ring[SLOT][0], acc[j], 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < TM; ++i)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[SLOT][AT * TM + j], ring[SLOT][i * AT], acc[i][j], 0, 0, 0);
                     }
                 }
             }
@@ -209,44 +223,54 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
 
     if constexpr (KSPLIT) {
         // the other parts of K hand their accumulators to part 0: [column pair][part - 1][tile][q][lane] x 4 ints
-        int* xch = reinterpret_cast<int*>(stage_raw + STAGE_BYTES) + cg * (KS - 1) * TN * 16 * 64;
+        // (tiles of a wave counted i * TN + j)
+        int* xch = reinterpret_cast<int*>(stage_raw + STAGE_BYTES) + cg * (KS - 1) * TM * TN * 16 * 64;
         if (kq > 0) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<v4i*>(xch + ((((kq - 1) * TN + j) * 4 + q) * 64 + lane) * 4) =
-                        v4i{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        *reinterpret_cast<v4i*>(xch + ((((kq - 1) * TM * TN + i * TN + j) * 4 + q) * 64 + lane) * 4) =
+                            v4i{acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
         }
         __syncthreads();
         if (kq > 0) return;
 #pragma unroll
         for (int w = 0; w < KS - 1; ++w)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const v4i got = *reinterpret_cast<const v4i*>(xch + (((w * TN + j) * 4 + q) * 64 + lane) * 4);
-                    acc[j][q * 4] += got.x;
-                    acc[j][q * 4 + 1] += got.y;
-                    acc[j][q * 4 + 2] += got.z;
-                    acc[j][q * 4 + 3] += got.w;
-                }
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const v4i got = *reinterpret_cast<const v4i*>(xch + (((w * TM * TN + i * TN + j) * 4 + q) * 64 + lane) * 4);
+                        acc[i][j][q * 4] += got.x;
+                        acc[i][j][q * 4 + 1] += got.y;
+                        acc[i][j][q * 4 + 2] += got.z;
+                        acc[i][j][q * 4 + 3] += got.w;
+                    }
     }
     if constexpr (W4) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[j][r] >>= 4;
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] >>= 4;
     }
     uint8_t* stage_lds = stage_raw + wave * (32 * (32 * 4 + 8));
-    float as = 0.0f, ws[TN][16];
+    float as[TM], ws[TN][16];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) as[i] = 0.0f;
     if constexpr (EPI != RKH_EPI_I32) { // scales: lane-wise registers -> the wave's staging area -> per-lane order
         float* sc = reinterpret_cast<float*>(stage_lds);
         sc[lane] = ws_ok ? my_ws : 0.0f;
-        if (lane < 32) sc[64 + lane] = as_ok ? my_as : 0.0f;
+        if (lane < 32 * TM) sc[64 + lane] = as_ok ? my_as : 0.0f;
         __builtin_amdgcn_wave_barrier();
-        as = sc[64 + (lane & 31)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) as[i] = sc[64 + i * 32 + (lane & 31)];
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -259,11 +283,13 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
     // loop takes 14 us, 1.9 us for the plain fp32 tile pair.  A dry pass through the same code
     // while the first loads were in flight, to have it in the instruction cache, changed nothing.)
     if constexpr (EPI == RKH_EPI_SWIGLU) {
-        epilogue_swiglu_scaled(g, acc[0], acc[TN - 1], m0, pb0, lane, as, ws[0], ws[TN - 1], m_limit, stage_lds);
+        epilogue_swiglu_scaled(g, acc[0][0], acc[0][TN - 1], m0, pb0, lane, as[0], ws[0], ws[TN - 1], m_limit, stage_lds);
     } else {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-            epilogue_tile_scaled<EPI>(g, acc[j], m0, pb0 + j, lane, as, ws[j], m_limit, stage_lds);
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                epilogue_tile_scaled<EPI>(g, acc[i][j], m0 + i * 32, pb0 + j, lane, as[i], ws[j], m_limit, stage_lds);
     }
     RK_TS(TSB + 3);
     }; // run_unit
@@ -388,10 +414,29 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     return RKH_OK;
 }
 
+// Dense int8 GEMMs of a few hundred rows: two row blocks per wave, tiles of 64 rows x 128 columns, K split
+// over two waves.  (Tiles of 64 x 256 without the K split and int4 weights were measured as well and
+// lose to the LDS-ring kernel on every shape, so they are not compiled.)
+int launch_gemm_rows64(hipStream_t st, const rkh_gemm_args& g) {
+    if (g.blk_expert || g.w_int4 || g.epilogue == RKH_EPI_SWIGLU) return RKH_ERR_RUNTIME;
+    const int mblocks = (g.M + 63) / 64, nblocks = (g.N + 127) / 128;
+    const dim3 grid(mblocks * nblocks), block(256);
+    mark(st, "gemm_stream_kernel<64 x 128>");
+    switch (g.epilogue) {
+    case RKH_EPI_I32: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_I32, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
+    case RKH_EPI_F16: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_F16, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
+    case RKH_EPI_F32: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_F32, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
+    default: return RKH_ERR_RUNTIME;
+    }
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
 } // namespace
 
 namespace rkk {
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_grouped(st, g); }
+int launch_gemm_rows64(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_rows64(st, g); }
 #ifdef RK_DEBUG_TS
 void set_ts_stream(unsigned long long* p) { (void)hipMemcpyToSymbol(HIP_SYMBOL(rk_dbg_ts), &p, sizeof(p)); }
 #endif
