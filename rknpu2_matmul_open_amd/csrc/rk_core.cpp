@@ -112,7 +112,7 @@ void HostStage::init(size_t bytes) {
     if (rkh_host_alloc(&p, bytes) != RKH_OK) return;
     ptr_ = p;
     bytes_ = bytes;
-    if (bytes > kLimit) {
+    if (bytes > kLimit) { // (a mirror that may serve staged downloads)
         const size_t chunks = (bytes + kChunk - 1) / kChunk;
         for (size_t i = 0; i < chunks; ++i) {
             void* e = nullptr;

@@ -189,6 +189,11 @@ private:
 class HostStage {
 public:
     static constexpr size_t kLimit = size_t(1) << 20;
+    // Results of the W8A8 and MoE calls are written in place up to 4 MiB: the reference's bench_llm_i8 at 128
+    // rows (2 MiB of int32) 158 -> 143 us (4096 x 4096), 201 -> 183 us (11008 x 4096), the MoE layer of 256
+    // tokens 281 -> 262 us; 8 MiB and more lose (5.6 MiB of int32: 290 -> 340 - 390 us), and the W4A8 calls
+    // keep the input's limit (the FFN's 2 MiB of fp32 written in place: 510 -> 560 us).
+    static constexpr size_t kOutLimit = size_t(4) << 20;
     static constexpr size_t kPipeLimit = size_t(64) << 20;
     static constexpr size_t kChunk = size_t(2) << 20;
     HostStage() = default;
@@ -198,6 +203,7 @@ public:
     void init(size_t bytes);        // stays off for 0 or more than kPipeLimit bytes
     explicit operator bool() const { return ptr_ != nullptr; }
     bool direct(size_t bytes) const { return ptr_ && bytes <= bytes_ && bytes <= kLimit; }
+    bool direct_out(size_t bytes) const { return ptr_ && bytes <= bytes_ && bytes <= kOutLimit; }
     // direct use: the mirror filled with `bytes` from `user` (kernels read it in place) ...
     const void* fill(const void* user, size_t bytes) const;
     // ... and the mirror as a kernel's output; finish() copies it on to `user` after the wait.

@@ -90,7 +90,7 @@ int execute(rk_npu_i4_workspace* ws, const rk_npu_i4i4i32_weights* w, const int8
     const rk_npu_i4_config& c = ws->config;
     rk_npu_ctx* ctx = ws->owner.ctx;
     const size_t c_bytes = (size_t)c.M * c.N * sizeof(int32_t);
-    const bool direct_in = ws->stage_a.direct((size_t)c.M * c.K), direct_out = ws->stage_c.direct(c_bytes);
+    const bool direct_in = ws->stage_a.direct((size_t)c.M * c.K), direct_out = ws->stage_c.direct_out(c_bytes);
     int rc;
     auto start = Clock::now();
     {

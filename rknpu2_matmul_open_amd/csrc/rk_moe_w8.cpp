@@ -331,7 +331,7 @@ int moe_run(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w, int row
     // The routing table is read by every token's workgroup: in place only for a
     // decode-sized call, otherwise uploaded (from its mirror, without a wait).
     const size_t in_bytes = values * (f32 ? 4 : 1), out_bytes = values * 4;
-    const bool direct_in = ws->stage_in.direct(in_bytes), direct_out = ws->stage_out.direct(out_bytes);
+    const bool direct_in = ws->stage_in.direct(in_bytes), direct_out = ws->stage_out.direct_out(out_bytes);
     const bool direct_route = ws->stage_route && rows <= 16;
     const void* d_input = ws->input.as<>();
     const float* d_scales = ws->token_scale.as<float>();

@@ -189,7 +189,7 @@ int run_host(rk_npu_matmul_workspace* ws, const Weights* w, rk_npu_matmul_op_kin
     // Small operands skip the copies: the kernels read A from / write C into the
     // pinned mirrors.  Static scales are read by every workgroup of the GEMM, so
     // they are always uploaded (from their mirror when there is one).
-    const bool direct_in = ws->stage_a.direct(a_bytes), direct_out = ws->stage_c.direct(c_bytes);
+    const bool direct_in = ws->stage_a.direct(a_bytes), direct_out = ws->stage_c.direct_out(c_bytes);
     const size_t scale_bytes = (size_t)s.M * sizeof(float);
     // the mirrors are filled before the context's submission lock is taken
     const void* src = direct_in ? ws->stage_a.fill(A, a_bytes) : ws->a_raw.as<>();
