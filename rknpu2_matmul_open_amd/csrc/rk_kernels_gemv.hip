@@ -899,13 +899,14 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 // Whether the streaming MFMA kernel can take this dense GEMM at all (int4 codes ride as 16 * code).
 bool dense_stream_fits(const rkh_gemm_args& g) { return !g.w_int4 || g.K <= 131072; }
 
-// Most rows the dot-product kernels take for this matrix: eight, but four on a matrix of more than
+// Most rows the decode kernels take for this matrix: eight, but four on an int4 matrix of more than
 // 256 column blocks, where five to eight rows are faster as one 32-row block of the streaming MFMA
-// kernel behind a quantization launch (fp16 rows, every step from HBM, dot products against
-// stream, us: 4096 x 11008 int8 17.2 - 20.5 against 15.3 - 15.5, int4 15.5 - 18.9 against 12.3 - 12.5;
-// 4096 x 14336 18.8 - 21.9 against 16.2 - 16.5, int4 16.1 - 19.3 against 12.8 - 12.9; on narrower
-// matrices the dot products win: 4096 x 4096 9.5 - 11.6 against 13.6, 11008 x 4096 22.6 against 27.3;
-// up to four rows they win everywhere).  RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
+// kernel behind a quantization launch (fp16 rows, every step from HBM, dot products against stream,
+// us: 4096 x 11008 int4 15.5 - 18.9 against 12.3 - 12.5; 4096 x 14336 16.1 - 19.3 against 12.8 - 12.9).
+// On int8 matrices that was so too while the rows were multiplied by dot products (4096 x 14336
+// 18.8 - 21.9 against 16.2 - 16.5); with the products on the matrix cores the decode kernel keeps them:
+// five to eight rows 16.3 -> 12.6 - 14.7 us (4096 x 14336), 15.3 -> 12.2 - 14.1 (4096 x 11008).
+// RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
 int gemv_max_rows(const rkh_gemm_args& g) {
     static const int rows = [] {
         const char* e = getenv("RK_NPU_HIP_GEMV_MAX_ROWS");
@@ -913,7 +914,7 @@ int gemv_max_rows(const rkh_gemm_args& g) {
         return v >= 1 && v <= 8 ? v : 8;
     }();
     const bool wide = (g.N + 31) / 32 > 256;
-    return wide && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
+    return wide && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
 }
 
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {
