@@ -280,8 +280,10 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     // v_mfma_i32_16x16x64_i8), and the staged rows are the second one: lane l reads the 16 bytes
     // of row l % CW at its k-half -- one LDS read and one MFMA per tile however many rows.  Rows
     // past MR read row MR - 1 again: column j of the product depends on column j of the second
-    // operand only, and those columns are never stored.
-    constexpr bool MATRIX = MR >= (W4 ? GEMV_MFMA_ROWS : GEMV_MFMA_ROWS_I8) && CW >= 16 && !(W4 && CW == 32);
+    // operand only, and those columns are never stored.  (Int4 weights, 32 columns: the eight-row
+    // instantiation only -- the four-row one spills with the unpacked operands, so it keeps the dot
+    // products and the launcher sends three and four rows of a wide matrix to the eight-row kernel.)
+    constexpr bool MATRIX = MR >= (W4 ? GEMV_MFMA_ROWS : GEMV_MFMA_ROWS_I8) && CW >= 16 && !(W4 && CW == 32 && MR < 8);
     constexpr int CREGS = CW == 32 ? 16 : 4;                // accumulator registers of the matrix path
     constexpr int A_PAD = ROLLING ? GEMV_WAVES * (UNR + 1) * TPL * (W4 ? 64 : 32) : 0;
     __shared__ __attribute__((aligned(16))) uint8_t a_lds[gemv_lds_bytes(BIG) + A_PAD];
@@ -340,32 +342,45 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
     FusedRows<QT_T, MR, BIG> rows;
-    if constexpr (FUSEQ) {
-        const int tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
-        if constexpr (BURST) {
+    // Several rows: the first group of weight tiles is requested a quarter at a time, between the
+    // prologue's barriers.  Requested all at once (as for one row) the sixteen waves of a compute unit
+    // ask for 256 KB, more than its memory path holds in flight: a wave's later requests wait at issue
+    // until earlier data has arrived, and the prologue's first barrier, which every wave reaches only
+    // behind its last request, came 1.9 us later than with one row (in-kernel time stamps, two rows,
+    // 4096 x 14336 int4: 4.8 against 3.0 us after the start).
+#ifndef RK_GEMV_PRE_STAGES
+#define RK_GEMV_PRE_STAGES 4
+#endif
+    constexpr int STAGES = (FUSEQ && MR > 1 && !BURST) ? RK_GEMV_PRE_STAGES : 1;
+    static_assert(UNR % STAGES == 0, "whole tiles per stage");
+    const int pre_tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
+    auto prefetch_stage = [&](int stage) {
 #pragma unroll
-            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        for (int u = 0; u < UNR / STAGES; ++u)
+            wpre[stage * (UNR / STAGES) + u] = load_tile(wave + (stage * (UNR / STAGES) + u) * GEMV_WAVES, pre_tiles, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    (void)prefetch_stage;
+    if constexpr (FUSEQ) {
+        if constexpr (BURST) prefetch_stage(0);
         rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!BURST) {
-#pragma unroll
-            for (int u = 0; u < UNR; ++u) wpre[u] = load_tile(wave + u * GEMV_WAVES, tiles, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        if constexpr (!BURST) prefetch_stage(0);
         RK_TS(4);
     }
     if constexpr (FUSEQ) {
         if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
         __syncthreads();
         RK_TS(5);
+        if constexpr (STAGES >= 2) prefetch_stage(1);
         const bool bad = rows.maxima(g.M, g.K, row_max);
         __syncthreads();
+        if constexpr (STAGES >= 4) prefetch_stage(2);
         rows.scales(g.M, q.mode, row_max, row_scale, row_inv, first_wg ? q.scale : nullptr);
         if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
         rows.zero_padding(g.M, g.K, Kp, a_lds);
         __syncthreads();
+        if constexpr (STAGES >= 4) prefetch_stage(3);
         rows.template quantize<W4 && !MATRIX>(g.M, g.K, Kp, row_inv, a_lds, first_wg ? q.dst : nullptr);
         // a_scale of the epilogue comes from LDS in this path
         RK_TS(1);
@@ -559,19 +574,27 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
+            // (int4 tiles on the matrix cores take two LDS reads and eight unpacked registers each: left
+            // to itself the scheduler gathers the reads of a whole group up front and spills)
+            constexpr bool FENCED = MATRIX && W4;
             if constexpr (FUSEQ) {
 #pragma unroll
-                for (int u = 0; u < UNR; ++u)
+                for (int u = 0; u < UNR; ++u) {
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(wpre[u], tb + u * GEMV_WAVES);
+                    if constexpr (FENCED) __builtin_amdgcn_sched_barrier(0);
+                }
                 tb += GEMV_WAVES * UNR;
             }
             for (; tb < tiles; tb += GEMV_WAVES * UNR) {
                 v4i w[UNR];
 #pragma unroll
                 for (int u = 0; u < UNR; ++u) w[u] = load_unit(tb + u * GEMV_WAVES);
+                if constexpr (FENCED) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int u = 0; u < UNR; ++u)
+                for (int u = 0; u < UNR; ++u) {
                     if (tb + u * GEMV_WAVES < tiles) consume_unit(w[u], tb + u * GEMV_WAVES);
+                    if constexpr (FENCED) __builtin_amdgcn_sched_barrier(0);
+                }
             }
             }
         }
@@ -667,34 +690,56 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
     const __amdgpu_buffer_rsrc_t wrsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)(2 * block_bytes), 0x00020000);
     v4i w[2][GEMV_SWIGLU_UNROLL];
+    auto load_pair = [&](int u, int tb, int tiles, int tile0) { // tile u of the group: its gate and its up block
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int tt = tb + u * GEMV_WAVES;
+            const unsigned off = tt < tiles ? (unsigned)(b * block_bytes) + (unsigned)(tile0 + tt) * 1024u + (unsigned)lane * 16u
+                                            : 0xFFFFFFF0u;
+            w[b][u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
+        }
+    };
     auto load_group = [&](int tb, int tiles, int tile0) {
 #pragma unroll
-        for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u)
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const int tt = tb + u * GEMV_WAVES;
-                const unsigned off = tt < tiles ? (unsigned)(b * block_bytes) + (unsigned)(tile0 + tt) * 1024u + (unsigned)lane * 16u
-                                                : 0xFFFFFFF0u;
-                w[b][u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)off, 0, 2 /* streaming */));
-            }
+        for (int u = 0; u < GEMV_SWIGLU_UNROLL; ++u) load_pair(u, tb, tiles, tile0);
     };
 
     if constexpr (QT != 0) { // (the fused path has a single K chunk: rows fit the staging area)
         using T = typename std::conditional<QT == 2, float, uint16_t>::type;
         const bool first_wg = blockIdx.x == 0;
         FusedRows<T, MR, false> rows;
+        // (the first group of weight tiles a quarter at a time between the barriers, as in gemv_kernel)
+#ifndef RK_GEMV_SWIGLU_STAGED
+#define RK_GEMV_SWIGLU_STAGED 1
+#endif
+        constexpr bool STAGED = RK_GEMV_SWIGLU_STAGED != 0;
+        static_assert(GEMV_SWIGLU_UNROLL == 4, "one tile pair per stage");
+        const int pre_tiles = W4 ? Kp >> 6 : Kp >> 5;
         rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
-        load_group(wave, W4 ? Kp >> 6 : Kp >> 5, 0);
+        if constexpr (STAGED) load_pair(0, wave, pre_tiles, 0);
+        else load_group(wave, pre_tiles, 0);
         __builtin_amdgcn_sched_barrier(0);
         if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
         __syncthreads();
+        if constexpr (STAGED) {
+            load_pair(1, wave, pre_tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         const bool bad = rows.maxima(g.M, g.K, row_max);
         __syncthreads();
+        if constexpr (STAGED) {
+            load_pair(2, wave, pre_tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         rows.scales(g.M, q.mode, row_max, row_scale, row_inv, first_wg ? q.scale : nullptr);
         if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
         rows.zero_padding(g.M, g.K, Kp, a_lds);
         __syncthreads();
+        if constexpr (STAGED) {
+            load_pair(3, wave, pre_tiles, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         rows.template quantize<W4>(g.M, g.K, Kp, row_inv, a_lds, first_wg ? q.dst : nullptr);
     }
 
@@ -887,10 +932,28 @@ int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant
     return launch_gemv_swiglu<2>(st, g, fuse);
 }
 
+// An int4 matrix of more than 256 column blocks whose rows fit the staging area eight at a time: from
+// three rows on the eight-row instantiation, the only 32-column int4 one whose products go through the
+// matrix cores (the four-row one would spill).  4096 x 14336, fp16 rows, us, four-row dot products /
+// streaming MFMA kernel -> eight-row kernel: three rows 9.5 -> 8.65, four 10.3 -> 9.3, five 11.3 -> 9.95,
+// six 11.3 -> 10.85; eight rows stay on the streaming kernel (11.5 against 12.3), two on the dot products
+// (7.7 against 8.0).
+constexpr int GEMV_W4_WIDE_ROWS = 7; // (seven: a tie)
+static bool w4_wide_eight(const rkh_gemm_args& g) {
+    return (g.N + 31) / 32 > 256 && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU &&
+           rkh_align_up(g.K, RKH_K_ALIGN) * 8 <= (size_t)GEMV_LDS_BYTES;
+}
+// Rows of the kernel instantiation that takes the M rows of g.
+int gemv_mr(const rkh_gemm_args& g) {
+    if (g.M >= 3 && w4_wide_eight(g)) return 8;
+    return g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
+}
+
 int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
-    if (g.M == 1) return launch_gemv<1>(st, g, fuse);
-    if (g.M == 2) return launch_gemv<2>(st, g, fuse);
-    if (g.M <= 4) return launch_gemv<4>(st, g, fuse);
+    const int mr = gemv_mr(g);
+    if (mr == 1) return launch_gemv<1>(st, g, fuse);
+    if (mr == 2) return launch_gemv<2>(st, g, fuse);
+    if (mr == 4) return launch_gemv<4>(st, g, fuse);
     return launch_gemv<8>(st, g, fuse);
 }
 
@@ -906,6 +969,8 @@ bool dense_stream_fits(const rkh_gemm_args& g) { return !g.w_int4 || g.K <= 1310
 // On int8 matrices that was so too while the rows were multiplied by dot products (4096 x 14336
 // 18.8 - 21.9 against 16.2 - 16.5); with the products on the matrix cores the decode kernel keeps them:
 // five to eight rows 16.3 -> 12.6 - 14.7 us (4096 x 14336), 15.3 -> 12.2 - 14.1 (4096 x 11008).
+// A wide int4 matrix whose rows fit the staging area eight at a time keeps up to seven rows as well, on
+// the eight-row kernel (see gemv_mr).
 // RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
 int gemv_max_rows(const rkh_gemm_args& g) {
     static const int rows = [] {
@@ -914,6 +979,7 @@ int gemv_max_rows(const rkh_gemm_args& g) {
         return v >= 1 && v <= 8 ? v : 8;
     }();
     const bool wide = (g.N + 31) / 32 > 256;
+    if (w4_wide_eight(g)) return min(rows, GEMV_W4_WIDE_ROWS);
     return wide && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
 }
 
@@ -924,7 +990,7 @@ bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu 
     if (q.in_dtype == RKH_I8) return q.mode == RKH_Q_COPY_I8 && !g.w_int4 && !swiglu;
     if (q.mode != RKH_Q_W8_DYNAMIC && q.mode != RKH_Q_W4A8) return false;
     if (q.in_dtype != RKH_F16 && q.in_dtype != RKH_F32) return false;
-    const int mr = g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
+    const int mr = gemv_mr(g);
     const long kp = (long)rkh_align_up(g.K, RKH_K_ALIGN);
     const bool big = !swiglu && gemv_big_applies(mr, g.w_int4 != 0, kp); // (the SwiGLU kernel keeps the small area)
     if (kp * mr > gemv_lds_bytes(big)) return false;

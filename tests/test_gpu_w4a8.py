@@ -41,7 +41,10 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           (1, 1, 1), (2500, 3, 2), (1, 70001, 64), (9, 70001, 40), (300, 30000, 70),
           # 64-row tiles of the large-tile kernel; K split over workgroups + reduce launch; two / three rows
           # on a wide matrix
-          (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200)]
+          (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200),
+          # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), four-row
+          # dot products beyond
+          (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
