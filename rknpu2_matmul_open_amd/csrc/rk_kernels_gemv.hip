@@ -241,7 +241,9 @@ struct FusedRows {
 // again), the column scales of the epilogue fetched with the first loads (10.7), a first group
 // of 4 / 6 / 10 / 12 tiles per wave with the rest in one group behind the prologue (11.8 / 11.1 /
 // 11.0 / 11.6), four tiles per group throughout (11.4), the exact-wait kernel with four loads
-// per wave in flight (10.7), 28 instead of 32 columns per workgroup (512 workgroups, two for
+// per wave in flight (10.7), the exact-wait kernel with its first eight loads in four stages between
+// the prologue's barriers, the first stage ahead of the row, as the int4 single-row kernel has them
+// (10.6: the same; twelve / sixteen loads in stages 11.4 / spills), 28 instead of 32 columns per workgroup (512 workgroups, two for
 // every compute unit, instead of 448 -- 11.85 us; the per-lane addresses this needs cost 0.4 us
 // already with 32 columns).
 template <int MR, bool W4, int QT, int CW, bool BURST = false, bool BIG = false>
@@ -254,12 +256,13 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     static_assert(QT != 3 || !W4, "int8 rows as given: the exact int8 x int8 product only");
     // Load instructions of a wave in flight.  One row, exact waits: four -- the quantization
     // prologue and the first dot products start after half as many bytes, and nothing is gained
-    // by queueing more in front of the memory system (4096 x 14336 int4: 7.25 -> 6.8 us; int4
-    // 4096 x 4096 4.9 -> 4.1, 4096 x 11008 7.0 -> 6.6, 8192 x 1024 5.1 -> 4.5; int8 2048 x 2048
-    // 4.2 -> 3.6, 14336 x 4096 12.8 -> 12.5, the other int8 shapes within 1 %).  Several rows
-    // and the burst variant are faster with eight (two rows lose 2 - 9 % with four on most
-    // shapes; the burst variant 10.6 -> 11.4 us).
-    constexpr int UNR = (MR == 1 && !BURST) ? 4 : GEMV_UNROLL;
+    // by queueing more in front of the memory system (int4 4096 x 4096 4.9 -> 4.1, 4096 x 11008
+    // 7.0 -> 6.6, 8192 x 1024 5.1 -> 4.5; int8 2048 x 2048 4.2 -> 3.6, 14336 x 4096 12.8 -> 12.5, the
+    // other int8 shapes within 1 %).  Several rows and the burst variant are faster with eight (two
+    // rows lose 2 - 9 % with four on most shapes; the burst variant 10.6 -> 11.4 us), and so is one
+    // row on 32-column workgroups when it quantizes the row itself and requests the eight in
+    // stages (see STAGES below).
+    constexpr int UNR = (MR == 1 && !BURST && !(FUSEQ && CW == 32)) ? 4 : GEMV_UNROLL;
     static_assert(!BURST || (MR == 1 && !W4 && CW == 32), "the burst variant serves one int8 row, whole column blocks");
     static_assert(!BIG || (MR >= 4 && !W4), "the larger staging area: four to eight rows, int8 weights");
     constexpr int TPL = 32 / CW;            // k-tiles (int4: super-tiles) covered by one load instruction
@@ -334,7 +337,7 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 
     // Fused path: put the first batch of weight loads in flight before the
     // quantization prologue so that its latency hides behind them.
-    // The activation rows are requested FIRST: loads return in issue order, so
+    // The activation rows are requested ahead of a whole batch: loads return in issue order, so
     // behind the weight loads they would arrive with the last of those, and the
     // prologue (and with it the second batch of weight loads) would start only
     // then.  Fetched first they are back after one L2 round trip and the whole
@@ -342,16 +345,20 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     v4i wpre[UNR];
     using QT_T = typename std::conditional<QT == 2, float, uint16_t>::type;
     FusedRows<QT_T, MR, BIG> rows;
-    // Several rows: the first group of weight tiles is requested a quarter at a time, between the
-    // prologue's barriers.  Requested all at once (as for one row) the sixteen waves of a compute unit
-    // ask for 256 KB, more than its memory path holds in flight: a wave's later requests wait at issue
-    // until earlier data has arrived, and the prologue's first barrier, which every wave reaches only
-    // behind its last request, came 1.9 us later than with one row (in-kernel time stamps, two rows,
-    // 4096 x 14336 int4: 4.8 against 3.0 us after the start).
-#ifndef RK_GEMV_PRE_STAGES
-#define RK_GEMV_PRE_STAGES 4
-#endif
-    constexpr int STAGES = (FUSEQ && MR > 1 && !BURST) ? RK_GEMV_PRE_STAGES : 1;
+    // A batch of eight tiles is requested a quarter at a time, between the prologue's barriers.
+    // Requested all at once the sixteen waves of a compute unit ask for 256 KB, more than its memory
+    // path holds in flight: a wave's later requests wait at issue until earlier data has arrived, and
+    // the prologue's first barrier, which every wave reaches only behind its last request, came 1.9 us
+    // later than with four tiles (in-kernel time stamps, two rows, 4096 x 14336 int4: 4.8 against 3.0
+    // us after the start).  In stages, fp16 rows, us: 4096 x 14336 int8 two / four / eight rows 12.0 ->
+    // 11.05 / 12.1 -> 11.55 / 15.4 -> 14.0, int4 8.4 -> 7.55 / 10.8 -> 9.2 / 13.5 -> 12.5; 4096 x 4096 int8
+    // 5.77 -> 5.25 / 6.8 -> 5.8 / 8.8 -> 7.4.  One row on 32-column int4 workgroups (eight tiles are all
+    // of K = 4096 there): 6.75 -> 6.5 us, and 6.2 with the first quarter requested ahead of the row
+    // (two tiles delay the row by little and are on their way a microsecond earlier; with several
+    // rows that order loses 3 - 8 %).  Unequal stages (4-2-1-1, 3-3-1-1, 1-3-2-2, 4-4-0-0) measured
+    // 6.3 - 6.7 against 6.2, and the single-row kernels of narrow matrices (four tiles in a rolling
+    // window) lose 2 - 5 % with stages.
+    constexpr int STAGES = (FUSEQ && !BURST && UNR == GEMV_UNROLL) ? 4 : 1;
     static_assert(UNR % STAGES == 0, "whole tiles per stage");
     const int pre_tiles = (W4 ? Kp >> 6 : Kp >> 5) / TPL;
     auto prefetch_stage = [&](int stage) {
@@ -362,10 +369,11 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
     };
     (void)prefetch_stage;
     if constexpr (FUSEQ) {
-        if constexpr (BURST) prefetch_stage(0);
+        constexpr bool W_FIRST = BURST || (STAGES > 1 && MR == 1);
+        if constexpr (W_FIRST) prefetch_stage(0);
         rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!BURST) prefetch_stage(0);
+        if constexpr (!W_FIRST) prefetch_stage(0);
         RK_TS(4);
     }
     if constexpr (FUSEQ) {
@@ -708,38 +716,29 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
         using T = typename std::conditional<QT == 2, float, uint16_t>::type;
         const bool first_wg = blockIdx.x == 0;
         FusedRows<T, MR, false> rows;
-        // (the first group of weight tiles a quarter at a time between the barriers, as in gemv_kernel)
-#ifndef RK_GEMV_SWIGLU_STAGED
-#define RK_GEMV_SWIGLU_STAGED 1
-#endif
-        constexpr bool STAGED = RK_GEMV_SWIGLU_STAGED != 0;
+        // (the first group of weight tiles a quarter at a time between the barriers, as in gemv_kernel:
+        // a whole 4096 -> 14336 -> 4096 FFN of one / two rows 20.55 -> 19.9 / 24.4 -> 23.3 us; the first
+        // quarter ahead of the row changes nothing here)
         static_assert(GEMV_SWIGLU_UNROLL == 4, "one tile pair per stage");
         const int pre_tiles = W4 ? Kp >> 6 : Kp >> 5;
         rows.fetch(q.src, g.M, g.K);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (STAGED) load_pair(0, wave, pre_tiles, 0);
-        else load_group(wave, pre_tiles, 0);
+        load_pair(0, wave, pre_tiles, 0);
         __builtin_amdgcn_sched_barrier(0);
         if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
         __syncthreads();
-        if constexpr (STAGED) {
-            load_pair(1, wave, pre_tiles, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        load_pair(1, wave, pre_tiles, 0);
+        __builtin_amdgcn_sched_barrier(0);
         const bool bad = rows.maxima(g.M, g.K, row_max);
         __syncthreads();
-        if constexpr (STAGED) {
-            load_pair(2, wave, pre_tiles, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        load_pair(2, wave, pre_tiles, 0);
+        __builtin_amdgcn_sched_barrier(0);
         rows.scales(g.M, q.mode, row_max, row_scale, row_inv, first_wg ? q.scale : nullptr);
         if (first_wg && bad && q.mode == RKH_Q_W4A8 && q.bad_flag) atomicOr(q.bad_flag, 1);
         rows.zero_padding(g.M, g.K, Kp, a_lds);
         __syncthreads();
-        if constexpr (STAGED) {
-            load_pair(3, wave, pre_tiles, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        load_pair(3, wave, pre_tiles, 0);
+        __builtin_amdgcn_sched_barrier(0);
         rows.template quantize<W4>(g.M, g.K, Kp, row_inv, a_lds, first_wg ? q.dst : nullptr);
     }
 
