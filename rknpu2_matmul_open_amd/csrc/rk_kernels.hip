@@ -741,39 +741,65 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(RK_MOE_DECODE_HEAD
     const int slots = a.top_k + a.shared;
     const int j = blockIdx.x, asg = blockIdx.y, t = asg / slots, s = asg - t * slots;
     const int tid = threadIdx.x, lane = lane_id(), wave = wave_id(), half = lane >> 5;
+    const int H = a.H, Hp = (int)rkh_align_up(H, RKH_K_ALIGN), nchunks = (H + 15) >> 4;
+
+    // ---- the token row is requested first: its address depends on nothing but the block index,
+    // so it travels together with the routing entry instead of behind the first weight tiles
+    // (loads return in issue order)
+    const float* row = a.x + (size_t)t * H;
+    const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+    constexpr int CACHE = MOE_DECODE_MAX_K / 16 / 512; // chunks per thread
+    float v[CACHE][16];
+#pragma unroll
+    for (int i = 0; i < CACHE; ++i) {
+        const int c = tid + i * 512;
+        if (c < nchunks) RowLoader<float>::load16(row, c * 16, H, vec, v[i]);
+    }
     const MoeSlot slot = moe_slot(a, t, s);
     const bool reporter = j == 0 && tid == 0;
     if (slot.bad && reporter && a.bad_flag) atomicOr(a.bad_flag, 1);
     if (!slot.live) return;
 
-    // ---- gate block 2j and up block 2j + 1 of the expert: the first tiles are requested now
-    const int H = a.H, Hp = (int)rkh_align_up(H, RKH_K_ALIGN), nchunks = (H + 15) >> 4;
+    // ---- gate block 2j and up block 2j + 1 of the expert.  Two groups of PF tiles per wave and
+    // block are in flight: the first is requested now, the second when the token is quantized (one
+    // token per call gained 0.3 us with the second group requested between the barriers of the
+    // quantization, four and eight tokens lost 1.5 and 3.5 us).  The loads are unconditional -- past
+    // the end of the block a wave reads its last tile again and does not use it -- so that the
+    // compiler counts them and the quantization waits for the row only, not for the tiles.
+    // Against the first group requested ahead of the row, behind branches, and the rest in the
+    // loop: 17.8 -> 15.7 / 24.1 -> 23.8 / 37.3 -> 35.9 us for one / four / eight tokens (both launches).
     const int e = slot.expert;
     const bool int4 = e < a.int4_experts;
     const int tiles = int4 ? Hp / 64 : Hp / 32; // per column block
     const size_t block_bytes = (size_t)tiles * 1024;
     const uint8_t* wb = (int4 ? a.gate_W4 + (size_t)e * a.gate_stride4
                               : a.gate_W + (size_t)(e - a.int4_experts) * a.gate_stride) + (size_t)(2 * j) * block_bytes;
-    v4i pre[2][MOE_DECODE_PREFETCH];
+    constexpr int PF = MOE_DECODE_PREFETCH;
+    v4i cur[2][PF], nxt[2][PF];
+    auto load_group = [&](v4i (*regs)[PF], int grp) {
 #pragma unroll
-    for (int u = 0; u < MOE_DECODE_PREFETCH; ++u)
+        for (int u = 0; u < PF; ++u) {
+            const int idx = min(wave + 8 * (grp * PF + u), tiles - 1);
 #pragma unroll
-        for (int b = 0; b < 2; ++b) pre[b][u] = moe_load_tile(wb + b * block_bytes, wave + 8 * u, tiles, lane);
+            for (int b = 0; b < 2; ++b)
+                regs[b][u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + b * block_bytes + (size_t)idx * 1024 + lane * 16));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    load_group(cur, 0);
+    // (the two column scales of the epilogue ride behind the first group)
+    const float* ws = a.gate_scales + (size_t)e * 2 * a.I;
+    const int n = j * 32 + (tid & 31); // (I is a multiple of 32)
+    const float ws_gate = ws[n], ws_up = ws[a.I + n];
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- the token as int8 codes in LDS (s = max > 0 ? max / 127 : 1, ties to even)
-    const float* row = a.x + (size_t)t * H;
-    const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
-    constexpr int CACHE = MOE_DECODE_MAX_K / 16 / 512; // chunks per thread
-    float v[CACHE][16];
     float mx = 0.0f;
     float taint = 0.0f; // (NaN once an Inf or a NaN was seen, see absmax16)
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
         const int c = tid + i * 512;
-        if (c < nchunks) {
-            RowLoader<float>::load16(row, c * 16, H, vec, v[i]);
-            absmax16(v[i], mx, taint);
-        }
+        if (c < nchunks) absmax16(v[i], mx, taint);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
@@ -801,19 +827,27 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(RK_MOE_DECODE_HEAD
     }
     for (int c = nchunks + tid; c < Hp / 16; c += 512) *reinterpret_cast<uint4*>(a_lds + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
     __syncthreads();
+    load_group(nxt, 1);
 
     // ---- dot products: the waves take the tiles of both blocks in turn
     int acc[2] = {0, 0};
+    const int groups = (tiles + 8 * PF - 1) / (8 * PF);
+    for (int grp = 0; grp < groups; ++grp) {
 #pragma unroll
-    for (int u = 0; u < MOE_DECODE_PREFETCH; ++u)
+        for (int u = 0; u < PF; ++u) {
+            const int idx = wave + 8 * (grp * PF + u);
+            if (idx < tiles) {
+                moe_dot_tile(int4, a_lds, idx, half, cur[0][u], acc[0]);
+                moe_dot_tile(int4, a_lds, idx, half, cur[1][u], acc[1]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
-            if (wave + 8 * u < tiles) moe_dot_tile(int4, a_lds, wave + 8 * u, half, pre[b][u], acc[b]);
-#pragma unroll 2
-    for (int idx = wave + 8 * MOE_DECODE_PREFETCH; idx < tiles; idx += 8) {
-        const v4i w0 = moe_load_tile(wb, idx, tiles, lane), w1 = moe_load_tile(wb + block_bytes, idx, tiles, lane);
-        moe_dot_tile(int4, a_lds, idx, half, w0, acc[0]);
-        moe_dot_tile(int4, a_lds, idx, half, w1, acc[1]);
+        for (int u = 0; u < PF; ++u) {
+            cur[0][u] = nxt[0][u];
+            cur[1][u] = nxt[1][u];
+        }
+        if (grp + 2 < groups) load_group(nxt, grp + 2); // (uniform)
     }
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
@@ -833,12 +867,8 @@ __global__ __launch_bounds__(512) void moe_decode_gate_kernel(RK_MOE_DECODE_HEAD
             gate >>= 4;
             up >>= 4;
         }
-        const int n = j * 32 + tid; // (I is a multiple of 32)
-        // (fetched here, not with the first tiles: requested early the two scales made the kernel a
-        // third slower for four and eight tokens)
-        const float* ws = a.gate_scales + (size_t)e * 2 * a.I;
-        const float gf = dequant(gate, scale, ws[n]);
-        const float uf = dequant(up, scale, ws[a.I + n]);
+        const float gf = dequant(gate, scale, ws_gate);
+        const float uf = dequant(up, scale, ws_up);
         const float y = __fmul_rn(silu_poly(gf), uf);
         a.hidden[(size_t)asg * a.I + n] = y;
         uint32_t bits = __float_as_uint(y) & 0x7fffffffu;
@@ -898,26 +928,30 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
         return (int4 ? a.down_W4 + (size_t)e * a.down_stride4
                      : a.down_W + (size_t)(e - a.int4_experts) * a.down_stride) + (size_t)pb * tiles * 1024;
     };
+    // (unconditional loads -- past the end of a block a lane reads the block's last tile again and does
+    // not use it -- so that the compiler counts them: a wait for older data then leaves them in flight)
     auto load_group = [&](int li, int grp, v4i* regs) {
         bool int4;
         int tiles;
         const uint8_t* wb = block_of(li, int4, tiles);
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            const int tile = ((grp * PF + u) * 8 + wave) * TPL + sub;
-            regs[u] = tile < tiles ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + (size_t)tile * 1024 + lane_byte))
-                                   : v4i{0, 0, 0, 0};
+            const int tile = min(((grp * PF + u) * 8 + wave) * TPL + sub, tiles - 1);
+            regs[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wb + (size_t)tile * 1024 + lane_byte));
         }
+        __builtin_amdgcn_sched_barrier(0);
     };
-    v4i cur[PF], nxt[PF];
-    if (nlive > 0) load_group(0, 0, cur);
+    if (nlive == 0) { // (nothing routed to this token)
+        if (tid < CW) a.out[(size_t)t * a.H + pb * 32 + col0 + tid] = 0.0f;
+        return;
+    }
 
-    // ---- the middle rows (max != 0 ? max / 127 : 1, ties to even)
-    for (int li = wave; li < nlive; li += 8) {
+    // ---- the middle rows (max != 0 ? max / 127 : 1, ties to even): wave li quantizes live slot li.
+    // Its row and partial maxima are requested first, the first group of down tiles behind them.
+    constexpr int CACHE = (MOE_DECODE_DOWN_K / 16 + 63) / 64; // chunks per lane
+    auto fetch_row = [&](int li, float (*v)[16], uint32_t& bits) {
         const int asg = t * slots + live_slot[li];
         const float* hrow = a.hidden + (size_t)asg * I;
-        constexpr int CACHE = (MOE_DECODE_DOWN_K / 16 + 63) / 64; // chunks per lane
-        float v[CACHE][16];
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
             const int c = lane + 64 * i;
@@ -929,8 +963,10 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
                 }
             }
         }
-        uint32_t bits = 0;
+        bits = 0;
         for (int i = lane; i < parts; i += 64) bits = max(bits, a.row_max_bits[(size_t)asg * parts + i]);
+    };
+    auto quantize_row = [&](int li, float (*v)[16], uint32_t bits) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) bits = max(bits, (uint32_t)__shfl_xor((int)bits, off));
         const float mx = __uint_as_float(bits);
@@ -944,7 +980,28 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
                 *reinterpret_cast<uint4*>(a_lds + (size_t)li * Ip + (size_t)c * 16) =
                     c < nchunks ? quantize16<true>(v[i], inv) : make_uint4(0, 0, 0, 0);
         }
+    };
+    v4i cur[PF], nxt[PF];
+    {
+        float v[CACHE][16];
+        uint32_t bits = 0;
+        if (wave < nlive) fetch_row(wave, v, bits);
+        __builtin_amdgcn_sched_barrier(0);
+        load_group(0, 0, cur);
+        if (wave < nlive) quantize_row(wave, v, bits);
     }
+    for (int li = wave + 8; li < nlive; li += 8) { // (more than eight live slots: top-8 and a shared expert)
+        float v[CACHE][16];
+        uint32_t bits = 0;
+        fetch_row(li, v, bits);
+        quantize_row(li, v, bits);
+    }
+    // the slots' column scales of the epilogue, requested now instead of one after the other at the end
+    float dsc[MOE_DECODE_SLOTS];
+#pragma unroll
+    for (int li = 0; li < MOE_DECODE_SLOTS; ++li)
+        dsc[li] = a.down_scales[(size_t)live_expert[li < nlive ? li : 0] * a.H + pb * 32 + col0 + tid % CW];
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
     // ---- the down blocks
@@ -956,14 +1013,15 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
         const uint8_t* codes = a_lds + (size_t)li * Ip;
         int acc = 0;
         for (int grp = 0; grp < groups; ++grp) {
-            const bool last = grp + 1 == groups;
-            if (!last) load_group(li, grp + 1, nxt);
-            else if (li + 1 < nlive) load_group(li + 1, 0, nxt);
+            // the next group: of this slot, else the first of the next slot, else (nothing left) this one again
+            const bool last = grp + 1 == groups, more = li + 1 < nlive;
+            load_group(last && more ? li + 1 : li, last ? (more ? 0 : grp) : grp + 1, nxt);
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
                 const int tile = ((grp * PF + u) * 8 + wave) * TPL + sub;
                 if (tile < tiles) moe_dot_tile(int4, codes, tile, half, cur[u], acc);
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < PF; ++u) cur[u] = nxt[u];
         }
@@ -976,14 +1034,17 @@ __global__ __launch_bounds__(512) void moe_decode_down_kernel(RK_MOE_DECODE_HEAD
     if (tid < CW) {
         const int n = pb * 32 + col0 + tid; // (H is a multiple of 32)
         float sum = 0.0f;
-        for (int li = 0; li < nlive; ++li) {
-            int acc = 0;
 #pragma unroll
-            for (int w = 0; w < 8; ++w) acc += red[li][w][tid];
-            const int e = live_expert[li];
-            if (e < a.int4_experts) acc >>= 4;
-            const float y = dequant(acc, live_scale[li], a.down_scales[(size_t)e * a.H + n]);
-            sum = fmaf(y, live_coeff[li], sum);
+        for (int li = 0; li < MOE_DECODE_SLOTS; ++li) {
+            if (li < nlive) {
+                int acc = 0;
+#pragma unroll
+                for (int w = 0; w < 8; ++w) acc += red[li][w][tid];
+                const int e = live_expert[li];
+                if (e < a.int4_experts) acc >>= 4;
+                const float y = dequant(acc, live_scale[li], dsc[li]);
+                sum = fmaf(y, live_coeff[li], sum);
+            }
         }
         a.out[(size_t)t * a.H + n] = sum;
     }
