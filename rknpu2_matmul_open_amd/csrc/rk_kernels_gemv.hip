@@ -243,7 +243,8 @@ struct FusedRows {
 // 11.0 / 11.6), four tiles per group throughout (11.4), the exact-wait kernel with four loads
 // per wave in flight (10.7), the exact-wait kernel with its first eight loads in four stages between
 // the prologue's barriers, the first stage ahead of the row, as the int4 single-row kernel has them
-// (10.6: the same; twelve / sixteen loads in stages 11.4 / spills), 28 instead of 32 columns per workgroup (512 workgroups, two for
+// (10.6: the same, also with the epilogue's scales requested early; twelve / sixteen loads in stages
+// 11.4 / spills), 28 instead of 32 columns per workgroup (512 workgroups, two for
 // every compute unit, instead of 448 -- 11.85 us; the per-lane addresses this needs cost 0.4 us
 // already with 32 columns).
 template <int MR, bool W4, int QT, int CW, bool BURST = false, bool BIG = false>
@@ -375,6 +376,21 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!W_FIRST) prefetch_stage(0);
         RK_TS(4);
+    }
+    // The epilogue's column scale (and, for the int4 dot products, the column sum) of the output
+    // element this thread may write: requested now, unconditionally (counted by the compiler, so no
+    // wait below covers more than it has to), instead of as a round trip at the end of the kernel.
+    // 32-column workgroups only (4096 x 14336 int4, one row: 6.22 -> 6.12 us; int8, two / four rows
+    // 11.1 -> 11.0 / 11.6 -> 11.4); the 16- and 8-column kernels of narrow matrices lose 3 - 6 % with it.
+    constexpr bool EPI_EARLY = FUSEQ && !BURST && CW == 32;
+    float early_ws = 1.0f;
+    int early_colsum = 0;
+    if constexpr (EPI_EARLY) {
+        const int n_e = block_first_col(p, g.interleave_F) + col0 + (int)threadIdx.x % CW;
+        const int n_c = n_e < g.N ? n_e : 0;
+        if (g.w_scale) early_ws = g.w_scale[n_c];            // (uniform)
+        if constexpr (W4 && !MATRIX) early_colsum = g.w_colsum[n_c];
+        __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (FUSEQ) {
         if ((int)threadIdx.x < MR) row_max[threadIdx.x] = 0u;
@@ -648,11 +664,11 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) sum += red[w][m][j];
         const int n = block_first_col(p, g.interleave_F) + col0 + j;
-        if (W4 && !MATRIX && n < g.N) sum += 8 * g.w_colsum[n]; // (the constant term of the digit split)
+        if (W4 && !MATRIX && n < g.N) sum += 8 * (EPI_EARLY ? early_colsum : g.w_colsum[n]); // (the constant term of the digit split)
         if (n < g.N)
             store_out(g.C, g.epilogue, (size_t)m * g.ldc + n, sum,
                       FUSEQ ? row_scale[m] : (g.a_scale ? g.a_scale[m] : 1.0f),
-                      g.w_scale ? g.w_scale[n] : 1.0f);
+                      EPI_EARLY ? early_ws : g.w_scale ? g.w_scale[n] : 1.0f);
     }
 }
 
