@@ -1417,6 +1417,15 @@ static bool dense_streams(const rkh_gemm_args& g) {
     const int max_rows = forced ? atoi(forced) : DENSE_STREAM_MAX_M;
     if (g.blk_expert || g.M <= gemv_max_rows(g) || g.M > max_rows) return false;
     if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
+    // 65 .. 128 rows on an int8 matrix so wide that the tiles of 32 rows x 256 columns walk K without a
+    // split: three or four row blocks stream every weight byte three or four times through the compute
+    // units' memory paths, and tiles of 64 rows (two row blocks per wave, dense_rows64) or the LDS-ring
+    // kernel's 128-row tiles do better.  fp16 in / out, quantization included, us, K = 4096 at 128 rows:
+    // N = 11008 28.4 -> 24.1, 14336 28.5 -> 24.3, 28672 36 -> 26; K = 6144, N = 11008 36.4 -> 30.2; K = 2048,
+    // N = 11008 17.0 -> 15.7.  (Narrower matrices split K over the waves of 64- or 32-column tiles and
+    // stay: 4096 x 6144 19.9 against 22.8, 4096 x 8192 at 96 rows 18.1 against 21.7.)
+    if (!forced && !g.w_int4 && g.M > 64 && g.K <= 6144 &&
+        (long)((g.M + 31) / 32) * ((g.N + 255) / 256) >= DENSE_KS4_BELOW) return false;
     return !g.w_int4 || g.K <= 131072;
 }
 

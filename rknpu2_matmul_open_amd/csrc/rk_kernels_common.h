@@ -280,6 +280,11 @@ __device__ __forceinline__ uint4 quantize16(const float* v, float inv) {
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// Workgroups of the streaming kernel's 32-row x 256-column grid below which a dense launch splits K
+// over the waves of narrower tiles instead.  (256 or 512 instead, int8, 128 rows, K = 4096: 11008
+// columns 25.6 -> 23.4 us, 14336 columns 27.3 -> 30.4 us.)
+constexpr long DENSE_KS4_BELOW = 128;
+
 // ---- leading scalar arguments
 // The first 14 dwords of a kernel's scalar arguments arrive in registers when a wave starts
 // (kernel-argument preload, switched on by the build's -amdgpu-kernarg-preload-count);

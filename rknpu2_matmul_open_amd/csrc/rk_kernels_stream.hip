@@ -325,9 +325,7 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
 constexpr long GROUPED_KS4_BELOW = 96;
 constexpr long GROUPED_BALANCED_UNITS_PER_CU = 4; // (row block, column pair) units per compute unit from which the balanced launch is used
 
-// dense use of the same kernel: every row block is live.  (256 or 512 instead, int8, 128 rows, K = 4096:
-// 11008 columns 25.6 -> 23.4 us, 14336 columns 27.3 -> 30.4 us.)
-constexpr long DENSE_KS4_BELOW = 128;
+// (dense use of the same kernel, every row block live: DENSE_KS4_BELOW in rk_kernels_common.h)
 // Grouped (MoE) launches: one workgroup per (32-row block of the sorted rows,
 // 256-column tile); blocks beyond the live count exit at once.  When that grid
 // would leave compute units idle (max_blocks is the caller's bound for this

@@ -28,6 +28,9 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               (300, 8448, 200), (130, 96, 4100),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
               (100, 8448, 160), (128, 96, 3000),
+              # 65 .. 128 rows on a very wide matrix: tiles of 64 rows (the case above), the large-tile kernel where
+              # even those outnumber the compute units; up to 64 rows stay on the streaming kernel's full-K tiles
+              (70, 33000, 64), (40, 33000, 96),
               # >= 160 tiles of 128 x 256: the large-tile kernel (ragged M / N / K, K shorter than its look-ahead)
               (641, 6900, 200), (700, 6900, 1100),
               # decode GEMV: 16 columns per workgroup (65 .. 256 column blocks) / 32 columns (more)
@@ -104,7 +107,11 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               (2, 9000, 300), (4, 4100, 300),   # two rows on a wide matrix; four rows, 16 columns per workgroup
               # weight-streaming kernel on a wide grid; 64-row tiles of the large-tile kernel;
               # eight rows per quantization workgroup (M >= 4096)
-              (100, 8448, 160), (300, 8448, 200), (4200, 64, 100)]
+              (100, 8448, 160), (300, 8448, 200), (4200, 64, 100),
+              # full-K tiles of the streaming kernel (up to 64 rows, very wide); 65 .. 128 rows there: large-tile kernel
+              (40, 33000, 96), (70, 33000, 64),
+              # K split over the waves of 64-column tiles (enough of them that 32-column tiles are not needed)
+              (100, 4100, 300)]
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
