@@ -1426,6 +1426,10 @@ static bool dense_streams(const rkh_gemm_args& g) {
     // stay: 4096 x 6144 19.9 against 22.8, 4096 x 8192 at 96 rows 18.1 against 21.7.)
     if (!forced && !g.w_int4 && g.M > 64 && g.K <= 6144 &&
         (long)((g.M + 31) / 32) * ((g.N + 255) / 256) >= DENSE_KS4_BELOW) return false;
+    // (int4 weights: the two kernels measure the same there -- until the 32 x 256 tiles outnumber the compute
+    // units and run in two rounds: 4096 x 28672 at 72 / 128 rows 33.5 / 34.8 -> 23.5 / 25.5 us on the large tiles)
+    if (!forced && g.w_int4 && g.M > 64 && g.K <= 6144 &&
+        (long)((g.M + 31) / 32) * ((g.N + 255) / 256) > (compute_units() > 0 ? compute_units() : 256)) return false;
     return !g.w_int4 || g.K <= 131072;
 }
 

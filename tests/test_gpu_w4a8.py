@@ -44,7 +44,9 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200),
           # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), four-row
           # dot products beyond
-          (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200)]
+          (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200),
+          # 65 .. 128 rows whose 32 x 256 tiles outnumber the compute units: the large-tile kernel
+          (70, 22100, 64)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
