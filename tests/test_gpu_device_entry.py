@@ -369,3 +369,36 @@ def test_i8i8i32_device_random_shapes(sess, oracle):
             sess.free_device(baseA)
             sess.free_device(dC)
             op.close()
+
+
+# The decode dispatch changes kernel at these sizes: 256 / 257 column blocks (16- / 32-column workgroups),
+# rows of 4096 / 4097+ elements (eight rows fit the staging area of the wide int4 matrices or not; one
+# K chunk or two), three rows (the eight-row kernel on wide int4 matrices) and seven / eight rows (the
+# decode kernel's limit there).  Both weight formats through the device entries, fp16 rows.
+BOUNDARY_SHAPES = [(M, N, K) for M in (2, 3, 7, 8) for N in (8192, 8224) for K in (4096, 4100)] + \
+                  [(1, 8224, 4096), (4, 8193, 4095), (5, 8224, 8200), (6, 8160, 4097)]
+
+
+@pytest.mark.parametrize("M,N,K", BOUNDARY_SHAPES)
+def test_decode_dispatch_boundaries(sess, oracle, M, N, K):
+    rng = np.random.default_rng(M * 131 + N + K)
+    lib = sess.lib
+    c = workloads.w8a8_case(M, K, N, seed_w=N + K, seed_a=M + 11)
+    B4 = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    s4 = (rng.random(N).astype(np.float32) + 0.5) * np.float32(0.02)
+    A16 = c["A"]
+    op = ops.W8A8Linear(sess, capi.F16I8F16_DYNAMIC, M, c["B"], c["w_scale"])
+    w = ops.W4A8Weights(sess, B4, s4)
+    wsp = ops.W4A8Workspace(sess, M, N, K)
+    dA, dC = sess.to_device(A16), sess.empty_device(M * N * 2)
+    try:
+        assert op.run_device(dA, dC) == 0 and sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.uint16), oracle.w8a8(A16, c["B"], c["w_scale"])["C"])
+        assert lib.rk_npu_w4a8_run_f16_device(wsp.h, w.h, dA, dC) == 0 and sess.sync() == 0
+        assert np.array_equal(sess.from_device(dC, (M, N), np.uint16), oracle.w4a8(A16, B4, s4)["C"])
+    finally:
+        sess.free_device(dA)
+        sess.free_device(dC)
+        wsp.close()
+        w.close()
+        op.close()
