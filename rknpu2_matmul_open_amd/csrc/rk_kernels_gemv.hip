@@ -931,20 +931,22 @@ int launch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_a
     return RKH_OK;
 }
 
-// gate/up + SwiGLU of one or two rows as a GEMV (columns gate/up interleaved in blocks of 32,
+// gate/up + SwiGLU of up to four rows as a GEMV (columns gate/up interleaved in blocks of 32,
 // F a multiple of 32, both blocks of a workgroup within the 4 GiB reach of its descriptor).
 // Measured for 4096 -> 2 x 14336 int4 against 14.9 us on the MFMA kernel: 12.8 us for one row,
-// 13.8 for two, 15.1 for four, 20.1 for eight -- so from three rows on the MFMA kernel keeps it
-// (also when the GEMV could quantize the rows itself and save that launch: a whole 4096 -> 14336
-// -> 4096 FFN of three / four rows took 33.6 / 34.8 us that way against 34.6 / 34.5).
+// 13.8 for two, 15.1 for four, 20.1 for eight.  Three and four rows: the kernel as such is no
+// faster than the MFMA kernel, but it quantizes the rows itself and saves that launch -- a whole
+// 4096 -> 14336 -> 4096 FFN of three / four rows 31.9 / 32.0 -> 28.9 / 30.35 us (33.6 / 34.8 against
+// 34.6 / 34.5 before its first weight tiles were requested in stages).
 bool gemv_swiglu_applies(const rkh_gemm_args& g) {
-    return !g.blk_expert && g.w_int4 && g.M <= 2 && g.epilogue == RKH_EPI_SWIGLU && g.interleave_F >= 32 &&
+    return !g.blk_expert && g.w_int4 && g.M <= 4 && g.epilogue == RKH_EPI_SWIGLU && g.interleave_F >= 32 &&
            g.interleave_F % 32 == 0 && g.N == 2 * g.interleave_F && g.K <= (1 << 24);
 }
 
 int dispatch_gemv_swiglu(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fuse) {
     if (g.M == 1) return launch_gemv_swiglu<1>(st, g, fuse);
-    return launch_gemv_swiglu<2>(st, g, fuse);
+    if (g.M == 2) return launch_gemv_swiglu<2>(st, g, fuse);
+    return launch_gemv_swiglu<4>(st, g, fuse);
 }
 
 // An int4 matrix of more than 256 column blocks whose rows fit the staging area eight at a time: from

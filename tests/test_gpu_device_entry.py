@@ -144,7 +144,7 @@ def test_w4a8_device_rejects_nonfinite_rows(sess):
 # one / two rows: gate/up + SwiGLU as a GEMV that quantizes its rows itself, and a down GEMV that
 # re-quantizes the middle itself; more rows: the MFMA kernels with kernels of their own for both
 FFN_SHAPES = [(1, 64, 64, 64), (1, 1000, 4160, 300), (2, 256, 2048, 300), (2, 20003, 96, 65),
-              (3, 256, 2048, 300), (4, 1000, 4160, 300), (4, 4096, 1056, 40), (3, 9000, 96, 65),  # three / four rows: the MFMA kernel behind a quantization launch
+              (3, 256, 2048, 300), (4, 1000, 4160, 300), (4, 4096, 1056, 40), (3, 9000, 96, 65),  # three / four rows: the SwiGLU GEMV as well (rows of 9000: behind a quantization launch)
               (5, 128, 96, 65), (8, 512, 1024, 4100), (33, 256, 160, 128)]
 
 

@@ -237,6 +237,7 @@ def test_w4a8_rejections(sess):
 
 
 SWIGLU_SHAPES = [(1, 64, 64), (1, 4160, 1000), (2, 192, 20003),  # one / two rows: the SwiGLU GEMV (ragged K, K in chunks)
+                 (3, 4160, 1000), (4, 192, 20003), (4, 64, 64),     # three / four rows on the same kernel
                  (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
                  (128, 1024, 512),
                  (20, 32896, 128), (32, 2048, 700),  # weight-streaming kernel: wide grid / K split inside the workgroup
@@ -268,7 +269,7 @@ def test_swiglu_bit_exact_poly_and_close_to_libm(sess, oracle, M, N, K):
         w.close()
 
 
-FFN_SHAPES = [(1, 64, 64, 64), (2, 256, 2048, 300), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
+FFN_SHAPES = [(1, 64, 64, 64), (2, 256, 2048, 300), (3, 1000, 4160, 300), (4, 256, 2048, 65), (7, 128, 96, 65), (33, 256, 160, 128), (64, 512, 1024, 300),
               (128, 384, 2048, 256),
               # an intermediate beyond 2^17: the down projection's K is split into parts, M <= 8 and M > 8
               (2, 64, 131072 + 2112, 40), (9, 64, 131072 + 2112, 40),
