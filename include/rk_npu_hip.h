@@ -77,7 +77,7 @@ int rk_npu_w4a8_run_ffn_f32_device(rk_npu_w4a8_workspace* gate_up,
                                    rk_npu_w4a8_workspace* down,
                                    const rk_npu_w4a8_weights* down_weights, const float* A_device,
                                    float* middle_device, float* C_device);
-/* (The MoE layer: up to eight tokens per call take two launches of dot-product kernels, more tokens the
+/* (The MoE layer: up to twelve tokens per call take two launches of dot-product kernels, more tokens the
  * five launches of the routed, grouped path; same results bit for bit.) */
 int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* workspace,
                                  const rk_npu_moe_w8_weights* weights, int rows,

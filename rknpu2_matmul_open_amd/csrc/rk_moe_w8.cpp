@@ -770,7 +770,7 @@ int rk_npu_moe_w8_run_f32(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weigh
 // Device-resident variant: ids, coefficients and tokens cannot be inspected without a copy back,
 // so the kernels look at them: an id out of range, a negative or non-finite coefficient and a
 // non-finite token raise the context's flag, which the next rk_npu_hip_sync returns as ERR_PARAM.
-// Up to eight tokens take the two-launch path (see enqueue), more the routed, grouped one.
+// Up to twelve tokens take the two-launch path (see enqueue), more the routed, grouped one.
 int rk_npu_moe_w8_run_f32_device(rk_npu_moe_w8_workspace* ws, const rk_npu_moe_w8_weights* w,
                                  int rows, const float* input, const int32_t* ids,
                                  const float* routes, float* out) {

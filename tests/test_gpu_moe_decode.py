@@ -47,7 +47,8 @@ def _run_device(sess, moe, x, ids, routes):
 # the last two: output widths at which the down kernel takes 16 columns per workgroup (the others: 8 or 32)
 CASES = [(1, 64, 32, 3, 2, 1), (1, 2048, 1024, 32, 4, 0), (2, 128, 64, 6, 2, 0), (3, 96, 160, 5, 3, 1),
          (4, 2048, 1024, 32, 4, 1), (5, 416, 96, 9, 8, 0), (7, 64, 8192, 4, 2, 1), (8, 4096, 512, 16, 4, 0),
-         (8, 160, 32, 40, 8, 1), (6, 32768, 32, 2, 1, 0), (2, 2048, 64, 4, 2, 1), (3, 1408, 128, 5, 2, 0)]
+         (8, 160, 32, 40, 8, 1), (6, 32768, 32, 2, 1, 0), (2, 2048, 64, 4, 2, 1), (3, 1408, 128, 5, 2, 0),
+         (10, 2048, 1024, 32, 4, 1), (12, 256, 128, 12, 4, 0)]
 
 
 def _flavours(case):
