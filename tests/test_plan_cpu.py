@@ -63,14 +63,14 @@ def test_plan_invariants(scratch_bytes):
 
 
 def test_which_moe_calls_take_the_two_launch_path():
-    """Up to eight tokens, a hidden size that fits the staging area, a middle short enough for nine
+    """Up to twelve tokens, a hidden size that fits the staging area, a middle short enough for nine
     re-quantized rows side by side; everything else takes the routed, grouped path."""
     lib = capi.load_library()
     f = lib.rkh_moe_decode_applies
     f.restype = C.c_int
     f.argtypes = [C.c_int] * 3
-    for rows in range(1, 9):
+    for rows in range(1, 13):
         assert f(rows, 2048, 1024) and f(rows, 64, 32) and f(rows, 32768, 3584)
-    assert not f(9, 2048, 1024) and not f(256, 2048, 1024) and not f(0, 2048, 1024)
+    assert not f(13, 2048, 1024) and not f(256, 2048, 1024) and not f(0, 2048, 1024)
     assert not f(4, 32768 + 32, 1024) and not f(4, 2048, 3584 + 32) and not f(4, 2048, 8192)
     assert not f(4, 2040, 1024) and not f(4, 2048, 1000)   # (the layer's geometry is in multiples of 32)
