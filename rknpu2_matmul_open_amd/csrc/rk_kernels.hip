@@ -72,7 +72,7 @@ using rkk::gemv_can_fuse;
 using rkk::gemv_max_rows;
 using rkk::gemv_swiglu_applies;
 using rkk::launch_gemm_grouped;
-using rkk::launch_gemm_rows64;
+using rkk::launch_gemm_wk_narrow;
 using rkk::wk_scratch_bytes;
 
 // ------------------------------------------------------------------ fill
@@ -1419,8 +1419,8 @@ static bool dense_streams(const rkh_gemm_args& g) {
     if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
     // 65 .. 128 rows on an int8 matrix so wide that the tiles of 32 rows x 256 columns walk K without a
     // split: three or four row blocks stream every weight byte three or four times through the compute
-    // units' memory paths, and tiles of 64 rows (two row blocks per wave, dense_rows64) or the LDS-ring
-    // kernel's 128-row tiles do better.  fp16 in / out, quantization included, us, K = 4096 at 128 rows:
+    // units' memory paths, and the LDS-ring kernel's tiles of 64 rows x 128 columns (dense_narrow) or its
+    // 128-row tiles do better.  fp16 in / out, quantization included, us, K = 4096 at 128 rows:
     // N = 11008 28.4 -> 24.1, 14336 28.5 -> 24.3, 28672 36 -> 26; K = 6144, N = 11008 36.4 -> 30.2; K = 2048,
     // N = 11008 17.0 -> 15.7.  (Narrower matrices split K over the waves of 64- or 32-column tiles and
     // stay: 4096 x 6144 19.9 against 22.8, 4096 x 8192 at 96 rows 18.1 against 21.7.)
@@ -1433,26 +1433,29 @@ static bool dense_streams(const rkh_gemm_args& g) {
     return !g.w_int4 || g.K <= 131072;
 }
 
-// A few hundred rows on int8 weights, while tiles of 64 rows x 128 columns still give every compute
-// unit at most one: the streaming kernel with two row blocks per wave (K split over two waves, no
-// second launch) instead of the LDS-ring kernel with its K split over workgroups and the reduce
-// launch behind it.  Measured, fp16 in / out, quantization included, us: 4096 x 4096 at 192 / 256 /
-// 384 / 512 rows 25.1 / 28.4 / 28.2 / 28.4 -> 23.0 / 23.1 / 24.1 / 24.9; 4096 x 11008 at 192 rows 31.1 ->
-// 27.7.  It loses where the tiles outnumber the compute units (4096 x 4096 at 768 rows 30.8 -> 35.8:
-// operands straight to registers are 1 KiB through the compute unit's 64 B / clock memory path per
-// MFMA, twice what the matrix pipes can wait for), for a long K (11008 x 4096 at 192 rows 33.4 -> 48.3:
-// there the other kernel's K split pays) and with int4 weights (everywhere by 1 - 10 us).
-// RK_NPU_HIP_ROWS64 = 0 switches it off, 1 forces it for every dense int8 GEMM beyond the streaming
-// kernel's rows (tuning aid).
-static bool dense_rows64(const rkh_gemm_args& g) {
-    if (g.blk_expert || g.w_int4 || g.epilogue == RKH_EPI_SWIGLU) return false;
-    static const char* forced = getenv("RK_NPU_HIP_ROWS64");
+// A few hundred rows, while tiles of 64 rows x 128 columns still give every compute unit at most one: the
+// LDS-ring kernel with one column block per wave (launch_gemm_wk_narrow) instead of its 256-column tiles
+// with K split over workgroups and a reduce launch behind them.  A tile pulls K x (64 + 128) bytes through
+// its compute unit (int4 weights: K x (64 + 64)) and every compute unit has one.  fp16 in / out,
+// quantization included, weights from HBM, us: int8 4096 x 4096 at 160 / 256 / 512 rows 22.6 / 23.1 / 24.5 ->
+// 20.5 / 20.9 / 22.1, 4096 x 11008 at 192 rows 27.2 -> 26.3, at 128 rows 23.9 -> 20.6, 4096 x 14336 at 128 rows
+// 24.6 -> 22.1, 6144 x 11008 at 128 rows 30.1 -> 27.0; int4 4096 x 4096 at 160 / 256 / 512 rows 19.8 / 18.0 / 20.6 ->
+// 16.1 / 15.5 / 17.8, 2048 x 8192 at 192 rows 13.7 -> 12.0.  (The int8 shapes ran on the streaming kernel with two
+// row blocks per wave before, which pulled 1 MB per tile where this one pulls 768 KB and which lost to the
+// other plans with int4 weights; those instantiations are gone.)  It loses where the tiles outnumber
+// the compute units (int8 4096 x 4096 at 768 rows 30.8 -> 31.9, 4096 x 14336 at 512 rows 41 -> 68; int4
+// 4096 x 11008 at 160 rows, 258 tiles: 20.6 -> 23.2) and for a long K (11008 x 4096 at 192 rows 33.2 -> 42:
+// there the K split pays), which is where the rule stops.  RK_NPU_HIP_NARROW_TILES = 0 switches it off,
+// 1 forces it for every dense GEMM beyond the streaming kernel's rows that needs no K split (tuning aid).
+static bool dense_narrow(const rkh_gemm_args& g) {
+    if (g.blk_expert || g.epilogue == RKH_EPI_SWIGLU || min_ksplit(g.K, g.w_int4) > 1) return false;
+    static const char* forced = getenv("RK_NPU_HIP_NARROW_TILES");
     if (forced && forced[0]) return forced[0] == '1';
-    static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the LDS-ring kernel)
+    static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the 256-column tiles)
     if (plan && plan[0]) return false;
     const int cus = compute_units() > 0 ? compute_units() : 256;
     const long tiles = (long)((g.M + 63) / 64) * ((g.N + 127) / 128);
-    return g.K <= 6144 && tiles <= cus + cus / 50;
+    return g.K <= 6144 && tiles <= (g.w_int4 ? cus : cus + cus / 50);
 }
 
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
@@ -1470,7 +1473,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     if (gemv_swiglu_applies(g) && gemv_ok) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
-    if (dense_rows64(g)) return launch_gemm_rows64(st, g);
+    if (dense_narrow(g)) return launch_gemm_wk_narrow(st, g);
     const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {

@@ -78,7 +78,9 @@ __device__ __forceinline__ void wk_tile_coords(unsigned tile, unsigned mblocks, 
 
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm" // m0 is set and clobbered on purpose below
-template <int TM, bool W4, int EPI>
+// TN: 32-column blocks per wave.  Two -- tiles of 256 columns; one -- tiles of 128 columns, for a few
+// hundred rows whose 256-column tiles would leave compute units without one (launch_gemm_wk_narrow).
+template <int TM, bool W4, int EPI, int TN = 2>
 __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const uint8_t* h_W, int h_M, int h_K,
                                                       int mblocks, int nblocks, int ksplit, int ksteps_per_part,
                                                       rkh_gemm_args g) {
@@ -86,7 +88,9 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
     // prologue's loads depend on, ten dwords, arrives in registers)
     g.A = h_A; g.W = h_W; g.M = h_M; g.K = h_K;
     RK_TS(0);
-    constexpr int TN = 2, KTS = 8 / TM, KTW = KTS / 2; // k-tiles per sub-step: all / this wave's
+    constexpr int KTS = 8 / TM, KTW = KTS / 2; // k-tiles per sub-step: all / this wave's
+    constexpr int NMF = TM * KTW * TN;         // MFMAs of a wave per sub-step
+    static_assert(TN == 2 || (TN == 1 && EPI != RKH_EPI_SWIGLU), "gate / up pairs need two column blocks per wave");
     // Look-ahead: weights NSW - 1 sub-steps, activation copies D sub-steps.  The 128-row tile runs
     // one tile per compute unit, all of them at once, so what the prologue requests before the first
     // MFMA (D copies + NSW - 1 weight groups per wave, 152 KB per compute unit with 8 / 12) is
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
     const uint8_t* wsrc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int pb = nblk * 8 + wn * TN + j;
+        const int pb = nblk * (4 * TN) + wn * TN + j;
         wsrc[j] = W4 ? Wb + ((size_t)pb * (KB / 2) + (size_t)kstep0 * KTW) * 1024 + (PAIRED ? wk * 1024 : wk * 8)
                      : Wb + ((size_t)pb * KB + (size_t)kstep0 * KTS + wk) * 1024 + W_BIAS;
     }
@@ -244,7 +248,8 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         copy_a((SLOT + D) % NBUF);
         load_w(wring[(SLOT + NSW - 1) % NSW]);
         __builtin_amdgcn_sched_barrier(0);
-        static_for<8>([&](auto q_tag) {
+        static_assert(NMF >= 4 && NWREG <= ((NWREG + 3) / 4) * (NMF - 2), "the slots below: four fragment reads, the wait, the unpack items");
+        static_for<NMF>([&](auto q_tag) {
             constexpr int Q = decltype(q_tag)::value;
             constexpr int U = Q / (TN * TM), J = Q % (TN * TM) / TM, I = Q % TM;
             if constexpr (W4)
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
     if constexpr (EPI != RKH_EPI_I32) {
         const int t = threadIdx.x;
         const int m = mblk * BM + (t & (BM - 1));
-        const int pb = nblk * 8 + ((t & 255) >> 5);
+        const int pb = nblk * (4 * TN) + ((t & (128 * TN - 1)) >> 5);
         int n;
         if constexpr (EPI == RKH_EPI_SWIGLU) {
             // pb even = gate, odd = up block of middle columns (pb / 2) * 32
@@ -344,7 +349,7 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
         float* sc = reinterpret_cast<float*>(lds_raw + WK_SCALES_OFF);
         const int t = threadIdx.x;
         if (t < BM) sc[t] = as_valid ? my_as : 0.0f;
-        if (t < 256) sc[128 + t] = ws_valid ? my_ws : 0.0f;
+        if (t < 128 * TN) sc[128 + t] = ws_valid ? my_ws : 0.0f;
     }
     lds_barrier();
 
@@ -428,9 +433,9 @@ __global__ __launch_bounds__(512) void gemm_wk_kernel(const uint8_t* h_A, const 
 #pragma unroll
                         for (int r = 0; r < 16; ++r) acc[i0 + ii][j][r] >>= 4;
                 }
-                const int pb0 = nblk * 8 + wn * TN;
+                const int pb0 = nblk * (4 * TN) + wn * TN;
                 if constexpr (EPI == RKH_EPI_SWIGLU) {
-                    epilogue_swiglu_scaled(g, acc[i0 + ii][0], acc[i0 + ii][1], m0, pb0, lane, as[ii], ws[0], ws[1],
+                    epilogue_swiglu_scaled(g, acc[i0 + ii][0], acc[i0 + ii][TN - 1], m0, pb0, lane, as[ii], ws[0], ws[TN - 1],
                                            m_limit, stage_lds);
                 } else {
 #pragma unroll
@@ -564,9 +569,44 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
     return RKH_OK;
 }
 
+// Tiles of 64 rows x 128 columns (one column block per wave), K not split over workgroups: a few hundred
+// rows whose 256-column tiles would leave compute units without one.  The 64 activation rows of a tile go
+// through LDS once for the eight waves, so a tile pulls K x (64 + 128) bytes through its compute unit.
+int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) {
+    constexpr int TM = 2, TN = 1, KTS = 8 / TM;
+    const int mblocks = (g.M + 63) / 64, nblocks = (g.N + 127) / 128;
+    const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 32 / KTS);
+    const dim3 grid(mblocks * nblocks), block(512);
+    mark(st, "gemm_wk_kernel<64 x 128>");
+#define RK_WKN(W4, EPI)                                                                             \
+    do {                                                                                            \
+        static std::atomic<bool> opted_in[64] = {};                                                 \
+        int dev = 0;                                                                                \
+        RKH_CHECK(hipGetDevice(&dev));                                                              \
+        if (dev < 0 || dev >= 64) return RKH_ERR_RUNTIME;                                           \
+        if (!opted_in[dev].load(std::memory_order_acquire)) {                                       \
+            RKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wk_kernel<TM, W4, EPI, TN>), \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, WK_LDS_BYTES)); \
+            opted_in[dev].store(true, std::memory_order_release);                                   \
+        }                                                                                           \
+        hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI, TN>), grid, block, WK_LDS_BYTES, st,       \
+                           g.A, g.W, g.M, g.K, mblocks, nblocks, 1, ksteps_total, g);               \
+    } while (0)
+    switch (g.epilogue) {
+    case RKH_EPI_I32: if (g.w_int4) RK_WKN(true, RKH_EPI_I32); else RK_WKN(false, RKH_EPI_I32); break;
+    case RKH_EPI_F16: if (g.w_int4) RK_WKN(true, RKH_EPI_F16); else RK_WKN(false, RKH_EPI_F16); break;
+    case RKH_EPI_F32: if (g.w_int4) RK_WKN(true, RKH_EPI_F32); else RK_WKN(false, RKH_EPI_F32); break;
+    default: return RKH_ERR_RUNTIME;
+    }
+#undef RK_WKN
+    RKH_CHECK(hipGetLastError());
+    return RKH_OK;
+}
+
 } // namespace
 
 namespace rkk {
+int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_wk_narrow(st, g); }
 size_t wk_scratch_bytes(long tiles, int bm, int ksplit) { return ::wk_scratch_bytes(tiles, bm, ksplit); }
 int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int tile_rows, int ksplit) {
     if (tile_rows == 128) return ::launch_gemm_wk<4>(st, g, ksplit);

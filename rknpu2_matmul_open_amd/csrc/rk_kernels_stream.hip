@@ -36,10 +36,12 @@ __global__ __launch_bounds__(BAL ? 512 : 256) void gemm_stream_kernel(RK_GEMM_HE
                                                                       rkh_gemm_args g) {
     RK_GEMM_HEAD_APPLY(g);
     constexpr int WAVES = BAL ? 8 : 4;
-    // TM: 32-row blocks per wave.  One; two for dense GEMMs of a few hundred rows (`mblocks` then
-    // counts units of TM row blocks): a weight tile in registers is multiplied with both blocks'
-    // activation tiles, so a workgroup pulls K x (64 rows + its columns) bytes through its compute
-    // unit for twice the products -- tiles of 64 x 128, K split over two waves.
+    // TM: 32-row blocks per wave (`mblocks` counts units of TM row blocks).  One in every launch of this
+    // library.  Two -- a weight tile in registers multiplied with both blocks' activation tiles, tiles
+    // of 64 x 128 with K split over two waves -- served dense int8 GEMMs of a few hundred rows until
+    // the LDS-ring kernel got tiles of that shape: four waves that each fetch their own operands pull
+    // 1 MB per tile through the compute unit, the ring's eight waves 768 KB, and 4096 x 4096 at 512 rows
+    // took 24.5 us here against 22.1 there.
     static_assert(TM == 1 || (TM == 2 && !BAL && TN == 2 && EPI != RKH_EPI_SWIGLU), "two row blocks per wave: dense launches");
     // TN: 32-column blocks per wave.  Two; one for small launches whose K is split over the waves
     // (32-column tiles: twice the workgroups where 64-column tiles leave most compute units idle).
@@ -412,29 +414,10 @@ int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) {
     return RKH_OK;
 }
 
-// Dense int8 GEMMs of a few hundred rows: two row blocks per wave, tiles of 64 rows x 128 columns, K split
-// over two waves.  (Tiles of 64 x 256 without the K split and int4 weights were measured as well and
-// lose to the LDS-ring kernel on every shape, so they are not compiled.)
-int launch_gemm_rows64(hipStream_t st, const rkh_gemm_args& g) {
-    if (g.blk_expert || g.w_int4 || g.epilogue == RKH_EPI_SWIGLU) return RKH_ERR_RUNTIME;
-    const int mblocks = (g.M + 63) / 64, nblocks = (g.N + 127) / 128;
-    const dim3 grid(mblocks * nblocks), block(256);
-    mark(st, "gemm_stream_kernel<64 x 128>");
-    switch (g.epilogue) {
-    case RKH_EPI_I32: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_I32, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
-    case RKH_EPI_F16: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_F16, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
-    case RKH_EPI_F32: hipLaunchKernelGGL((gemm_stream_kernel<RKH_EPI_F32, 2, false, false, 2, 2>), grid, block, 0, st, RK_GEMM_HEAD(g), mblocks, nblocks, g); break;
-    default: return RKH_ERR_RUNTIME;
-    }
-    RKH_CHECK(hipGetLastError());
-    return RKH_OK;
-}
-
 } // namespace
 
 namespace rkk {
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_grouped(st, g); }
-int launch_gemm_rows64(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_rows64(st, g); }
 #ifdef RK_DEBUG_TS
 void set_ts_stream(unsigned long long* p) { (void)hipMemcpyToSymbol(HIP_SYMBOL(rk_dbg_ts), &p, sizeof(p)); }
 #endif
