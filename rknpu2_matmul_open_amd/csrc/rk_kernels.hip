@@ -1446,16 +1446,28 @@ static bool dense_streams(const rkh_gemm_args& g) {
 // the compute units (int8 4096 x 4096 at 768 rows 30.8 -> 31.9, 4096 x 14336 at 512 rows 41 -> 68; int4
 // 4096 x 11008 at 160 rows, 258 tiles: 20.6 -> 23.2) and for a long K (11008 x 4096 at 192 rows 33.2 -> 42:
 // there the K split pays), which is where the rule stops.  RK_NPU_HIP_NARROW_TILES = 0 switches it off,
-// 1 forces it for every dense GEMM beyond the streaming kernel's rows that needs no K split (tuning aid).
-static bool dense_narrow(const rkh_gemm_args& g) {
-    if (g.blk_expert || g.epilogue == RKH_EPI_SWIGLU || min_ksplit(g.K, g.w_int4) > 1) return false;
+// 1 forces it (2: the 128-row tiles below) for every dense GEMM beyond the streaming kernel's rows that
+// needs no K split (tuning aid).
+static int dense_narrow(const rkh_gemm_args& g) { // rows of the tile, or 0: another plan
+    if (g.blk_expert || g.epilogue == RKH_EPI_SWIGLU || min_ksplit(g.K, g.w_int4) > 1) return 0;
     static const char* forced = getenv("RK_NPU_HIP_NARROW_TILES");
-    if (forced && forced[0]) return forced[0] == '1';
+    if (forced && forced[0]) return forced[0] == '1' ? 64 : forced[0] == '2' ? (g.w_int4 ? 64 : 128) : 0;
     static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the 256-column tiles)
-    if (plan && plan[0]) return false;
+    if (plan && plan[0]) return 0;
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    const long tiles = (long)((g.M + 63) / 64) * ((g.N + 127) / 128);
-    return g.K <= 6144 && tiles <= (g.w_int4 ? cus : cus + cus / 50);
+    const long nblocks = (g.N + 127) / 128;
+    if (g.K <= 6144 && (long)((g.M + 63) / 64) * nblocks <= (g.w_int4 ? cus : cus + cus / 50)) return 64;
+    // Beyond that, int8 weights: tiles of 128 rows x 128 columns of the same kernel while THEY give every
+    // compute unit at most one and at least five in eight of them have one.  A tile pulls K x (128 + 128)
+    // bytes for twice the products, and no K split means no reduce launch; a long K is no obstacle here.
+    // us as above, against the 256-column tiles' plan: 4096 x 4096 at 640 / 768 / 1024 rows 31.7 / 30.8 / 32.6 ->
+    // 27.8 / 27.8 / 28.8, 11008 x 4096 65.3 / 68.6 / 78.0 -> 62.5 / 65.4 / 70.6.  With more tiles than compute
+    // units it loses (4096 x 4096 at 1536 rows 39.5 -> 44.8, 4096 x 11008 at 640 rows 44.3 -> 49.5), and so it
+    // does with int4 weights at every size measured (4096 x 4096 at 640 rows 23.5 -> 25.5, 4096 x 8192
+    // 34.8 -> 42.3), whose tiles pull half the weight bytes to begin with.
+    const long tiles128 = (long)((g.M + 127) / 128) * nblocks;
+    if (!g.w_int4 && tiles128 >= cus * 5L / 8 && tiles128 <= cus + cus / 50) return 128;
+    return 0;
 }
 
 size_t rkh_gemm_scratch_bytes(int M, int N, int K, int w_int4) {
@@ -1473,7 +1485,7 @@ int rkh_gemm(void* stream, const rkh_gemm_args* args) {
     if (gemv_swiglu_applies(g) && gemv_ok) return dispatch_gemv_swiglu(st, g, nullptr);
     if (grouped) return launch_gemm_grouped(st, g);
     if (dense_streams(g)) return launch_gemm_grouped(st, g);
-    if (dense_narrow(g)) return launch_gemm_wk_narrow(st, g);
+    if (const int tile_rows = dense_narrow(g)) return launch_gemm_wk_narrow(st, g, tile_rows);
     const DensePlan plan = effective_plan(g.M, g.N, g.K, g.w_int4);
     int ksplit = plan.ksplit;
     if (ksplit > 1 && !g.splitk_acc) {

@@ -41,7 +41,7 @@ size_t wk_scratch_bytes(long tiles, int bm, int ksplit);
 int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int tile_rows, int ksplit);
 // rk_kernels_stream.hip
 int launch_gemm_grouped(hipStream_t st, const rkh_gemm_args& g);
-int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g);
+int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g, int tile_rows);
 #ifdef RK_DEBUG_TS
 void set_ts_gemv(unsigned long long* p);
 void set_ts_gemm(unsigned long long* p);

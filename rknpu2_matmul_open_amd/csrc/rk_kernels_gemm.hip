@@ -569,15 +569,16 @@ int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int ksplit) {
     return RKH_OK;
 }
 
-// Tiles of 64 rows x 128 columns (one column block per wave), K not split over workgroups: a few hundred
-// rows whose 256-column tiles would leave compute units without one.  The 64 activation rows of a tile go
-// through LDS once for the eight waves, so a tile pulls K x (64 + 128) bytes through its compute unit.
+// Tiles of 64 or 128 rows x 128 columns (one column block per wave), K not split over workgroups: a few
+// hundred rows whose 256-column tiles would leave compute units without one.  The activation rows of a tile
+// go through LDS once for the eight waves, so a tile pulls K x (rows + 128) bytes through its compute unit.
+template <int TM>
 int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) {
-    constexpr int TM = 2, TN = 1, KTS = 8 / TM;
-    const int mblocks = (g.M + 63) / 64, nblocks = (g.N + 127) / 128;
+    constexpr int TN = 1, KTS = 8 / TM;
+    const int mblocks = (g.M + 32 * TM - 1) / (32 * TM), nblocks = (g.N + 127) / 128;
     const int ksteps_total = (int)(rkh_align_up(g.K, RKH_K_ALIGN) / 32 / KTS);
     const dim3 grid(mblocks * nblocks), block(512);
-    mark(st, "gemm_wk_kernel<64 x 128>");
+    mark(st, TM == 2 ? "gemm_wk_kernel<64 x 128>" : "gemm_wk_kernel<128 x 128>");
 #define RK_WKN(W4, EPI)                                                                             \
     do {                                                                                            \
         static std::atomic<bool> opted_in[64] = {};                                                 \
@@ -592,12 +593,20 @@ int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) {
         hipLaunchKernelGGL((gemm_wk_kernel<TM, W4, EPI, TN>), grid, block, WK_LDS_BYTES, st,       \
                            g.A, g.W, g.M, g.K, mblocks, nblocks, 1, ksteps_total, g);               \
     } while (0)
+    // (int4 weights: the 64-row tiles only -- the 128-row ones measured slower than the other plans everywhere)
+#define RK_WKN_W(EPI)                                                                               \
+    do {                                                                                            \
+        if (!g.w_int4) RK_WKN(false, EPI);                                                          \
+        else if constexpr (TM == 2) RK_WKN(true, EPI);                                              \
+        else return RKH_ERR_RUNTIME;                                                                \
+    } while (0)
     switch (g.epilogue) {
-    case RKH_EPI_I32: if (g.w_int4) RK_WKN(true, RKH_EPI_I32); else RK_WKN(false, RKH_EPI_I32); break;
-    case RKH_EPI_F16: if (g.w_int4) RK_WKN(true, RKH_EPI_F16); else RK_WKN(false, RKH_EPI_F16); break;
-    case RKH_EPI_F32: if (g.w_int4) RK_WKN(true, RKH_EPI_F32); else RK_WKN(false, RKH_EPI_F32); break;
+    case RKH_EPI_I32: RK_WKN_W(RKH_EPI_I32); break;
+    case RKH_EPI_F16: RK_WKN_W(RKH_EPI_F16); break;
+    case RKH_EPI_F32: RK_WKN_W(RKH_EPI_F32); break;
     default: return RKH_ERR_RUNTIME;
     }
+#undef RK_WKN_W
 #undef RK_WKN
     RKH_CHECK(hipGetLastError());
     return RKH_OK;
@@ -606,7 +615,9 @@ int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) {
 } // namespace
 
 namespace rkk {
-int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g) { return ::launch_gemm_wk_narrow(st, g); }
+int launch_gemm_wk_narrow(hipStream_t st, const rkh_gemm_args& g, int tile_rows) {
+    return tile_rows == 128 ? ::launch_gemm_wk_narrow<4>(st, g) : ::launch_gemm_wk_narrow<2>(st, g);
+}
 size_t wk_scratch_bytes(long tiles, int bm, int ksplit) { return ::wk_scratch_bytes(tiles, bm, ksplit); }
 int launch_gemm_wk(hipStream_t st, const rkh_gemm_args& g, int tile_rows, int ksplit) {
     if (tile_rows == 128) return ::launch_gemm_wk<4>(st, g, ksplit);

@@ -25,7 +25,9 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               # a very wide matrix for one row, for a row block and for many rows
               (1, 1, 1), (5000, 3, 1), (2, 1, 5000), (4100, 40, 70), (1, 70001, 64), (9, 70001, 40), (300, 40000, 33),
               # 64-row tiles of the large-tile kernel (too few 128-row tiles); K split over workgroups + reduce launch
-              (300, 8448, 200), (130, 96, 4100),
+              (330, 6600, 200), (130, 96, 4100),
+              # tiles of 128 x 128 with one column block per wave (160 .. 261 of them, more 64-row tiles than that)
+              (300, 8448, 200), (257, 8200, 300), (640, 4200, 96),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
               (100, 8448, 160), (128, 96, 3000),
               # 65 .. 128 rows on a very wide matrix: tiles of 64 rows (the case above), the large-tile kernel where
@@ -105,9 +107,9 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               # with several rows, with K staged in several chunks; wide matrices with one / several rows
               (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300),
               (2, 9000, 300), (4, 4100, 300),   # two rows on a wide matrix; four rows, 16 columns per workgroup
-              # weight-streaming kernel on a wide grid; 64-row tiles of the large-tile kernel;
-              # eight rows per quantization workgroup (M >= 4096)
-              (100, 8448, 160), (300, 8448, 200), (4200, 64, 100),
+              # weight-streaming kernel on a wide grid; 128 x 128 tiles with one column block per wave; 64-row
+              # tiles of the large-tile kernel; eight rows per quantization workgroup (M >= 4096)
+              (100, 8448, 160), (300, 8448, 200), (330, 6600, 200), (4200, 64, 100),
               # full-K tiles of the streaming kernel (up to 64 rows, very wide); 65 .. 128 rows there: large-tile kernel
               (40, 33000, 96), (70, 33000, 64),
               # K split over the waves of 64-column tiles (enough of them that 32-column tiles are not needed)
@@ -135,9 +137,11 @@ def test_f16i8f16_dynamic_bit_exact(sess, oracle, M, N, K):
         op.close()
 
 
-# second: many-row quantization path; then 128- and 64-row tiles of the large-tile kernel, K split over
-# workgroups + reduce launch, eight rows per quantization workgroup
-@pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203), (650, 7000, 300), (300, 8448, 200), (261, 96, 3000),
+# second: many-row quantization path; then 128-row tiles of the large-tile kernel, 128 x 128 tiles with one
+# column block per wave, 64-row tiles of the large-tile kernel, K split over workgroups + reduce launch,
+# eight rows per quantization workgroup
+@pytest.mark.parametrize("M,N,K", [(37, 200, 300), (261, 96, 203), (650, 7000, 300), (300, 8448, 200), (330, 6600, 200),
+                                   (261, 96, 3000),
                                    (4200, 64, 100),
                                    # an input / an output of more than 64 MiB: beyond the pinned staging mirrors
                                    (4200, 64, 4100), (4200, 4100, 64)])
