@@ -979,15 +979,13 @@ int dispatch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* 
 // Whether the streaming MFMA kernel can take this dense GEMM at all (int4 codes ride as 16 * code).
 bool dense_stream_fits(const rkh_gemm_args& g) { return !g.w_int4 || g.K <= 131072; }
 
-// Most rows the decode kernels take for this matrix: eight, but four on an int4 matrix of more than
-// 256 column blocks, where five to eight rows are faster as one 32-row block of the streaming MFMA
-// kernel behind a quantization launch (fp16 rows, every step from HBM, dot products against stream,
-// us: 4096 x 11008 int4 15.5 - 18.9 against 12.3 - 12.5; 4096 x 14336 16.1 - 19.3 against 12.8 - 12.9).
-// On int8 matrices that was so too while the rows were multiplied by dot products (4096 x 14336
-// 18.8 - 21.9 against 16.2 - 16.5); with the products on the matrix cores the decode kernel keeps them:
-// five to eight rows 16.3 -> 12.6 - 14.7 us (4096 x 14336), 15.3 -> 12.2 - 14.1 (4096 x 11008).
-// A wide int4 matrix whose rows fit the staging area eight at a time keeps up to seven rows as well, on
-// the eight-row kernel (see gemv_mr).
+// Most rows the decode kernels take for this matrix; the rows beyond go to the streaming MFMA kernel as
+// one 32-row block behind a quantization launch.  Eight on int8 weights: with the products of five to
+// eight rows on the matrix cores the decode kernel is ahead (4096 x 14336 12.6 - 14.7 us against 16.3,
+// 4096 x 11008 12.2 - 14.1 against 15.3).  On int4 weights: seven on a wide matrix (more than 256 column
+// blocks) whose rows fit the staging area eight at a time (the eight-row kernel, see gemv_mr); eight on
+// a narrower one with such rows; otherwise four or two, see below.  (The four-row dot products on a wide
+// matrix took 15.5 - 19.3 us for five to eight rows of 4096 x 11008 / 14336 against 12.3 - 12.9 streamed.)
 // RK_NPU_HIP_GEMV_MAX_ROWS = 1..8 lowers the limit (tuning aid).
 int gemv_max_rows(const rkh_gemm_args& g) {
     static const int rows = [] {
@@ -997,7 +995,25 @@ int gemv_max_rows(const rkh_gemm_args& g) {
     }();
     const bool wide = (g.N + 31) / 32 > 256;
     if (w4_wide_eight(g)) return min(rows, GEMV_W4_WIDE_ROWS);
-    return wide && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g) ? min(rows, 4) : rows;
+    if (g.w_int4 && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g)) {
+        // int4 rows that do not fit the staging area at once (the kernel then walks K in chunks and cannot
+        // quantize the rows itself): the streaming kernel behind a quantization launch is faster from three
+        // rows on -- K > 8192, four-row instantiation -- or from five -- K > 4096, eight-row instantiation
+        // (fp16 rows, weights from HBM, us: 14336 x 4096 three / four rows 16.1 -> 15.0, five to eight 18.0 -> 15.1 - 15.6;
+        // 11008 x 4096 13.8 -> 13.0 and 15.0 -> 13.0; 8192 x 8192 five to eight 15.4 -> 12.1; 6144 x 8192 13.3 -> 10.6;
+        // 5120 x 5120 11.8 -> 9.65; 20000 x 2048 21.9 -> 20.1 and 26.2 -> 20.2; 11008 x 11008 three / four rows
+        // 22.4 -> 17.1, 14336 x 14336 30.0 -> 23.4).  A wide matrix whose K is beyond the eight-row instantiation's
+        // reach (K > 4096) does the same from three rows on, although four rows would fit: 5120 x 11008 three /
+        // four rows 12.3 / 13.1 -> 11.7 / 11.8, 8192 x 14336 16.7 / 18.4 -> 16.2, 8192 x 28672 30.3 / 33.0 -> 23.9,
+        // 6144 x 14336 13.9 / 15.4 -> 14.1.  Two rows stay on the dot products everywhere (8192 x 14336 12.2
+        // against 16.2), and so do three and four on a narrower matrix that fits (6144 x 4096 6.1 / 6.6 against
+        // 10.1, 8192 x 8192 10.5 / 11.8 against 11.9).  On int8 weights the decode kernel stays ahead
+        // (14336 x 4096 five to eight rows 23.1 against 25.9 us, 11008 x 4096 19.6 against 21.2).
+        const size_t kp = rkh_align_up(g.K, RKH_K_ALIGN);
+        if (kp * 4 > (size_t)GEMV_LDS_BYTES || wide) return min(rows, 2);
+        if (kp * 8 > (size_t)GEMV_LDS_BYTES) return min(rows, 4);
+    }
+    return rows;
 }
 
 bool gemv_can_fuse(const rkh_quant_args& q, const rkh_gemm_args& g, bool swiglu = false) {

@@ -79,8 +79,13 @@ W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 900
              # two rows at every column width of the kernel; four rows, 8 columns; six rows, 16 columns
              (2, 4096, 512), (2, 9000, 300), (2, 1000, 200), (4, 1000, 300), (6, 4100, 300),
              # three to seven rows on a wide matrix whose rows fit the staging area eight at a time: the
-             # eight-row kernel with matrix-core products (ragged K, a full 4096); K beyond that: four-row dot products
-             (3, 8200, 1000), (5, 9000, 4096), (7, 8224, 300), (6, 14336, 4096), (4, 8200, 4100)]
+             # eight-row kernel with matrix-core products (ragged K, a full 4096); K beyond that: the streaming
+             # kernel from three rows on, two rows on the dot products
+             (3, 8200, 1000), (5, 9000, 4096), (7, 8224, 300), (6, 14336, 4096), (4, 8200, 4100), (3, 8300, 4100),
+             (2, 8300, 4100),
+             # a narrower matrix: rows that fit the staging area four / eight at a time stay on the decode
+             # kernel, longer ones go to the streaming kernel
+             (4, 2000, 8192), (3, 4100, 8300), (4, 2000, 4100), (5, 2000, 4100), (8, 2000, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", W4_SHAPES)
