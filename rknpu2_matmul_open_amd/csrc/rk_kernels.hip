@@ -1415,8 +1415,28 @@ constexpr int DENSE_STREAM_MAX_M = 128, DENSE_STREAM_SWIGLU_MAX_M = 32;
 static bool dense_streams(const rkh_gemm_args& g) {
     static const char* forced = getenv("RK_NPU_HIP_STREAM_MAX_ROWS"); // (tuning aid)
     const int max_rows = forced ? atoi(forced) : DENSE_STREAM_MAX_M;
-    if (g.blk_expert || g.M <= gemv_max_rows(g) || g.M > max_rows) return false;
+    if (g.blk_expert) return false;
+    if (g.M > max_rows) {
+        // 129 .. 256 rows on a narrow matrix, while the grid is small enough that K is split over the
+        // waves (64-column tiles): up to eight row blocks x N / 64 workgroups of this kernel against a few
+        // dozen tiles of the LDS-ring kernel.  fp16 in / out, quantization included, us, 136 / 256 rows:
+        // int8 2048 x 2048 12.9 / 13.4 -> 10.0 / 10.5, 4096 x 2048 18.1 / 18.9 -> 13.1 / 14.1, 8192 x 2048
+        // 27.4 / 29.2 -> 20.5 / 23.1, 4096 x 1024 20.2 / 19.1 -> 11.9 / 12.0, 4096 x 4096 at 136 / 224 rows
+        // 20.2 / 20.5 -> 18.5 / 19.3, 6144 x 4096 26.8 / 27.3 -> 24.3 / 26.1; int4 2048 x 2048 10.7 -> 9.5,
+        // 4096 x 2048 15.8 / 16.1 -> 12.3 / 13.1, 8192 x 2048 21.9 / 26.1 -> 17.4 / 18.8, 14336 x 2048
+        // 29.8 / 32.3 -> 25.3 / 26.1.  Where it stops: a longer K (int8 11008 x 4096 32.5 -> 37.8, 14336 x 2048
+        // 30.0 -> 31.3, 8192 x 4096 a tie), int4 weights from 4096 columns on (a tie), 256-column tiles
+        // (4096 x 4096 at 256 rows 20.9 -> 27.1), more rows (4096 x 2048 at 384 rows a tie).
+        static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the large-tile kernel)
+        if (forced || (plan && plan[0]) || g.epilogue == RKH_EPI_SWIGLU || g.M > 2 * DENSE_STREAM_MAX_M) return false;
+        if ((long)((g.M + 31) / 32) * ((g.N + 255) / 256) >= DENSE_KS4_BELOW) return false;
+        if (g.N <= 2048) return g.K <= (g.w_int4 ? 16384 : 8192);
+        return !g.w_int4 && g.N <= 4096 && g.K <= 6144;
+    }
+    // (the SwiGLU decode kernel has taken its calls by now -- up to four rows -- whatever the row limit of
+    // the plain decode kernels is: five to eight rows of a gate/up GEMM stream too)
     if (g.epilogue == RKH_EPI_SWIGLU) return g.w_int4 && g.K <= 131072 && g.M <= DENSE_STREAM_SWIGLU_MAX_M;
+    if (g.M <= gemv_max_rows(g)) return false;
     // 65 .. 128 rows on an int8 matrix so wide that the tiles of 32 rows x 256 columns walk K without a
     // split: three or four row blocks stream every weight byte three or four times through the compute
     // units' memory paths, and the LDS-ring kernel's tiles of 64 rows x 128 columns (dense_narrow) or its

@@ -42,8 +42,10 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           # 64-row tiles of the large-tile kernel; K split over workgroups + reduce launch; two / three rows
           # on a wide matrix
           (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200),
-          # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), four-row
-          # dot products beyond
+          # 129 .. 256 rows on a narrow matrix: the streaming kernel (K split over its waves); beyond its K limit: 64-row tiles
+          (200, 2000, 300), (256, 1000, 8300), (150, 96, 17000),
+          # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), the
+          # streaming kernel beyond
           (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200),
           # 65 .. 128 rows whose 32 x 256 tiles outnumber the compute units: the large-tile kernel
           (70, 22100, 64)]
@@ -241,6 +243,7 @@ SWIGLU_SHAPES = [(1, 64, 64), (1, 4160, 1000), (2, 192, 20003),  # one / two row
                  (5, 128, 96), (16, 192, 257), (33, 256, 512), (70, 640, 384),
                  (128, 1024, 512),
                  (20, 32896, 128), (32, 2048, 700),  # weight-streaming kernel: wide grid / K split inside the workgroup
+                 (8, 32896, 128), (6, 2048, 700),    # the same with five to eight rows (beyond the SwiGLU GEMV's four)
                  (650, 6912, 520), (641, 7040, 300),  # large-tile kernel (F a multiple of 64 / only of 32)
                  (40, 128, 4100)]  # two 32-row tiles: K split over workgroups, SwiGLU in the reduce launch
 

@@ -25,11 +25,12 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               # a very wide matrix for one row, for a row block and for many rows
               (1, 1, 1), (5000, 3, 1), (2, 1, 5000), (4100, 40, 70), (1, 70001, 64), (9, 70001, 40), (300, 40000, 33),
               # 64-row tiles of the large-tile kernel (too few 128-row tiles); K split over workgroups + reduce launch
-              (330, 6600, 200), (130, 96, 4100),
+              (330, 6600, 200), (150, 96, 8300),
               # tiles of 128 x 128 with one column block per wave (160 .. 261 of them, more 64-row tiles than that)
               (300, 8448, 200), (257, 8200, 300), (640, 4200, 96),
-              # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split
-              (100, 8448, 160), (128, 96, 3000),
+              # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split; 129 .. 256 rows on a
+              # narrow matrix with it (a longer K there: the 64-row tiles above)
+              (100, 8448, 160), (128, 96, 3000), (200, 2048, 96), (250, 4000, 200), (130, 96, 4100),
               # 65 .. 128 rows on a very wide matrix: tiles of 64 rows (the case above), the large-tile kernel where
               # even those outnumber the compute units; up to 64 rows stay on the streaming kernel's full-K tiles
               (70, 33000, 64), (40, 33000, 96),
@@ -113,7 +114,9 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               # full-K tiles of the streaming kernel (up to 64 rows, very wide); 65 .. 128 rows there: large-tile kernel
               (40, 33000, 96), (70, 33000, 64),
               # K split over the waves of 64-column tiles (enough of them that 32-column tiles are not needed)
-              (100, 4100, 300)]
+              (100, 4100, 300),
+              # 129 .. 256 rows on a narrow matrix: the streaming kernel
+              (250, 1500, 300), (136, 4000, 200), (224, 520, 4100)]
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
