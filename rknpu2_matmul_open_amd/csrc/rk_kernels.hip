@@ -1428,7 +1428,8 @@ static bool dense_streams(const rkh_gemm_args& g) {
         // 30.0 -> 31.3, 8192 x 4096 a tie), int4 weights from 4096 columns on (a tie), 256-column tiles
         // (4096 x 4096 at 256 rows 20.9 -> 27.1), more rows (4096 x 2048 at 384 rows a tie).
         static const char* plan = getenv("RK_NPU_HIP_GEMM_PLAN"); // (a forced plan is a plan of the large-tile kernel)
-        if (forced || (plan && plan[0]) || g.epilogue == RKH_EPI_SWIGLU || g.M > 2 * DENSE_STREAM_MAX_M) return false;
+        // (a matrix of up to 1024 columns: up to 512 rows -- 4096 x 1024 at 384 rows 19.9 -> 14.6, int4 14.1 -> 12.7)
+        if (forced || (plan && plan[0]) || g.epilogue == RKH_EPI_SWIGLU || g.M > (g.N <= 1024 ? 4 : 2) * DENSE_STREAM_MAX_M) return false;
         if ((long)((g.M + 31) / 32) * ((g.N + 255) / 256) >= DENSE_KS4_BELOW) return false;
         if (g.N <= 2048) return g.K <= (g.w_int4 ? 16384 : 8192);
         return !g.w_int4 && g.N <= 4096 && g.K <= 6144;
