@@ -416,8 +416,10 @@ void gemv_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) {
         const int chunks = kc >> 4;
         if (kc0) __syncthreads();
         if constexpr (QT == 0) {
+            // (rows fastest: the MR rows of a chunk are MR adjacent 16-byte slots of a tile, so a wave's loads
+            // cover whole lines; chunk by chunk along a row, every lane fetched a line of its own for 16 bytes)
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
-                const int m = idx / chunks, c = idx - m * chunks;
+                const int c = idx / MR, m = idx - c * MR;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = (W4 && !MATRIX) ? digits16(v) : v;
             }
@@ -763,8 +765,10 @@ void gemv_swiglu_kernel(RK_GEMV_HEAD_PARAMS, rkh_gemm_args g, rkh_quant_args q) 
         const int chunks = kc >> 4;
         if (kc0) __syncthreads();
         if constexpr (QT == 0) {
+            // (rows fastest: the MR rows of a chunk are MR adjacent 16-byte slots of a tile, so a wave's loads
+            // cover whole lines; chunk by chunk along a row, every lane fetched a line of its own for 16 bytes)
             for (int idx = threadIdx.x; idx < MR * chunks; idx += GEMV_WAVES * 64) {
-                const int m = idx / chunks, c = idx - m * chunks;
+                const int c = idx / MR, m = idx - c * MR;
                 const uint4 v = *reinterpret_cast<const uint4*>(g.A + tiled_chunk_offset(m, (kc0 >> 4) + c, KB));
                 *reinterpret_cast<uint4*>(a_lds + (size_t)m * kc + (size_t)c * 16) = W4 ? digits16(v) : v;
             }
@@ -996,21 +1000,26 @@ int gemv_max_rows(const rkh_gemm_args& g) {
     const bool wide = (g.N + 31) / 32 > 256;
     if (w4_wide_eight(g)) return min(rows, GEMV_W4_WIDE_ROWS);
     if (g.w_int4 && g.epilogue != RKH_EPI_SWIGLU && dense_stream_fits(g)) {
-        // int4 rows that do not fit the staging area at once (the kernel then walks K in chunks and cannot
-        // quantize the rows itself): the streaming kernel behind a quantization launch is faster from three
-        // rows on -- K > 8192, four-row instantiation -- or from five -- K > 4096, eight-row instantiation
-        // (fp16 rows, weights from HBM, us: 14336 x 4096 three / four rows 16.1 -> 15.0, five to eight 18.0 -> 15.1 - 15.6;
-        // 11008 x 4096 13.8 -> 13.0 and 15.0 -> 13.0; 8192 x 8192 five to eight 15.4 -> 12.1; 6144 x 8192 13.3 -> 10.6;
-        // 5120 x 5120 11.8 -> 9.65; 20000 x 2048 21.9 -> 20.1 and 26.2 -> 20.2; 11008 x 11008 three / four rows
-        // 22.4 -> 17.1, 14336 x 14336 30.0 -> 23.4).  A wide matrix whose K is beyond the eight-row instantiation's
-        // reach (K > 4096) does the same from three rows on, although four rows would fit: 5120 x 11008 three /
-        // four rows 12.3 / 13.1 -> 11.7 / 11.8, 8192 x 14336 16.7 / 18.4 -> 16.2, 8192 x 28672 30.3 / 33.0 -> 23.9,
-        // 6144 x 14336 13.9 / 15.4 -> 14.1.  Two rows stay on the dot products everywhere (8192 x 14336 12.2
-        // against 16.2), and so do three and four on a narrower matrix that fits (6144 x 4096 6.1 / 6.6 against
-        // 10.1, 8192 x 8192 10.5 / 11.8 against 11.9).  On int8 weights the decode kernel stays ahead
-        // (14336 x 4096 five to eight rows 23.1 against 25.9 us, 11008 x 4096 19.6 against 21.2).
+        // int4 rows that do not fit the staging area at once (the kernel then walks K in chunks behind a
+        // quantization launch): the streaming kernel behind the same launch is faster from five rows on --
+        // K > 4096, eight-row instantiation (fp16 rows, weights from HBM, us: 14336 x 4096 18.1 -> 15.5,
+        // 11008 x 4096 15.2 -> 13.0, 8192 x 8192 15.7 -> 12.05, 6144 x 8192 13.5 -> 10.6, 5120 x 5120 12.5 -> 9.7,
+        // 20000 x 2048 28.0 -> 20.1, 28672 x 8192 42.4 -> 30.1) -- and from three rows on for K > 16384
+        // (20000 x 2048 22.2 -> 20.2, 28672 x 8192 33.5 -> 29.8; between 8192 and 16384 the four-row kernel
+        // with its chunks keeps up: 14336 x 4096 14.7 against 15.4, 11008 x 4096 12.95 both).  A wide matrix
+        // whose K is beyond the eight-row instantiation's reach (K > 4096) does the same from three rows on,
+        // although four rows would fit: 5120 x 11008 three / four rows 12.3 / 13.1 -> 11.7 / 11.8, 8192 x 14336
+        // 16.8 / 18.6 -> 16.3, 8192 x 28672 30.3 / 33.0 -> 23.9, 11008 x 11008 23.4 -> 17.2.  Two rows stay on
+        // the dot products (8192 x 14336 12.5 against 16.3) unless K > 16384 on a matrix of more than 4096
+        // columns (20000 x 8192 28.3 -> 23.1, 28672 x 8192 37.3 -> 29.8, 17000 x 14336 34.9 -> 30.4; a tie at
+        // 4096 columns, and at 2048 the streaming kernel has too few workgroups: 20000 x 2048 18.1 against
+        // 20.0), and three and four rows on a narrower matrix that fits (6144 x 4096 6.1 / 6.6 against 10.1,
+        // 8192 x 8192 10.3 / 12.0 against 12.0).  On int8 weights the decode kernel stays ahead or within
+        // 6 % (14336 x 4096 five to eight rows 21.4 against 25.9 us, 13824 x 5120 27.8 against 26.2, 28672 x 8192
+        // 55.4 against 54.5; int8 rows as given 19.6 against 23.0).
         const size_t kp = rkh_align_up(g.K, RKH_K_ALIGN);
-        if (kp * 4 > (size_t)GEMV_LDS_BYTES || wide) return min(rows, 2);
+        if (kp * 2 > (size_t)GEMV_LDS_BYTES && g.N > 4096) return 1;
+        if (kp * 4 > 2 * (size_t)GEMV_LDS_BYTES || wide) return min(rows, 2);
         if (kp * 8 > (size_t)GEMV_LDS_BYTES) return min(rows, 4);
     }
     return rows;

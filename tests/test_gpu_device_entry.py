@@ -83,9 +83,12 @@ W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 900
              # kernel from three rows on, two rows on the dot products
              (3, 8200, 1000), (5, 9000, 4096), (7, 8224, 300), (6, 14336, 4096), (4, 8200, 4100), (3, 8300, 4100),
              (2, 8300, 4100),
-             # a narrower matrix: rows that fit the staging area four / eight at a time stay on the decode
-             # kernel, longer ones go to the streaming kernel
-             (4, 2000, 8192), (3, 4100, 8300), (4, 2000, 4100), (5, 2000, 4100), (8, 2000, 4096)]
+             # a narrower matrix: eight rows that fit the staging area stay on the decode kernel, five to eight
+             # longer ones go to the streaming kernel; three and four rows stay up to K = 16384 (in chunks
+             # beyond 8192)
+             (4, 2000, 8192), (3, 4100, 8300), (4, 2000, 4100), (5, 2000, 4100), (8, 2000, 4096), (3, 2000, 16500),
+             # two rows that do not fit it (K > 16384): the streaming kernel beyond 4096 columns
+             (2, 4200, 16500), (2, 2000, 16500)]
 
 
 @pytest.mark.parametrize("M,N,K", W4_SHAPES)
