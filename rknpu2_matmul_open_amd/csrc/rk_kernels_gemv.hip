@@ -870,7 +870,19 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const int cus = compute_units() > 0 ? compute_units() : 256;
     const bool halves = fuse && fuse->in_dtype == RKH_I8 &&
                         ((2 * pblocks + cus - 1) / cus) * 16 < ((pblocks + cus - 1) / cus) * 32;
-    const int cw = want == 8 || want == 16 || want == 32 ? want : pblocks <= 64 ? 8 : pblocks <= 256 || halves ? 16 : 32;
+    // Five to eight rows, from 160 blocks on: whole blocks as well.  Every workgroup stages (and, fused,
+    // quantizes) all the rows, so with eight of them the prologues of 16-column workgroups move as many
+    // bytes as the weights: fp16 rows, us, five / eight rows, int8 5120 x 5120 11.0 / 14.3 -> 10.2 / 11.8,
+    // 6144 x 8192 13.6 / 17.45 -> 13.0 / 14.9, 8192 x 8192 16.5 / 21.55 -> 16.6 / 19.5, 4096 x 8192 8.9 / 10.95 ->
+    // 8.8 / 10.2, 13824 x 5120 (rows in chunks behind a quantization launch) 27.8 -> 23.1; int4 4096 x 8192
+    // 8.4 / 10.7 -> 6.8 / 8.3, 4096 x 5120 8.1 / 10.6 -> 6.6 / 8.0, 2048 x 8192 6.2 / 7.2 -> 5.5 / 6.0.  (128 blocks:
+    // half the compute units would idle, int8 8192 x 4096 eight rows 14.6 -> 16.2; four rows: 5120 x 5120
+    // 10.0 -> 8.8 but 8192 x 8192 14.6 -> 15.2, left alone.)
+    const bool several_wide = MR == 8 && pblocks >= 160 && !(fuse && fuse->in_dtype == RKH_I8);
+    const int cw = want == 8 || want == 16 || want == 32 ? want
+                   : pblocks <= 64                       ? 8
+                   : (pblocks <= 256 && !several_wide) || halves ? 16
+                                                         : 32;
     const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);
     const rkh_quant_args q = fuse ? *fuse : rkh_quant_args{};
     const int qt = !fuse ? 0 : fuse->in_dtype == RKH_F16 ? 1 : fuse->in_dtype == RKH_F32 ? 2 : 3;
@@ -967,6 +979,13 @@ static bool w4_wide_eight(const rkh_gemm_args& g) {
 // Rows of the kernel instantiation that takes the M rows of g.
 int gemv_mr(const rkh_gemm_args& g) {
     if (g.M >= 3 && w4_wide_eight(g)) return 8;
+    // The same from 160 column blocks on, where the eight-row kernel takes whole blocks per workgroup (see
+    // launch_gemv), and there from two rows on: 4096 x 8192 two / three / four rows 7.1 / 7.55 / 8.3 ->
+    // 5.6 / 5.95 / 6.45 us, 4096 x 5120 6.7 / 7.3 / 7.9 -> 5.4 / 5.8 / 6.3, 2048 x 8192 5.75 / 6.3 / 6.4 -> 4.7 / 5.25 / 5.4.
+    // (Two rows on a matrix of more than 256 blocks: 4096 x 14336 7.7 -> 8.0, left on the dot products.)
+    if (g.M >= 2 && (g.N + 31) / 32 >= 160 && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU &&
+        rkh_align_up(g.K, RKH_K_ALIGN) * 8 <= (size_t)GEMV_LDS_BYTES)
+        return 8;
     return g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;
 }
 
