@@ -43,7 +43,7 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           # on a wide matrix
           (300, 8448, 200), (200, 96, 5000), (2, 9000, 300), (3, 9000, 200),
           # 129 .. 256 rows on a narrow matrix: the streaming kernel (K split over its waves); beyond its K limit: 64-row tiles
-          (200, 2000, 300), (256, 1000, 8300), (150, 96, 17000), (300, 1024, 200),
+          (200, 2000, 300), (256, 1000, 8300), (150, 96, 17000), (300, 1024, 200), (200, 1, 70), (512, 2, 16384),
           # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), the
           # streaming kernel beyond
           (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200),

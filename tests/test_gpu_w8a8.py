@@ -32,6 +32,7 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               # narrow matrix with it (a longer K there: the 64-row tiles above)
               (100, 8448, 160), (128, 96, 3000), (200, 2048, 96), (250, 4000, 200), (130, 96, 4100),
               (400, 1000, 96),  # up to 512 rows on a matrix of up to 1024 columns
+              (300, 1, 40), (500, 2, 8000), (129, 33, 1),  # the same, degenerate: one / two columns, a single k
               # 65 .. 128 rows on a very wide matrix: tiles of 64 rows (the case above), the large-tile kernel where
               # even those outnumber the compute units; up to 64 rows stay on the streaming kernel's full-K tiles
               (70, 33000, 64), (40, 33000, 96),
@@ -117,7 +118,7 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               # K split over the waves of 64-column tiles (enough of them that 32-column tiles are not needed)
               (100, 4100, 300),
               # 129 .. 256 rows on a narrow matrix: the streaming kernel
-              (250, 1500, 300), (136, 4000, 200), (224, 520, 4100), (500, 520, 300)]
+              (250, 1500, 300), (136, 4000, 200), (224, 520, 4100), (500, 520, 300), (260, 3, 3)]
 
 
 @pytest.mark.parametrize("M,N,K", F16_SHAPES)
