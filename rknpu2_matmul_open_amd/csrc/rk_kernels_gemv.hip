@@ -878,7 +878,15 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     // 8.4 / 10.7 -> 6.8 / 8.3, 4096 x 5120 8.1 / 10.6 -> 6.6 / 8.0, 2048 x 8192 6.2 / 7.2 -> 5.5 / 6.0.  (128 blocks:
     // half the compute units would idle, int8 8192 x 4096 eight rows 14.6 -> 16.2; four rows: 5120 x 5120
     // 10.0 -> 8.8 but 8192 x 8192 14.6 -> 15.2, left alone.)
-    const bool several_wide = MR == 8 && pblocks >= 160 && !(fuse && fuse->in_dtype == RKH_I8);
+    // While K <= 5120 the same holds for two to four rows on int8 weights (4096 x 8192 two / three / four rows
+    // 8.05 / 8.3 / 8.6 -> 7.6 / 7.8 / 8.3, 4096 x 5120 7.1 / 7.5 / 8.2 -> 6.7 / 7.0 / 7.5, 5120 x 5120 8.5 / 9.2 / 9.85 ->
+    // 7.8 / 8.35 / 8.75; K = 8192: 12.3 -> 13.4) and for one row on int4 weights, whose 32-column instantiation
+    // requests its first weights in stages and its scales early (4096 x 8192 5.4 -> 4.65, 4096 x 5120 5.1 -> 4.2,
+    // 4096 x 7168 5.5 -> 4.4, 5120 x 5120 6.15 -> 5.9; 8192 x 8192 7.3 -> 8.1).  One int8 row keeps 16 columns
+    // (4096 x 8192 7.4 -> 8.5).
+    const bool short_k = rkh_align_up(g.K, RKH_K_ALIGN) <= 5120;
+    const bool several_wide = pblocks >= 160 && !(fuse && fuse->in_dtype == RKH_I8) &&
+                              (MR == 8 || (short_k && (g.w_int4 ? MR == 1 : MR >= 2)));
     const int cw = want == 8 || want == 16 || want == 32 ? want
                    : pblocks <= 64                       ? 8
                    : (pblocks <= 256 && !several_wide) || halves ? 16

@@ -390,7 +390,9 @@ def test_i8i8i32_device_random_shapes(sess, oracle):
 # decode kernel's limit there).  Both weight formats through the device entries, fp16 rows.
 BOUNDARY_SHAPES = [(M, N, K) for M in (2, 3, 7, 8) for N in (8192, 8224) for K in (4096, 4100)] + \
                   [(1, 8224, 4096), (4, 8193, 4095), (5, 8224, 8200), (6, 8160, 4097)] + \
-                  [(M, N, 4096) for M in (2, 5) for N in (5088, 5120)]  # 159 / 160 column blocks: 16- / 32-column workgroups for several rows
+                  [(M, N, 4096) for M in (2, 5) for N in (5088, 5120)] + \
+                  [(M, 5120, K) for M in (1, 2, 4) for K in (5120, 5400)]
+# (159 / 160 column blocks: 16- / 32-column workgroups for several rows; K up to 5120 / beyond: for a few rows too)
 
 
 @pytest.mark.parametrize("M,N,K", BOUNDARY_SHAPES)
