@@ -870,23 +870,24 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const int cus = compute_units() > 0 ? compute_units() : 256;
     const bool halves = fuse && fuse->in_dtype == RKH_I8 &&
                         ((2 * pblocks + cus - 1) / cus) * 16 < ((pblocks + cus - 1) / cus) * 32;
-    // Five to eight rows, from 160 blocks on: whole blocks as well.  Every workgroup stages (and, fused,
-    // quantizes) all the rows, so with eight of them the prologues of 16-column workgroups move as many
-    // bytes as the weights: fp16 rows, us, five / eight rows, int8 5120 x 5120 11.0 / 14.3 -> 10.2 / 11.8,
-    // 6144 x 8192 13.6 / 17.45 -> 13.0 / 14.9, 8192 x 8192 16.5 / 21.55 -> 16.6 / 19.5, 4096 x 8192 8.9 / 10.95 ->
-    // 8.8 / 10.2, 13824 x 5120 (rows in chunks behind a quantization launch) 27.8 -> 23.1; int4 4096 x 8192
-    // 8.4 / 10.7 -> 6.8 / 8.3, 4096 x 5120 8.1 / 10.6 -> 6.6 / 8.0, 2048 x 8192 6.2 / 7.2 -> 5.5 / 6.0.  (128 blocks:
-    // half the compute units would idle, int8 8192 x 4096 eight rows 14.6 -> 16.2; four rows: 5120 x 5120
-    // 10.0 -> 8.8 but 8192 x 8192 14.6 -> 15.2, left alone.)
+    // Beyond 128 blocks the 16-column workgroups outnumber the compute units, and several rows take whole
+    // blocks as well.  Every workgroup stages (and, fused, quantizes) all the rows, so with eight of them the
+    // prologues of 16-column workgroups move as many bytes as the weights: fp16 rows, us, five / eight rows,
+    // int8 5120 x 5120 11.0 / 14.3 -> 10.2 / 11.8, 6144 x 8192 13.6 / 17.45 -> 13.0 / 14.9, 8192 x 8192 16.5 / 21.55 ->
+    // 16.6 / 19.5, 4096 x 8192 8.9 / 10.95 -> 8.8 / 10.2, 4096 x 4160 8.3 / 10.45 -> 7.8 / 9.2, 13824 x 5120 (rows
+    // in chunks behind a quantization launch) 27.8 -> 23.1; int4 4096 x 8192 8.4 / 10.7 -> 6.8 / 8.3, 4096 x 4160
+    // 7.8 / 10.3 -> 6.4 / 7.8, 2048 x 8192 6.2 / 7.2 -> 5.5 / 6.0.  (128 blocks: half the compute units would
+    // idle, int8 8192 x 4096 eight rows 14.6 -> 16.2.)
     // While K <= 5120 the same holds for two to four rows on int8 weights (4096 x 8192 two / three / four rows
-    // 8.05 / 8.3 / 8.6 -> 7.6 / 7.8 / 8.3, 4096 x 5120 7.1 / 7.5 / 8.2 -> 6.7 / 7.0 / 7.5, 5120 x 5120 8.5 / 9.2 / 9.85 ->
-    // 7.8 / 8.35 / 8.75; K = 8192: 12.3 -> 13.4) and for one row on int4 weights, whose 32-column instantiation
-    // requests its first weights in stages and its scales early (4096 x 8192 5.4 -> 4.65, 4096 x 5120 5.1 -> 4.2,
-    // 4096 x 7168 5.5 -> 4.4, 5120 x 5120 6.15 -> 5.9; 8192 x 8192 7.3 -> 8.1).  One int8 row keeps 16 columns
-    // (4096 x 8192 7.4 -> 8.5).
+    // 8.05 / 8.3 / 8.6 -> 7.6 / 7.8 / 8.3, 4096 x 5120 7.1 / 7.5 / 8.2 -> 6.7 / 7.0 / 7.5, 4096 x 4160 6.85 / 8.1 (two /
+    // four) -> 6.5 / 7.3, 5120 x 5120 8.5 / 9.2 / 9.85 -> 7.8 / 8.35 / 8.75; K = 8192: 12.3 -> 13.4) and for one and
+    // two rows on int4 weights, whose 32-column instantiations request their first weights in stages and
+    // their scales early (one row 4096 x 8192 5.4 -> 4.65, 4096 x 5120 5.1 -> 4.2, 4096 x 4160 4.7 -> 4.1,
+    // 5120 x 5120 6.15 -> 5.9, two rows 4096 x 4608 6.6 -> 5.1, 4096 x 8192 7.1 -> 5.4; K = 8192: one row
+    // 7.3 -> 8.1).  One int8 row keeps 16 columns (4096 x 8192 7.4 -> 8.5, 4096 x 4160 6.0 -> 7.0).
     const bool short_k = rkh_align_up(g.K, RKH_K_ALIGN) <= 5120;
-    const bool several_wide = pblocks >= 160 && !(fuse && fuse->in_dtype == RKH_I8) &&
-                              (MR == 8 || (short_k && (g.w_int4 ? MR == 1 : MR >= 2)));
+    const bool several_wide = pblocks > 128 && !(fuse && fuse->in_dtype == RKH_I8) &&
+                              (MR == 8 || (short_k && (g.w_int4 ? MR <= 2 : MR >= 2)));
     const int cw = want == 8 || want == 16 || want == 32 ? want
                    : pblocks <= 64                       ? 8
                    : (pblocks <= 256 && !several_wide) || halves ? 16
@@ -987,11 +988,13 @@ static bool w4_wide_eight(const rkh_gemm_args& g) {
 // Rows of the kernel instantiation that takes the M rows of g.
 int gemv_mr(const rkh_gemm_args& g) {
     if (g.M >= 3 && w4_wide_eight(g)) return 8;
-    // The same from 160 column blocks on, where the eight-row kernel takes whole blocks per workgroup (see
-    // launch_gemv), and there from two rows on: 4096 x 8192 two / three / four rows 7.1 / 7.55 / 8.3 ->
-    // 5.6 / 5.95 / 6.45 us, 4096 x 5120 6.7 / 7.3 / 7.9 -> 5.4 / 5.8 / 6.3, 2048 x 8192 5.75 / 6.3 / 6.4 -> 4.7 / 5.25 / 5.4.
-    // (Two rows on a matrix of more than 256 blocks: 4096 x 14336 7.7 -> 8.0, left on the dot products.)
-    if (g.M >= 2 && (g.N + 31) / 32 >= 160 && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU &&
+    // The same beyond 128 column blocks, where the eight-row kernel takes whole blocks per workgroup (see
+    // launch_gemv): 4096 x 8192 three / four rows 7.55 / 8.3 -> 5.95 / 6.45 us, 4096 x 5120 7.3 / 7.9 -> 5.8 / 6.3,
+    // 4096 x 4608 four rows 7.8 -> 6.3, 2048 x 8192 6.3 / 6.4 -> 5.25 / 5.4.  (Two rows: the two-row dot products
+    // on whole blocks are ahead of it there, 4096 x 4608 5.1 against 5.35, 4096 x 8192 5.4 against 5.6 -- and
+    // behind it on a matrix of more than 256 blocks it would be: 4096 x 14336 7.7 against 8.0 for the eight-row
+    // kernel, so two rows stay on the dot products everywhere.)
+    if (g.M >= 3 && (g.N + 31) / 32 > 128 && g.w_int4 && g.epilogue != RKH_EPI_SWIGLU &&
         rkh_align_up(g.K, RKH_K_ALIGN) * 8 <= (size_t)GEMV_LDS_BYTES)
         return 8;
     return g.M == 1 ? 1 : g.M == 2 ? 2 : g.M <= 4 ? 4 : 8;

@@ -39,9 +39,11 @@ W8_SHAPES = [(1, 64, 64), (1, 200, 200), (1, 513, 1000), (1, 4096, 4096), (1, 21
              (2, 3000, 700), (3, 65, 33), (4, 9000, 300), (4, 4100, 8000), (8, 128, 4096), (8, 8300, 2000),
              (7, 5000, 4100), (2, 2500, 20003), (16, 300, 500),
              (2, 1000, 300), (7, 4100, 300),   # two rows, 8 columns per workgroup; five to eight rows, 16 columns
-             # five to eight rows from 160 column blocks on: whole blocks per workgroup (159 blocks: halves); rows in
-             # chunks behind a quantization launch there
-             (5, 5120, 300), (8, 5100, 4100), (6, 5088, 1000), (8, 5120, 8300)]
+             # five to eight rows beyond 128 column blocks: whole blocks per workgroup; rows in chunks behind a
+             # quantization launch there
+             (5, 5120, 300), (8, 5100, 4100), (6, 5088, 1000), (8, 5120, 8300),
+             # up to 128 blocks: 16 columns per workgroup for any number of rows (small / large staging area)
+             (6, 3000, 300), (8, 4000, 5000), (4, 4000, 300)]
 
 
 @pytest.mark.parametrize("M,N,K", W8_SHAPES)
@@ -90,8 +92,10 @@ W4_SHAPES = [(1, 64, 64), (1, 65, 33), (1, 4096, 4096), (1, 2100, 8200), (1, 900
              # longer ones go to the streaming kernel; three and four rows stay up to K = 16384 (in chunks
              # beyond 8192)
              (4, 2000, 8192), (3, 4100, 8300), (4, 2000, 4100), (5, 2000, 4100), (8, 2000, 4096), (3, 2000, 16500),
-             # 160 .. 256 column blocks: the eight-row kernel with whole blocks per workgroup from two rows on
+             # 129 .. 256 column blocks: whole blocks per workgroup, the eight-row kernel from three rows on
              (2, 5120, 4096), (3, 8192, 1000), (4, 6000, 300), (8, 5130, 4096), (2, 5100, 4100),
+             # up to 128 blocks: 16 columns per workgroup for any number of rows
+             (6, 4000, 1000), (8, 3000, 300), (2, 4000, 300),
              # two rows that do not fit it (K > 16384): the streaming kernel beyond 4096 columns
              (2, 4200, 16500), (2, 2000, 16500)]
 
@@ -390,9 +394,9 @@ def test_i8i8i32_device_random_shapes(sess, oracle):
 # decode kernel's limit there).  Both weight formats through the device entries, fp16 rows.
 BOUNDARY_SHAPES = [(M, N, K) for M in (2, 3, 7, 8) for N in (8192, 8224) for K in (4096, 4100)] + \
                   [(1, 8224, 4096), (4, 8193, 4095), (5, 8224, 8200), (6, 8160, 4097)] + \
-                  [(M, N, 4096) for M in (2, 5) for N in (5088, 5120)] + \
+                  [(M, N, 4096) for M in (1, 2, 3, 5) for N in (4096, 4128)] + \
                   [(M, 5120, K) for M in (1, 2, 4) for K in (5120, 5400)]
-# (159 / 160 column blocks: 16- / 32-column workgroups for several rows; K up to 5120 / beyond: for a few rows too)
+# (128 / 129 column blocks: 16- / 32-column workgroups for several rows; K up to 5120 / beyond: for a few rows too)
 
 
 @pytest.mark.parametrize("M,N,K", BOUNDARY_SHAPES)

@@ -47,6 +47,8 @@ SHAPES = [(1, 64, 64), (1, 65, 33), (3, 65, 33), (2, 65, 20003), (8, 128, 512), 
           # four to seven rows on a wide matrix: the eight-row decode kernel (rows fit its staging area), the
           # streaming kernel beyond
           (6, 8224, 1000), (7, 9000, 4096), (4, 9000, 4200),
+          # up to 128 column blocks: 16 columns per workgroup, two / eight rows behind a quantization launch
+          (2, 4000, 300), (8, 3000, 300),
           # 65 .. 128 rows whose 32 x 256 tiles outnumber the compute units: the large-tile kernel
           (70, 22100, 64)]
 

@@ -109,7 +109,8 @@ F16_SHAPES = [(1, 64, 64), (1, 513, 1000), (4, 96, 200), (8, 128, 4096), (16, 64
               # decode GEMV variants: 16 columns per workgroup with the rolling load window (one row),
               # with several rows, with K staged in several chunks; wide matrices with one / several rows
               (1, 4096, 4096), (2, 3000, 700), (8, 4100, 9000), (1, 9000, 520), (4, 9000, 300),
-              (2, 9000, 300), (4, 4100, 300),   # two rows on a wide matrix; four rows, 16 columns per workgroup
+              (2, 9000, 300), (4, 4000, 300),   # two rows on a wide matrix; four rows, 16 columns per workgroup
+              (4, 4100, 300), (8, 4000, 5000),  # 129 blocks: whole blocks for four rows; eight rows of 5000 on 16 columns
               # weight-streaming kernel on a wide grid; 128 x 128 tiles with one column block per wave; 64-row
               # tiles of the large-tile kernel; eight rows per quantization workgroup (M >= 4096)
               (100, 8448, 160), (300, 8448, 200), (330, 6600, 200), (4200, 64, 100),
