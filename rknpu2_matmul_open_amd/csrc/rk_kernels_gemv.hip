@@ -888,8 +888,16 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     const bool short_k = rkh_align_up(g.K, RKH_K_ALIGN) <= 5120;
     const bool several_wide = pblocks > 128 && !(fuse && fuse->in_dtype == RKH_I8) &&
                               (MR == 8 || (short_k && (g.w_int4 ? MR <= 2 : MR >= 2)));
+    // Up to 64 blocks the same trade is between 8 and 16 columns: five to eight rows take 16 (fp16 rows, us,
+    // five / eight rows, both weight formats alike: 4096 x 2048 7.0 / 8.5 -> 5.7 / 7.2, 4096 x 1024 6.9 / 8.3 ->
+    // 5.65 / 7.2, int8 8192 x 2048 11.1 / 14.2 -> 10.5 / 13.4, 14336 x 2048 20.0 -> 18.0), four rows on int4 weights
+    // (4096 x 2048 5.85 -> 5.5, 8192 x 2048 8.5 -> 7.5, 14336 x 2048 15.9 -> 13.3) and, while K <= 5120, four and
+    // two rows on int8 weights (4096 x 2048 5.95 / 5.05 -> 5.55 / 4.7; K = 8192: 8.4 / 6.4 -> 9.0 / 7.1).  One row
+    // keeps 8 (4096 x 2048 int8 3.9 -> 4.6), and so do two int4 rows (4.65 -> 4.85).
+    const bool several_narrow = !(fuse && fuse->in_dtype == RKH_I8) &&
+                                (MR == 8 || (MR == 4 && (g.w_int4 || short_k)) || (MR == 2 && !g.w_int4 && short_k));
     const int cw = want == 8 || want == 16 || want == 32 ? want
-                   : pblocks <= 64                       ? 8
+                   : pblocks <= 64 && !several_narrow    ? 8
                    : (pblocks <= 256 && !several_wide) || halves ? 16
                                                          : 32;
     const dim3 grid(pblocks * (32 / cw)), block(GEMV_WAVES * 64);

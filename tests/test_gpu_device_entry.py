@@ -395,8 +395,10 @@ def test_i8i8i32_device_random_shapes(sess, oracle):
 BOUNDARY_SHAPES = [(M, N, K) for M in (2, 3, 7, 8) for N in (8192, 8224) for K in (4096, 4100)] + \
                   [(1, 8224, 4096), (4, 8193, 4095), (5, 8224, 8200), (6, 8160, 4097)] + \
                   [(M, N, 4096) for M in (1, 2, 3, 5) for N in (4096, 4128)] + \
-                  [(M, 5120, K) for M in (1, 2, 4) for K in (5120, 5400)]
-# (128 / 129 column blocks: 16- / 32-column workgroups for several rows; K up to 5120 / beyond: for a few rows too)
+                  [(M, 5120, K) for M in (1, 2, 4) for K in (5120, 5400)] + \
+                  [(M, 2048, K) for M in (2, 4, 6) for K in (5120, 5400)] + [(2, 2080, 4096), (5, 520, 300)]
+# (128 / 129 column blocks: 16- / 32-column workgroups for several rows; K up to 5120 / beyond: for a few rows too;
+# 64 / 65 blocks: 8 / 16 columns for one row, 16 for several)
 
 
 @pytest.mark.parametrize("M,N,K", BOUNDARY_SHAPES)
