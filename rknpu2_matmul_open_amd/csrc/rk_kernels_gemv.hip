@@ -886,16 +886,22 @@ int launch_gemv(hipStream_t st, const rkh_gemm_args& g, const rkh_quant_args* fu
     // 5120 x 5120 6.15 -> 5.9, two rows 4096 x 4608 6.6 -> 5.1, 4096 x 8192 7.1 -> 5.4; K = 8192: one row
     // 7.3 -> 8.1).  One int8 row keeps 16 columns (4096 x 8192 7.4 -> 8.5, 4096 x 4160 6.0 -> 7.0).
     const bool short_k = rkh_align_up(g.K, RKH_K_ALIGN) <= 5120;
-    const bool several_wide = pblocks > 128 && !(fuse && fuse->in_dtype == RKH_I8) &&
-                              (MR == 8 || (short_k && (g.w_int4 ? MR <= 2 : MR >= 2)));
+    // int8 rows as given (no quantization, but every workgroup still stages all the rows): the same from two
+    // rows on while K <= 5120 -- 4096 x 8192 two / four / eight rows 8.3 / 8.4 / 9.3 -> 7.5 / 7.9 / 8.3, 4096 x 5120
+    // 7.05 / 7.4 / 8.35 -> 6.2 / 6.4 / 6.95; 8192 x 8192 12.75 / 13.1 / 14.6 -> 13.4 / 13.8 / 14.8 -- and up to 64 blocks
+    // from four rows on, from two while K <= 5120: 4096 x 2048 two / four / eight rows 4.8 / 5.35 / 6.35 ->
+    // 4.45 / 4.7 / 5.6, 8192 x 2048 four / eight rows 7.1 / 9.1 -> 6.7 / 7.7.
+    const bool raw_rows = fuse && fuse->in_dtype == RKH_I8;
+    const bool several_wide = pblocks > 128 && (raw_rows ? MR >= 2 && short_k
+                                                         : MR == 8 || (short_k && (g.w_int4 ? MR <= 2 : MR >= 2)));
     // Up to 64 blocks the same trade is between 8 and 16 columns: five to eight rows take 16 (fp16 rows, us,
     // five / eight rows, both weight formats alike: 4096 x 2048 7.0 / 8.5 -> 5.7 / 7.2, 4096 x 1024 6.9 / 8.3 ->
     // 5.65 / 7.2, int8 8192 x 2048 11.1 / 14.2 -> 10.5 / 13.4, 14336 x 2048 20.0 -> 18.0), four rows on int4 weights
     // (4096 x 2048 5.85 -> 5.5, 8192 x 2048 8.5 -> 7.5, 14336 x 2048 15.9 -> 13.3) and, while K <= 5120, four and
     // two rows on int8 weights (4096 x 2048 5.95 / 5.05 -> 5.55 / 4.7; K = 8192: 8.4 / 6.4 -> 9.0 / 7.1).  One row
     // keeps 8 (4096 x 2048 int8 3.9 -> 4.6), and so do two int4 rows (4.65 -> 4.85).
-    const bool several_narrow = !(fuse && fuse->in_dtype == RKH_I8) &&
-                                (MR == 8 || (MR == 4 && (g.w_int4 || short_k)) || (MR == 2 && !g.w_int4 && short_k));
+    const bool several_narrow = raw_rows ? MR >= 4 || (MR == 2 && short_k)
+                                         : MR == 8 || (MR == 4 && (g.w_int4 || short_k)) || (MR == 2 && !g.w_int4 && short_k);
     const int cw = want == 8 || want == 16 || want == 32 ? want
                    : pblocks <= 64 && !several_narrow    ? 8
                    : (pblocks <= 256 && !several_wide) || halves ? 16

@@ -246,6 +246,9 @@ I8_SHAPES = [(1, 64, 64), (1, 200, 203), (1, 513, 1000), (1, 4096, 4096), (1, 21
              (4, 9000, 301), (4, 4100, 9001), (8, 128, 4096), (8, 8300, 2000), (7, 5000, 4100), (2, 2500, 20003),
              (1, 14336, 4096), (4, 14336, 600), (8, 14336, 300), (2, 100, 300),  # whole blocks (one row: the burst variant); two rows, 8 columns
              (16, 300, 500), (130, 520, 777),
+             # several rows: 32 columns per workgroup on 129 .. 256 blocks while K <= 5120 (16 beyond), 16 on up to 64 blocks
+             (2, 5120, 4096), (8, 4200, 5120), (4, 5000, 5400), (3, 8192, 300), (4, 2048, 8200), (2, 1000, 4100), (2, 2048, 5400),
+             (8, 520, 300), (5, 4096, 4096),
              # 9..128 rows on the streaming kernel behind the re-tiling launch (K split over the waves / not; a K
              # of one and of three k-tiles; ragged last row block)
              (16, 300, 512), (33, 4100, 4096), (128, 11008, 4096), (100, 64, 32), (9, 8448, 96), (64, 520, 2080),
