@@ -1486,17 +1486,15 @@ static int dense_narrow(const rkh_gemm_args& g) { // rows of the tile, or 0: ano
     // 70.6, 4096 x 8192 at 260 / 384 / 512 rows 31.9 / 33.2 / 34.7 -> 26.6 / 27.2 / 30.9, 8192 x 8192 at 260 / 480 rows
     // 51.8 / 61.3 -> 46.3 / 49.8, 4096 x 11008 at 136 / 256 rows 29.4 / 32.7 -> 25.4 / 28.0, 11008 x 11008 at 136 / 256
     // rows 59.3 / 62.3 -> 41.9 / 46.2.  A last row block that is mostly padding costs little (4096 x 4096 at
-    // 520 rows above) -- unless the tiles outnumber the compute units: 258 tiles (three row blocks of an
-    // 11008-wide matrix) run two of them in a second round and win only with a full last block (4096 x 11008
-    // at 288 / 320 / 384 rows 34.0 / 34.6 / 39.5 -> 34.4 / 34.7 / 35.8, 6144 x 11008 46.5 / 46.3 / 53.7 -> 48.9 / 50.2 /
-    // 50.6, 11008 x 11008 68.9 / 69.7 / 85.5 -> 78.6 / 81.8 / 84.1), so the 2 % allowance of the 64-row tiles
-    // applies here only when the last block is at least three quarters full.  With more tiles it loses
-    // (4096 x 4096 at 1536 rows 39.5 -> 44.8, 4096 x 11008 at 640 rows 44.3 -> 49.5), and so it does with int4
-    // weights at every size measured (4096 x 4096 at 640 rows 23.5 -> 25.5, 4096 x 8192 34.8 -> 42.3), whose
-    // tiles pull half the weight bytes to begin with.
+    // 520 rows above).  No allowance beyond the compute units here: 258 tiles (three row blocks of an
+    // 11008-wide matrix) run two of them in a second round and lose with a partly filled last block
+    // (6144 x 11008 at 288 / 320 rows 46.5 / 46.3 -> 48.9 / 50.2, 11008 x 11008 68.9 / 69.7 -> 78.6 / 81.8); with a full
+    // one, 384 rows, they won on one box (4096 x 11008 39.5 -> 35.8) and lost on another (39.2 -> 41.3).  With
+    // more tiles it loses (4096 x 4096 at 1536 rows 39.5 -> 44.8, 4096 x 11008 at 640 rows 44.3 -> 49.5), and so
+    // it does with int4 weights at every size measured (4096 x 4096 at 640 rows 23.5 -> 25.5, 4096 x 8192
+    // 34.8 -> 42.3), whose tiles pull half the weight bytes to begin with.
     const long tiles128 = (long)((g.M + 127) / 128) * nblocks;
-    const bool last_block_full = (g.M + 127) % 128 >= 95; // (rows of the last block: (M - 1) % 128 + 1 >= 96)
-    if (!g.w_int4 && tiles128 >= cus * 5L / 8 && tiles128 <= cus + (last_block_full ? cus / 50 : 0)) return 128;
+    if (!g.w_int4 && tiles128 >= cus * 5L / 8 && tiles128 <= cus) return 128;
     return 0;
 }
 

@@ -26,7 +26,7 @@ I32_SHAPES = [(1, 32, 32), (1, 200, 200), (3, 65, 33), (8, 64, 96), (9, 64, 96),
               (1, 1, 1), (5000, 3, 1), (2, 1, 5000), (4100, 40, 70), (1, 70001, 64), (9, 70001, 40), (300, 40000, 33),
               # 64-row tiles of the large-tile kernel (too few 128-row tiles); K split over workgroups + reduce launch
               (330, 6600, 200), (150, 96, 8300),
-              # tiles of 128 x 128 with one column block per wave (160 .. 261 of them, more 64-row tiles than that)
+              # tiles of 128 x 128 with one column block per wave (160 .. 256 of them, more 64-row tiles than that)
               (300, 8448, 200), (257, 8200, 300), (640, 4200, 96),
               # weight-streaming kernel (9 .. 128 rows) without / with the in-workgroup K split; 129 .. 256 rows on a
               # narrow matrix with it (a longer K there: the 64-row tiles above)
